@@ -1,0 +1,414 @@
+"""ctypes binding of libbeam_hip.so.
+
+Counterpart of the reference's pybind11 module (python/beam/_C/__init__.py:1-23, signatures in
+python/beam/_C/beam_C.pyi:4-23).  Every operator takes (a, b, c): a is [M, K], b is [N, K], c is
+[M, N], all 16-bit, all resident on the GPU; c is written in place and nothing is returned.
+
+Tensors may be torch CUDA tensors (launched on torch's current stream) or beam.DeviceArray
+objects (memory owned through the library's own allocator, launched on the default stream).
+There is no CPU fallback: if the shared library is missing the import fails, and every error
+code of the library becomes a BeamError.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from dataclasses import dataclass
+from typing import List, Optional, Sequence
+
+import numpy as np
+
+F16 = 0
+BF16 = 1
+_DTYPE_NAMES = {F16: "fp16", BF16: "bf16"}
+
+_PKG_DIR = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+_LIB_PATH = os.path.join(_PKG_DIR, "libbeam_hip.so")
+
+
+class BeamError(RuntimeError):
+    """A call into libbeam_hip.so returned a non-zero status."""
+
+    def __init__(self, status: int, message: str):
+        super().__init__(f"beam status {status}: {message}")
+        self.status = status
+
+
+class _TileCfg(ctypes.Structure):
+    _fields_ = [("block_m", ctypes.c_int), ("block_n", ctypes.c_int), ("wave_m", ctypes.c_int),
+                ("wave_n", ctypes.c_int), ("loader", ctypes.c_int), ("group_m", ctypes.c_int)]
+
+
+class _Problem(ctypes.Structure):
+    _fields_ = [("A", ctypes.c_void_p), ("B", ctypes.c_void_p), ("C", ctypes.c_void_p),
+                ("gamma", ctypes.c_void_p), ("beta", ctypes.c_void_p), ("eps", ctypes.c_float),
+                ("M", ctypes.c_int), ("N", ctypes.c_int), ("K", ctypes.c_int), ("dtype", ctypes.c_int),
+                ("split_k", ctypes.c_int), ("ws", ctypes.c_void_p), ("ws_bytes", ctypes.c_size_t)]
+
+
+def library_path() -> str:
+    return _LIB_PATH
+
+
+def _load() -> ctypes.CDLL:
+    if not os.path.exists(_LIB_PATH):
+        raise ImportError(
+            f"{_LIB_PATH} is missing: build it with `make -C {os.path.join(_PKG_DIR, 'csrc')}` "
+            "(hipcc, gfx950).  There is no fallback path.")
+    L = ctypes.CDLL(_LIB_PATH)
+    vp, i, sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t
+    cfgp = ctypes.POINTER(_TileCfg)
+    L.beam_last_error.restype = ctypes.c_char_p
+    L.beam_init.restype = i
+    L.beam_device_info.argtypes = [ctypes.c_char_p, i, ctypes.POINTER(i), ctypes.POINTER(i), ctypes.POINTER(sz)]
+    L.beam_num_configs.restype = i
+    L.beam_get_config.argtypes = [i, cfgp]
+    L.beam_default_config.argtypes = [i, i, i, cfgp, ctypes.POINTER(i)]
+    L.beam_gemmrc.argtypes = [vp, vp, vp, i, i, i, i, cfgp, vp]
+    for name in ("beam_custom_gemmrc_128x128", "beam_custom_gemmrc_128x256", "beam_custom_gemmrc_256x128"):
+        getattr(L, name).argtypes = [vp, vp, vp, i, i, i, vp]
+    L.beam_slice_heuristic.argtypes = [i, i]
+    L.beam_splitk_workspace_bytes.argtypes = [i, i, i]
+    L.beam_splitk_workspace_bytes.restype = sz
+    L.beam_gemmrc_splitk.argtypes = [vp, vp, vp, i, i, i, i, cfgp, i, vp, sz, vp]
+    L.beam_splitk_effective.argtypes = [i, i, i, cfgp, i]
+    L.beam_gemmrc_ln_workspace_bytes.argtypes = [i, i, cfgp]
+    L.beam_gemmrc_ln_workspace_bytes.restype = sz
+    L.beam_gemmrc_ln.argtypes = [vp, vp, vp, vp, ctypes.c_float, vp, i, i, i, i, cfgp, vp, sz, vp]
+    L.beam_bench.argtypes = [i, ctypes.POINTER(_Problem), cfgp, i, i, vp, ctypes.POINTER(ctypes.c_float)]
+    L.beam_event_create.argtypes = [ctypes.POINTER(vp)]
+    L.beam_event_record.argtypes = [vp, vp]
+    L.beam_event_elapsed_ms.argtypes = [vp, vp, ctypes.POINTER(ctypes.c_float)]
+    L.beam_event_destroy.argtypes = [vp]
+    L.beam_malloc.argtypes = [ctypes.POINTER(vp), sz]
+    L.beam_free.argtypes = [vp]
+    L.beam_memcpy_h2d.argtypes = [vp, vp, sz]
+    L.beam_memcpy_d2h.argtypes = [vp, vp, sz]
+    L.beam_memset.argtypes = [vp, i, sz]
+    L.beam_sync.argtypes = [vp]
+    L.beam_host_fill_uniform.argtypes = [vp, sz, i, ctypes.c_uint64, ctypes.c_uint64]
+    L.beam_host_fill_normal.argtypes = [vp, sz, i, ctypes.c_uint64, ctypes.c_uint64, ctypes.c_float, ctypes.c_float]
+    L.beam_dbg_tile_of_workgroup.argtypes = [i, i, i, i, ctypes.POINTER(i), ctypes.POINTER(i)]
+    L.beam_dbg_lds_offset.argtypes = [i, i]
+    return L
+
+
+lib = _load()
+
+
+def _check(status: int) -> None:
+    if status != 0:
+        raise BeamError(status, lib.beam_last_error().decode())
+
+
+# ---------------------------------------------------------------------------- configurations
+
+
+@dataclass(frozen=True)
+class TileConfig:
+    """One point of the tunable space: workgroup tile, wavefront tile, loader, raster group."""
+    block_m: int
+    block_n: int
+    wave_m: int
+    wave_n: int
+    loader: int = 0
+    group_m: int = 0
+
+    def to_c(self) -> _TileCfg:
+        return _TileCfg(self.block_m, self.block_n, self.wave_m, self.wave_n, self.loader, self.group_m)
+
+    @property
+    def name(self) -> str:
+        s = f"{self.block_m}x{self.block_n}_w{self.wave_m}x{self.wave_n}"
+        if self.loader:
+            s += "_staged"
+        if self.group_m:
+            s += f"_g{self.group_m}"
+        return s
+
+
+def list_configs() -> List[TileConfig]:
+    out = []
+    for idx in range(lib.beam_num_configs()):
+        c = _TileCfg()
+        _check(lib.beam_get_config(idx, ctypes.byref(c)))
+        out.append(TileConfig(c.block_m, c.block_n, c.wave_m, c.wave_n, c.loader, 0))
+    return out
+
+
+def default_config(M: int, N: int, K: int):
+    c = _TileCfg()
+    s = ctypes.c_int(1)
+    _check(lib.beam_default_config(M, N, K, ctypes.byref(c), ctypes.byref(s)))
+    return TileConfig(c.block_m, c.block_n, c.wave_m, c.wave_n, c.loader, c.group_m), s.value
+
+
+def device_info() -> dict:
+    name = ctypes.create_string_buffer(256)
+    cus, clk, mem = ctypes.c_int(), ctypes.c_int(), ctypes.c_size_t()
+    _check(lib.beam_device_info(name, 256, ctypes.byref(cus), ctypes.byref(clk), ctypes.byref(mem)))
+    return {"name": name.value.decode(), "compute_units": cus.value, "clock_khz": clk.value,
+            "memory_bytes": mem.value}
+
+
+# ---------------------------------------------------------------------------- device buffers
+
+
+class DeviceArray:
+    """A 16-bit (or raw byte) buffer in HBM owned through beam_malloc/beam_free."""
+
+    def __init__(self, shape: Sequence[int], dtype: int = F16, itemsize: int = 2):
+        self.shape = tuple(int(s) for s in shape)
+        self.dtype = dtype
+        self.itemsize = itemsize
+        self.nbytes = int(np.prod(self.shape, dtype=np.int64)) * itemsize
+        p = ctypes.c_void_p()
+        _check(lib.beam_malloc(ctypes.byref(p), self.nbytes))
+        self.ptr = p.value or 0
+
+    @classmethod
+    def from_numpy(cls, bits: np.ndarray, dtype: int = F16) -> "DeviceArray":
+        bits = np.ascontiguousarray(bits)
+        arr = cls(bits.shape, dtype, bits.dtype.itemsize)
+        _check(lib.beam_memcpy_h2d(arr.ptr, bits.ctypes.data, arr.nbytes))
+        return arr
+
+    def to_numpy(self, np_dtype=np.uint16) -> np.ndarray:
+        out = np.empty(self.shape, dtype=np_dtype)
+        assert out.nbytes == self.nbytes
+        _check(lib.beam_sync(None))
+        _check(lib.beam_memcpy_d2h(out.ctypes.data, self.ptr, self.nbytes))
+        return out
+
+    def fill_bytes(self, byte: int = 0) -> None:
+        _check(lib.beam_memset(self.ptr, byte, self.nbytes))
+
+    def data_ptr(self) -> int:
+        return self.ptr
+
+    def free(self) -> None:
+        if getattr(self, "ptr", 0):
+            lib.beam_free(self.ptr)
+            self.ptr = 0
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+def _is_torch(x) -> bool:
+    return type(x).__module__.split(".")[0] == "torch"
+
+
+def _describe(x):
+    """(pointer, shape, dtype code, stream handle) of a torch tensor or DeviceArray."""
+    if isinstance(x, DeviceArray):
+        return x.ptr, x.shape, x.dtype, None
+    if _is_torch(x):
+        import torch
+        if not x.is_cuda:
+            raise BeamError(1, "tensor is not on the GPU")
+        if not x.is_contiguous():
+            raise BeamError(1, "tensor is not contiguous")
+        if x.dtype == torch.float16:
+            d = F16
+        elif x.dtype == torch.bfloat16:
+            d = BF16
+        else:
+            raise BeamError(2, f"unsupported tensor type {x.dtype}")
+        return x.data_ptr(), tuple(x.shape), d, torch.cuda.current_stream().cuda_stream
+    raise TypeError(f"expected a torch CUDA tensor or beam.DeviceArray, got {type(x)!r}")
+
+
+def _problem(a, b, c):
+    """Shape conventions of cuda/cutlass_kernels/main.cc:25-35: M=a.size(0), N=b.size(0),
+    K=a.size(1); a.size(1)==b.size(1), c is [M, N]; all three of one 16-bit dtype."""
+    pa, sa, da, st = _describe(a)
+    pb, sb, db, _ = _describe(b)
+    pc, sc, dc, _ = _describe(c)
+    if len(sa) != 2 or len(sb) != 2 or len(sc) != 2:
+        raise BeamError(1, "a, b, c must be 2-D")
+    M, K = sa
+    N = sb[0]
+    if sb[1] != K:
+        raise BeamError(1, f"a.size(1)={K} != b.size(1)={sb[1]}")
+    if sc != (M, N):
+        raise BeamError(1, f"c has shape {sc}, expected {(M, N)}")
+    if not (da == db == dc):
+        raise BeamError(2, "a, b, c must share one dtype (fp16 or bf16)")
+    return pa, pb, pc, M, N, K, da, st
+
+
+def _cfg_from_shapes(shape_threadblock, shape_warp, loader=0, group_m=0) -> _TileCfg:
+    # An empty list means "default", as in cuda/cutlass_kernels/cutlass_gemmrc.cu:73-81.
+    tb = list(shape_threadblock) if shape_threadblock else [128, 128]
+    wp = list(shape_warp) if shape_warp else [64, 64]
+    if len(tb) != 2 or len(wp) != 2:
+        raise BeamError(1, "shape_threadblock and shape_warp must have two entries")
+    return _TileCfg(tb[0], tb[1], wp[0], wp[1], loader, group_m)
+
+
+# ---------------------------------------------------------------------------- workspaces
+
+_workspace: Optional[DeviceArray] = None
+
+
+def _get_workspace(nbytes: int) -> DeviceArray:
+    """Grow-only scratch owned by the Python layer (the C ABI itself keeps no hidden buffer);
+    counterpart of get_the_buffer, cuda/cutlass_kernels/cutlass_gemmrc_splitk.cu:31-42."""
+    global _workspace
+    if _workspace is None or _workspace.nbytes < nbytes:
+        if _workspace is not None:
+            _check(lib.beam_sync(None))
+            _workspace.free()
+        _workspace = DeviceArray((max(nbytes, 1 << 20),), itemsize=1)
+    return _workspace
+
+
+# ---------------------------------------------------------------------------- operators
+
+
+def gemmrc(a, b, c, config: Optional[TileConfig] = None) -> None:
+    """c = a @ b.T with the library's default tile (or `config`)."""
+    pa, pb, pc, M, N, K, d, st = _problem(a, b, c)
+    cfg = ctypes.byref(config.to_c()) if config is not None else None
+    _check(lib.beam_gemmrc(pa, pb, pc, M, N, K, d, cfg, st))
+
+
+def gemmrc_spec(a, b, c, shape_threadblock=(128, 128), shape_warp=(64, 64), loader: int = 0,
+                group_m: int = 0) -> None:
+    """c = a @ b.T with an explicit workgroup tile / wavefront tile
+    (reference: cutlass_gemmrc_spec, python/beam/_C/beam_C.pyi:16)."""
+    pa, pb, pc, M, N, K, d, st = _problem(a, b, c)
+    cfg = _cfg_from_shapes(shape_threadblock, shape_warp, loader, group_m)
+    _check(lib.beam_gemmrc(pa, pb, pc, M, N, K, d, ctypes.byref(cfg), st))
+
+
+def gemmrc_splitk(a, b, c, split_k_slices: int = 0) -> None:
+    """Split-K with the library's default small tile; split_k_slices <= 0 = heuristic
+    (reference: cutlass_gemmrc_splitk, python/beam/_C/beam_C.pyi:18)."""
+    gemmrc_splitk_spec(a, b, c, shape_threadblock=(128, 128), shape_warp=(64, 64),
+                       split_k_slices=split_k_slices)
+
+
+def gemmrc_splitk_spec(a, b, c, shape_threadblock=(128, 128), shape_warp=(64, 64), split_k_slices: int = 0,
+                       loader: int = 0, group_m: int = 0) -> None:
+    """Split-K with explicit tiles (reference: cutlass_gemmrc_splitk_spec, beam_C.pyi:20)."""
+    pa, pb, pc, M, N, K, d, st = _problem(a, b, c)
+    cfg = _cfg_from_shapes(shape_threadblock, shape_warp, loader, group_m)
+    s = lib.beam_splitk_effective(M, N, K, ctypes.byref(cfg), split_k_slices)
+    if s < 0:
+        raise BeamError(2, lib.beam_last_error().decode())
+    need = lib.beam_splitk_workspace_bytes(M, N, s) if s > 1 else 0
+    ws = _get_workspace(need) if need else None
+    _check(lib.beam_gemmrc_splitk(pa, pb, pc, M, N, K, d, ctypes.byref(cfg), split_k_slices,
+                                  ws.ptr if ws else None, ws.nbytes if ws else 0, st))
+
+
+def gemmrc_ln(a, b, c, gamma, beta, eps: float = 1e-5, config: Optional[TileConfig] = None) -> None:
+    """c = LayerNorm_N(a @ b.T) * gamma + beta, statistics from the fp32 accumulators."""
+    pa, pb, pc, M, N, K, d, st = _problem(a, b, c)
+    pg, sg, dg, _ = _describe(gamma)
+    pbt, sbt, dbt, _ = _describe(beta)
+    if tuple(sg) != (N,) or tuple(sbt) != (N,) or dg != d or dbt != d:
+        raise BeamError(1, "gamma and beta must be [N] of the same dtype as a, b, c")
+    cfg = config.to_c() if config is not None else None
+    need = lib.beam_gemmrc_ln_workspace_bytes(M, N, ctypes.byref(cfg) if cfg else None)
+    ws = _get_workspace(need)
+    _check(lib.beam_gemmrc_ln(pa, pb, pg, pbt, eps, pc, M, N, K, d, ctypes.byref(cfg) if cfg else None,
+                              ws.ptr, ws.nbytes, st))
+
+
+def _fixed(fn_name: str):
+    cfn = getattr(lib, fn_name)
+
+    def op(a, b, c) -> None:
+        pa, pb, pc, M, N, K, d, st = _problem(a, b, c)
+        if d != F16:
+            raise BeamError(2, f"{fn_name}: fp16 only")
+        _check(cfn(pa, pb, pc, M, N, K, st))
+
+    op.__name__ = fn_name[len("beam_"):]
+    op.__doc__ = f"Fixed-tile fp16 gemmrc ({fn_name}); reference: python/beam/_C/beam_C.pyi:8-11."
+    return op
+
+
+custom_gemmrc_128x128 = _fixed("beam_custom_gemmrc_128x128")
+custom_gemmrc_128x256 = _fixed("beam_custom_gemmrc_128x256")
+custom_gemmrc_256x128 = _fixed("beam_custom_gemmrc_256x128")
+
+# The reference's operator names (python/beam/_C/__init__.py:1-11), kept so that scripts written
+# against it run unchanged.  Nothing here involves CUTLASS.
+cutlass_gemmrc = gemmrc
+cutlass_gemmrc_spec = gemmrc_spec
+cutlass_gemmrc_splitk = gemmrc_splitk
+cutlass_gemmrc_splitk_spec = gemmrc_splitk_spec
+
+
+# ---------------------------------------------------------------------------- timing / data
+
+
+def bench(op: int, a, b, c, config: Optional[TileConfig] = None, split_k: int = 0, gamma=None, beta=None,
+          eps: float = 1e-5, warmup: int = 5, iters: int = 20) -> float:
+    """Average milliseconds per call (HIP events around `iters` back-to-back launches)."""
+    pa, pb, pc, M, N, K, d, st = _problem(a, b, c)
+    cfg = config.to_c() if config is not None else None
+    cfgp = ctypes.byref(cfg) if cfg is not None else None
+    q = _Problem(pa, pb, pc, None, None, eps, M, N, K, d, split_k, None, 0)
+    ws = None
+    if op == 1:
+        s = lib.beam_splitk_effective(M, N, K, cfgp, split_k)
+        if s < 0:
+            raise BeamError(2, lib.beam_last_error().decode())
+        ws = _get_workspace(max(lib.beam_splitk_workspace_bytes(M, N, s), 1))
+    elif op == 2:
+        q.gamma, q.beta = _describe(gamma)[0], _describe(beta)[0]
+        ws = _get_workspace(lib.beam_gemmrc_ln_workspace_bytes(M, N, cfgp))
+    if ws is not None:
+        q.ws, q.ws_bytes = ws.ptr, ws.nbytes
+    ms = ctypes.c_float()
+    _check(lib.beam_bench(op, ctypes.byref(q), cfgp, warmup, iters, st, ctypes.byref(ms)))
+    return ms.value
+
+
+def do_bench(fn, warmup: int = 5, rep: int = 20, stream=None) -> float:
+    """Average milliseconds per call of an arbitrary launcher `fn()` (HIP events on `stream`).
+    Host-side launch cost is included when the kernels are shorter than it; prefer bench()
+    for the library's own operators."""
+    for _ in range(warmup):
+        fn()
+    e0, e1 = ctypes.c_void_p(), ctypes.c_void_p()
+    _check(lib.beam_event_create(ctypes.byref(e0)))
+    _check(lib.beam_event_create(ctypes.byref(e1)))
+    try:
+        _check(lib.beam_event_record(e0, stream))
+        for _ in range(rep):
+            fn()
+        _check(lib.beam_event_record(e1, stream))
+        ms = ctypes.c_float()
+        _check(lib.beam_event_elapsed_ms(e0, e1, ctypes.byref(ms)))
+    finally:
+        lib.beam_event_destroy(e0)
+        lib.beam_event_destroy(e1)
+    return ms.value / rep
+
+
+def host_uniform(shape, dtype: int = F16, seed: int = 0, tensor_id: int = 0) -> np.ndarray:
+    """uint16 bit patterns of uniform[-1, 1) values (counter-based, reproducible)."""
+    out = np.empty(shape, dtype=np.uint16)
+    _check(lib.beam_host_fill_uniform(out.ctypes.data, out.size, dtype, seed, tensor_id))
+    return out
+
+
+def host_normal(shape, dtype: int = F16, seed: int = 0, tensor_id: int = 0, mean: float = 0.0,
+                scale: float = 1.0) -> np.ndarray:
+    """uint16 bit patterns of mean + scale * N(0, 1) values (counter-based, reproducible)."""
+    out = np.empty(shape, dtype=np.uint16)
+    _check(lib.beam_host_fill_normal(out.ctypes.data, out.size, dtype, seed, tensor_id, mean, scale))
+    return out
+
+
+def sync() -> None:
+    _check(lib.beam_sync(None))

@@ -1,0 +1,226 @@
+"""Autotuner for gemmrc on MI355X.
+
+Counterpart of the reference's python/beam/tuner.py:19-137:
+
+* Operator wraps a callable f(a=, b=, c=); str(op) is the callable's name;
+  check_callable makes one trial call; get_performance returns TFLOP/s (2*M*N*K / latency)
+  or -1 when the call fails or the number is implausible.
+* OperatorTuner enumerates candidates (plain tiles and split-K tiles x split factors), times
+  each on fresh inputs and memoises (best_op, best_tflops) per problem.
+
+What differs, on purpose: the cache key carries the dtype and is persisted as JSON; inputs are
+seeded; a candidate whose output disagrees with the library's default kernel is discarded
+instead of trusted (the reference's only guard is the >1000 TFLOP/s filter, tuner.py:42-43);
+the search space is the library's gfx950 tile table and split factors {4, 8, 16, 32, 64}.
+"""
+from __future__ import annotations
+
+import json
+import os
+from functools import partial
+from typing import Callable, Dict, List, Optional, Sequence, Tuple
+
+import numpy as np
+
+from . import _C
+
+# Dense fp16/bf16 matrix-core peak of MI355X is about 2.5 PFLOP/s; anything above is a
+# measurement artefact (a launch that failed or did nothing).
+PLAUSIBLE_TFLOPS = 2600.0
+SPLIT_FACTORS = (4, 8, 16, 32, 64)
+_DTYPES = {"fp16": _C.F16, "bf16": _C.BF16}
+
+
+def _callable_name(func) -> str:
+    name = getattr(func, "__name__", None)
+    if name:
+        return name
+    if isinstance(func, partial):
+        inner = _callable_name(func.func)
+        kw = ",".join(f"{k}={v}" for k, v in sorted(func.keywords.items()))
+        return f"{inner}[{kw}]"
+    return "Unknown"
+
+
+class Operator:
+    """A timed gemmrc candidate (reference: python/beam/tuner.py:19-44)."""
+
+    def __init__(self, func: Callable, native: Optional[dict] = None, name: Optional[str] = None):
+        self.func = func
+        self.native = native  # arguments for _C.bench (timing loop inside the library)
+        self._name = name
+
+    def __str__(self) -> str:
+        return self._name or _callable_name(self.func)
+
+    def __call__(self, a, b, c) -> None:
+        self.func(a=a, b=b, c=c)
+
+    def check_callable(self, a, b, c) -> bool:
+        try:
+            self.func(a=a, b=b, c=c)
+            _C.sync()
+            return True
+        except Exception:
+            return False
+
+    def latency_ms(self, a, b, c, warmup: int = 5, rep: int = 20) -> float:
+        if self.native is not None:
+            return _C.bench(self.native["op"], a, b, c, config=self.native.get("config"),
+                            split_k=self.native.get("split_k", 0), warmup=warmup, iters=rep)
+        stream = _C._describe(a)[3]
+        return _C.do_bench(lambda: self.func(a=a, b=b, c=c), warmup=warmup, rep=rep, stream=stream)
+
+    def get_performance(self, a, b, c, warmup: int = 5, rep: int = 20) -> float:
+        if not self.check_callable(a, b, c):
+            return -1
+        try:
+            latency = self.latency_ms(a, b, c, warmup=warmup, rep=rep) * 1e-3
+        except Exception:
+            return -1
+        if not latency > 0:
+            return -1
+        M, N = _C._describe(c)[1]
+        K = _C._describe(a)[1][1]
+        tflops = 2 * M * N * K / latency * 1e-12
+        if tflops > PLAUSIBLE_TFLOPS:  # obviously wrong
+            return -1
+        return tflops
+
+
+class OperatorTuner:
+    """Search over tiles and split factors, keyed by (M, N, K, dtype)
+    (reference: python/beam/tuner.py:47-137)."""
+
+    gemm_ops: List[Operator]
+    cache: Dict[str, Tuple[Operator, float]]
+
+    def __init__(self, cache_path: Optional[str] = None, verify: bool = True, seed: int = 1234,
+                 warmup: int = 3, rep: int = 10):
+        self.cache = {}
+        self.cache_path = cache_path
+        self.verify = verify
+        self.seed = seed
+        self.warmup = warmup
+        self.rep = rep
+        self.gemm_ops = [
+            Operator(_C.gemmrc, native={"op": 0}),
+            Operator(_C.gemmrc_splitk, native={"op": 1}),
+            Operator(_C.custom_gemmrc_128x128),
+            Operator(_C.custom_gemmrc_128x256),
+            Operator(_C.custom_gemmrc_256x128),
+        ]
+        self.gemm_ops.extend(self._get_gemm_specs())
+        self.gemm_ops.extend(self._get_gemm_splitk_specs())
+        self._by_name = {str(op): op for op in self.gemm_ops}
+        if cache_path and os.path.exists(cache_path):
+            self._load(cache_path)
+
+    # -- candidate enumeration ------------------------------------------------------------
+
+    def _get_gemm_specs(self) -> List[Operator]:
+        ret = []
+        for cfg in _C.list_configs():
+            for group_m in (4, 8, 16):
+                full = _C.TileConfig(cfg.block_m, cfg.block_n, cfg.wave_m, cfg.wave_n, 0, group_m)
+                ret.append(Operator(
+                    partial(_C.gemmrc_spec, shape_threadblock=[cfg.block_m, cfg.block_n],
+                            shape_warp=[cfg.wave_m, cfg.wave_n], group_m=group_m),
+                    native={"op": 0, "config": full}, name=f"gemmrc_spec[{full.name}]"))
+        return ret
+
+    def _get_gemm_splitk_specs(self) -> List[Operator]:
+        ret = []
+        for cfg in _C.list_configs():
+            if cfg.block_m * cfg.block_n > 128 * 128:
+                continue  # split-K is for problems with few output tiles
+            for s in SPLIT_FACTORS:
+                ret.append(Operator(
+                    partial(_C.gemmrc_splitk_spec, shape_threadblock=[cfg.block_m, cfg.block_n],
+                            shape_warp=[cfg.wave_m, cfg.wave_n], split_k_slices=s),
+                    native={"op": 1, "config": cfg, "split_k": s},
+                    name=f"gemmrc_splitk_spec[{cfg.name},s{s}]"))
+        return ret
+
+    # -- cache -----------------------------------------------------------------------------
+
+    def get_hash(self, name: str, args: Sequence) -> str:
+        ret = name + "("
+        for arg in args:
+            ret += str(arg) + ","
+        ret += ")"
+        return ret
+
+    def _load(self, path: str) -> None:
+        with open(path) as f:
+            blob = json.load(f)
+        for key, (name, tflops) in blob.get("entries", {}).items():
+            op = self._by_name.get(name)
+            if op is not None:
+                self.cache[key] = (op, float(tflops))
+
+    def save(self, path: Optional[str] = None) -> None:
+        path = path or self.cache_path
+        if not path:
+            return
+        blob = {"arch": "gfx950", "entries": {k: [str(op), t] for k, (op, t) in self.cache.items()}}
+        tmp = path + ".tmp"
+        with open(tmp, "w") as f:
+            json.dump(blob, f, indent=1, sort_keys=True)
+        os.replace(tmp, path)
+
+    # -- tuning ------------------------------------------------------------------------------
+
+    def _make_inputs(self, M: int, N: int, K: int, dtype: int):
+        a = _C.DeviceArray.from_numpy(_C.host_uniform((M, K), dtype, self.seed, 0), dtype)
+        b = _C.DeviceArray.from_numpy(_C.host_uniform((N, K), dtype, self.seed, 1), dtype)
+        c = _C.DeviceArray((M, N), dtype)
+        return a, b, c
+
+    @staticmethod
+    def _agrees(got: np.ndarray, want: np.ndarray, dtype: int, K: int) -> bool:
+        """Outputs of two kernels for the same inputs differ only by summation order and one
+        rounding: compare as floats against the RMS-relative bound used for the GEMM."""
+        def f32(bits):
+            if dtype == _C.BF16:
+                return (bits.astype(np.uint32) << 16).view(np.float32)
+            return bits.view(np.float16).astype(np.float32)
+        g, w = f32(got), f32(want)
+        rms = float(np.sqrt(np.mean(w.astype(np.float64) ** 2)))
+        tol = 2e-2 * max((K / 1024.0) ** 0.5, 1.0) * max(rms, 1e-30)
+        if dtype == _C.BF16:
+            tol += float(np.max(np.abs(w))) / 128.0
+        return bool(np.isfinite(g).all() and float(np.max(np.abs(g - w))) <= tol)
+
+    def tune(self, matmul_shape: Sequence[int], dtype: str = "fp16", ops: Optional[List[Operator]] = None,
+             verbose: bool = False) -> Tuple[Operator, float]:
+        M, N, K = (int(x) for x in matmul_shape)
+        d = _DTYPES[dtype]
+        hashval = self.get_hash("gemm", [M, N, K, dtype])
+        if hashval in self.cache:
+            return self.cache[hashval]
+        a, b, c = self._make_inputs(M, N, K, d)
+        want = None
+        if self.verify:
+            c.fill_bytes(0)
+            _C.gemmrc(a, b, c)
+            want = c.to_numpy()
+        best_op, best_tflops = None, -1
+        for op in (ops if ops is not None else self.gemm_ops):
+            if d != _C.F16 and str(op).startswith("custom_"):
+                continue  # fixed-tile entries are fp16 only
+            c.fill_bytes(0xFF)
+            tflops = op.get_performance(a, b, c, warmup=self.warmup, rep=self.rep)
+            if tflops > 0 and want is not None and not self._agrees(c.to_numpy(), want, d, K):
+                if verbose:
+                    print(f"  {op}: output disagrees with the default kernel; discarded")
+                tflops = -1
+            if verbose:
+                print(f"  {op}: {tflops:.2f} TFLOP/s")
+            if tflops > best_tflops:
+                best_op, best_tflops = op, tflops
+        for x in (a, b, c):
+            x.free()
+        self.cache[hashval] = (best_op, best_tflops)
+        self.save()
+        return self.cache[hashval]

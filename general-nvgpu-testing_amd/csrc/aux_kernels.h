@@ -1,0 +1,20 @@
+// Launchers of the split-K reduction and the LayerNorm normalisation pass.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+
+#include "../../include/beam_hip.h"
+
+namespace beam {
+
+// C[mn] (16-bit) = sum over `splits` fp32 slices of ws[splits][mn], added in slice order.
+hipError_t launch_splitk_reduce(const float* ws, void* C, size_t mn, int splits, int dtype,
+                                hipStream_t stream);
+
+// Y[M][N] (16-bit) = normalise fp32 X[M][N] with per-(row, column tile) (mean, M2) pairs.
+hipError_t launch_ln_apply(const float* X, const float* stats, const void* gamma, const void* beta,
+                           void* Y, int M, int N, int tiles_n, int block_n, float eps, int dtype,
+                           hipStream_t stream);
+
+}  // namespace beam

@@ -1,0 +1,115 @@
+// Bandwidth-bound companions of the tiled kernel: the split-K reduction and the LayerNorm
+// normalisation pass.  Both stream fp32 from the workspace once and write 16-bit once.
+#include "aux_kernels.h"
+
+namespace beam {
+
+namespace {
+
+template <typename T>
+struct Vec4Of;
+template <>
+struct Vec4Of<_Float16> { typedef _Float16 type __attribute__((ext_vector_type(4))); };
+template <>
+struct Vec4Of<__bf16> { typedef __bf16 type __attribute__((ext_vector_type(4))); };
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+// C[i] = round( ws[0][i] + ws[1][i] + ... + ws[S-1][i] ), slices added in index order.
+// The fixed order is what makes split-K bit-reproducible (the reference delegates this to
+// CUTLASS's reduce kernel, cuda/cutlass_kernels/cutlass_gemmrc_splitk.cu:73-75).
+template <typename T>
+__global__ void __launch_bounds__(256) splitk_reduce_kernel(const float* __restrict__ ws,
+                                                             T* __restrict__ C, size_t mn, int splits) {
+  typedef typename Vec4Of<T>::type vec4;
+  const size_t quads = mn / 4;
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (size_t q = (size_t)blockIdx.x * blockDim.x + threadIdx.x; q < quads; q += stride) {
+    f32x4 s = *(const f32x4*)(ws + q * 4);
+    for (int z = 1; z < splits; ++z) s += *(const f32x4*)(ws + (size_t)z * mn + q * 4);
+    vec4 o;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) o[e] = (T)s[e];
+    *(vec4*)(C + q * 4) = o;
+  }
+  // tail (mn not a multiple of 4)
+  const size_t t = quads * 4 + (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (t < mn) {
+    float s = ws[t];
+    for (int z = 1; z < splits; ++z) s += ws[(size_t)z * mn + t];
+    C[t] = (T)s;
+  }
+}
+
+// One workgroup per row: merge the per-column-tile (mean, M2) pairs in tile order (Chan's
+// update), then y = (x - mean) * rstd * gamma + beta from the fp32 x.
+template <typename T>
+__global__ void __launch_bounds__(256) ln_apply_kernel(const float* __restrict__ X,
+                                                        const float* __restrict__ stats,
+                                                        const T* __restrict__ gamma,
+                                                        const T* __restrict__ beta, T* __restrict__ Y,
+                                                        int N, int tiles_n, int block_n, float eps) {
+  typedef typename Vec4Of<T>::type vec4;
+  const int m = blockIdx.x;
+  const float* st = stats + (size_t)m * tiles_n * 2;
+  float mean = 0.0f, m2 = 0.0f, cnt = 0.0f;
+  for (int t = 0; t < tiles_n; ++t) {
+    int cw = N - t * block_n;
+    cw = cw > block_n ? block_n : cw;
+    const float nb = (float)cw;
+    const float tot = cnt + nb;
+    const float delta = st[2 * t] - mean;
+    mean += delta * (nb / tot);
+    m2 += st[2 * t + 1] + delta * delta * (cnt * nb / tot);
+    cnt = tot;
+  }
+  const float rstd = 1.0f / sqrtf(m2 / (float)N + eps);
+  const float* x = X + (size_t)m * N;
+  T* y = Y + (size_t)m * N;
+  if ((N & 3) == 0) {
+    for (int n = threadIdx.x * 4; n < N; n += blockDim.x * 4) {
+      const f32x4 v = *(const f32x4*)(x + n);
+      const vec4 g = *(const vec4*)(gamma + n);
+      const vec4 b = *(const vec4*)(beta + n);
+      vec4 o;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) o[e] = (T)((v[e] - mean) * rstd * (float)g[e] + (float)b[e]);
+      *(vec4*)(y + n) = o;
+    }
+  } else {
+    for (int n = threadIdx.x; n < N; n += blockDim.x)
+      y[n] = (T)((x[n] - mean) * rstd * (float)gamma[n] + (float)beta[n]);
+  }
+}
+
+}  // namespace
+
+hipError_t launch_splitk_reduce(const float* ws, void* C, size_t mn, int splits, int dtype,
+                                hipStream_t stream) {
+  size_t quads = (mn + 3) / 4;
+  size_t blocks = (quads + 255) / 256;
+  if (blocks < 1) blocks = 1;
+  if (blocks > 4096) blocks = 4096;
+  if (dtype == BEAM_BF16)
+    hipLaunchKernelGGL(splitk_reduce_kernel<__bf16>, dim3((unsigned)blocks), dim3(256), 0, stream, ws,
+                       (__bf16*)C, mn, splits);
+  else
+    hipLaunchKernelGGL(splitk_reduce_kernel<_Float16>, dim3((unsigned)blocks), dim3(256), 0, stream, ws,
+                       (_Float16*)C, mn, splits);
+  return hipGetLastError();
+}
+
+hipError_t launch_ln_apply(const float* X, const float* stats, const void* gamma, const void* beta,
+                           void* Y, int M, int N, int tiles_n, int block_n, float eps, int dtype,
+                           hipStream_t stream) {
+  if (dtype == BEAM_BF16)
+    hipLaunchKernelGGL(ln_apply_kernel<__bf16>, dim3(M), dim3(256), 0, stream, X, stats,
+                       (const __bf16*)gamma, (const __bf16*)beta, (__bf16*)Y, N, tiles_n, block_n, eps);
+  else
+    hipLaunchKernelGGL(ln_apply_kernel<_Float16>, dim3(M), dim3(256), 0, stream, X, stats,
+                       (const _Float16*)gamma, (const _Float16*)beta, (_Float16*)Y, N, tiles_n,
+                       block_n, eps);
+  return hipGetLastError();
+}
+
+}  // namespace beam

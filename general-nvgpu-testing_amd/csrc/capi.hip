@@ -1,0 +1,552 @@
+// C ABI of libbeam_hip.so (declarations and reference citations: include/beam_hip.h).
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <mutex>
+#include <thread>
+#include <vector>
+
+#include "../../include/beam_hip.h"
+#include "aux_kernels.h"
+#include "kernel_set.h"
+#include "tile_map.h"
+
+using namespace beam;
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof g_err, fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+int hip_fail(hipError_t e, const char* what) {
+  return fail(BEAM_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
+}
+
+#define BEAM_HIP(call)                                  \
+  do {                                                  \
+    hipError_t e_ = (call);                             \
+    if (e_ != hipSuccess) return hip_fail(e_, #call);   \
+  } while (0)
+
+struct Device {
+  int status = -1;  // -1 = not probed
+  char name[256] = "";
+  int cus = 0;
+  int clock_khz = 0;
+  size_t mem = 0;
+};
+Device g_dev;
+std::mutex g_dev_mu;
+
+const std::vector<KernelSet>& kernel_sets() {
+  static const std::vector<KernelSet> sets = [] {
+    std::vector<KernelSet> v;
+#define BEAM_PUSH(BM, BN, TM, TN) v.push_back(kernel_set_##BM##x##BN##_##TM##x##TN());
+    BEAM_FOR_EACH_SET(BEAM_PUSH)
+#undef BEAM_PUSH
+    return v;
+  }();
+  return sets;
+}
+
+const KernelSet* find_set(const beam_tile_cfg& c) {
+  for (const KernelSet& k : kernel_sets())
+    if (k.block_m == c.block_m && k.block_n == c.block_n && k.wave_m == c.wave_m && k.wave_n == c.wave_n)
+      return &k;
+  return nullptr;
+}
+
+constexpr int kDefaultGroupM = 8;
+constexpr int kMaxK = 1 << 22;
+
+int check_problem(const void* A, const void* B, const void* C, int M, int N, int K, int dtype) {
+  if (M < 0 || N < 0 || K < 0) return fail(BEAM_ERR_INVALID, "negative dimension (M=%d N=%d K=%d)", M, N, K);
+  if (dtype != BEAM_F16 && dtype != BEAM_BF16) return fail(BEAM_ERR_UNSUPPORTED, "dtype %d: only fp16 (0) and bf16 (1)", dtype);
+  if (M == 0 || N == 0) return BEAM_OK;
+  if (!C) return fail(BEAM_ERR_INVALID, "null output pointer");
+  if (K > 0 && (!A || !B)) return fail(BEAM_ERR_INVALID, "null input pointer");
+  if (K > kMaxK) return fail(BEAM_ERR_UNSUPPORTED, "K=%d exceeds %d", K, kMaxK);
+  if (K % 8 != 0) return fail(BEAM_ERR_UNSUPPORTED, "K=%d: rows must be multiples of 16 bytes (K %% 8 == 0)", K);
+  if (((uintptr_t)A | (uintptr_t)B) & 15) return fail(BEAM_ERR_UNSUPPORTED, "A and B must be 16-byte aligned");
+  if ((uintptr_t)C & 7) return fail(BEAM_ERR_UNSUPPORTED, "C must be 8-byte aligned");
+  if ((size_t)M * (size_t)N >= ((size_t)1 << 40)) return fail(BEAM_ERR_UNSUPPORTED, "M*N too large");
+  return BEAM_OK;
+}
+
+int resolve_cfg(const beam_tile_cfg* in, int M, int N, int K, beam_tile_cfg* out, const KernelSet** ks) {
+  if (in) {
+    *out = *in;
+  } else {
+    int s;
+    int rc = beam_default_config(M, N, K, out, &s);
+    if (rc) return rc;
+  }
+  if (out->loader != 0 && out->loader != 1) return fail(BEAM_ERR_UNSUPPORTED, "loader %d: 0 (direct to LDS) or 1 (register staged)", out->loader);
+  if (out->group_m <= 0) out->group_m = kDefaultGroupM;
+  *ks = find_set(*out);
+  if (!*ks)
+    return fail(BEAM_ERR_UNSUPPORTED, "no kernel for workgroup tile %dx%d / wavefront tile %dx%d", out->block_m,
+                out->block_n, out->wave_m, out->wave_n);
+  return BEAM_OK;
+}
+
+GemmParams base_params(const void* A, const void* B, int M, int N, int K, const beam_tile_cfg& c) {
+  GemmParams p;
+  std::memset(&p, 0, sizeof p);
+  p.A = A;
+  p.B = B;
+  p.M = M;
+  p.N = N;
+  p.K = K;
+  p.tiles_m = (M + c.block_m - 1) / c.block_m;
+  p.tiles_n = (N + c.block_n - 1) / c.block_n;
+  p.k_slice = ((K + kBK - 1) / kBK) * kBK;
+  if (p.k_slice == 0) p.k_slice = kBK;
+  p.group_m = c.group_m;
+  return p;
+}
+
+size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
+
+// ---- host data generation -------------------------------------------------------------
+
+inline uint64_t mix64(uint64_t x) {  // splitmix64 finaliser
+  x += 0x9E3779B97F4A7C15ull;
+  x = (x ^ (x >> 30)) * 0xBF58476D1CE4E5B9ull;
+  x = (x ^ (x >> 27)) * 0x94D049BB133111EBull;
+  return x ^ (x >> 31);
+}
+
+inline uint64_t draw(uint64_t seed, uint64_t tensor_id, uint64_t i) {
+  return mix64(mix64(seed + 0x632BE59BD9B4E019ull * (tensor_id + 1)) + i);
+}
+
+inline uint32_t f32_bits(float f) {
+  uint32_t u;
+  std::memcpy(&u, &f, 4);
+  return u;
+}
+
+inline uint16_t to_bf16_bits(float f) {
+  uint32_t x = f32_bits(f);
+  if ((x & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((x >> 16) | 0x40u);
+  return (uint16_t)((x + 0x7fffu + ((x >> 16) & 1u)) >> 16);
+}
+
+inline uint16_t to_f16_bits(float f) {
+  // Round the significand to 11 bits in float arithmetic, then repack.
+  const uint32_t x = f32_bits(f);
+  const uint16_t sign = (uint16_t)((x >> 16) & 0x8000u);
+  const uint32_t ax = x & 0x7fffffffu;
+  if (ax > 0x7f800000u) return (uint16_t)(sign | 0x7e00u);
+  if (ax >= 0x477ff000u) return (uint16_t)(sign | 0x7c00u);
+  float a;
+  std::memcpy(&a, &ax, 4);
+  if (ax < 0x38800000u) {
+    // subnormal half: a / 2^-24 rounded to nearest even integer
+    const float scaled = a * 16777216.0f;
+    const float r = std::nearbyintf(scaled);  // default rounding mode = to nearest even
+    return (uint16_t)(sign | (uint16_t)r);
+  }
+  uint32_t r = ax + 0xfffu + ((ax >> 13) & 1u);  // RN-even at bit 13
+  return (uint16_t)(sign | ((r - 0x38000000u) >> 13));
+}
+
+template <typename F>
+void parallel_for(size_t n, F f) {
+  unsigned hw = std::thread::hardware_concurrency();
+  unsigned nt = hw == 0 ? 4 : (hw > 16 ? 16 : hw);
+  if (n < (1u << 16)) nt = 1;
+  std::vector<std::thread> th;
+  const size_t chunk = (n + nt - 1) / nt;
+  for (unsigned t = 0; t < nt; ++t) {
+    const size_t lo = t * chunk, hi = lo + chunk < n ? lo + chunk : n;
+    if (lo >= hi) break;
+    th.emplace_back([=] { f(lo, hi); });
+  }
+  for (auto& t : th) t.join();
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* beam_last_error(void) { return g_err; }
+
+int beam_init(void) {
+  std::lock_guard<std::mutex> lk(g_dev_mu);
+  if (g_dev.status >= 0) return g_dev.status == BEAM_OK ? BEAM_OK : fail(g_dev.status, "device probe failed earlier");
+  int n = 0;
+  hipError_t e = hipGetDeviceCount(&n);
+  if (e != hipSuccess || n == 0) {
+    g_dev.status = BEAM_ERR_HIP;
+    return fail(BEAM_ERR_HIP, "no HIP device (%s)", e == hipSuccess ? "count is zero" : hipGetErrorString(e));
+  }
+  hipDeviceProp_t prop;
+  e = hipGetDeviceProperties(&prop, 0);
+  if (e != hipSuccess) {
+    g_dev.status = BEAM_ERR_HIP;
+    return hip_fail(e, "hipGetDeviceProperties");
+  }
+  std::snprintf(g_dev.name, sizeof g_dev.name, "%s (%s)", prop.name, prop.gcnArchName);
+  g_dev.cus = prop.multiProcessorCount;
+  g_dev.clock_khz = prop.clockRate;
+  g_dev.mem = prop.totalGlobalMem;
+  if (std::strncmp(prop.gcnArchName, "gfx950", 6) != 0) {
+    g_dev.status = BEAM_ERR_DEVICE;
+    return fail(BEAM_ERR_DEVICE, "device 0 is %s; this library holds gfx950 code only", prop.gcnArchName);
+  }
+  g_dev.status = BEAM_OK;
+  return BEAM_OK;
+}
+
+int beam_device_info(char* name, int len, int* compute_units, int* clock_khz, size_t* mem_bytes) {
+  int rc = beam_init();
+  if (rc != BEAM_OK && rc != BEAM_ERR_DEVICE) return rc;
+  if (name && len > 0) std::snprintf(name, (size_t)len, "%s", g_dev.name);
+  if (compute_units) *compute_units = g_dev.cus;
+  if (clock_khz) *clock_khz = g_dev.clock_khz;
+  if (mem_bytes) *mem_bytes = g_dev.mem;
+  return rc;
+}
+
+int beam_num_configs(void) { return (int)kernel_sets().size(); }
+
+int beam_get_config(int index, beam_tile_cfg* out) {
+  if (!out || index < 0 || index >= beam_num_configs()) return fail(BEAM_ERR_INVALID, "config index %d out of range", index);
+  const KernelSet& k = kernel_sets()[index];
+  out->block_m = k.block_m;
+  out->block_n = k.block_n;
+  out->wave_m = k.wave_m;
+  out->wave_n = k.wave_n;
+  out->loader = 0;
+  out->group_m = kDefaultGroupM;
+  return BEAM_OK;
+}
+
+int beam_slice_heuristic(int tiles, int compute_units) {
+  if (tiles < 1) tiles = 1;
+  const float units = (float)compute_units;
+  int s = 1;
+  if ((float)tiles < units) {
+    s = (int)((units - 1.0f) / (float)tiles + 1.0f);
+    float waves = (float)s * (float)tiles / units;
+    float rem = waves - (float)(int)waves;
+    while (rem < 0.5f) {
+      ++s;
+      waves = (float)s * (float)tiles / units;
+      rem = waves - (float)(int)waves;
+    }
+  }
+  return s;
+}
+
+int beam_default_config(int M, int N, int K, beam_tile_cfg* cfg, int* split_k) {
+  if (!cfg) return fail(BEAM_ERR_INVALID, "null cfg");
+  const int cus = g_dev.cus > 0 ? g_dev.cus : 256;
+  auto tiles = [&](int bm, int bn) { return (long)((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
+  beam_tile_cfg c = {256, 256, 128, 64, 0, kDefaultGroupM};
+  if (tiles(256, 256) >= (cus * 3) / 4) {
+    // big enough to fill the device with the largest tile
+  } else if (tiles(256, 128) >= (cus * 3) / 4) {
+    c = {256, 128, 64, 64, 0, kDefaultGroupM};
+  } else if (tiles(128, 128) >= cus / 2) {
+    c = {128, 128, 64, 64, 0, kDefaultGroupM};
+  } else if (tiles(128, 64) >= cus / 2) {
+    c = {128, 64, 64, 32, 0, kDefaultGroupM};
+  } else {
+    c = {64, 64, 32, 32, 0, kDefaultGroupM};
+  }
+  *cfg = c;
+  if (split_k) {
+    const long t = tiles(c.block_m, c.block_n);
+    int s = 1;
+    if (t < cus / 2 && K >= 2048) {
+      s = beam_slice_heuristic((int)t, cus);
+      const int ktiles = (K + kBK - 1) / kBK;
+      if (s > ktiles / 4) s = ktiles / 4;  // keep at least 4 K tiles per slice
+      if (s < 1) s = 1;
+    }
+    *split_k = s;
+  }
+  return BEAM_OK;
+}
+
+int beam_gemmrc(const void* A, const void* B, void* C, int M, int N, int K, int dtype,
+                const beam_tile_cfg* cfg, void* stream) {
+  int rc = check_problem(A, B, C, M, N, K, dtype);
+  if (rc) return rc;
+  if (M == 0 || N == 0) return BEAM_OK;
+  if ((rc = beam_init())) return rc;
+  hipStream_t st = (hipStream_t)stream;
+  if (K == 0) {
+    BEAM_HIP(hipMemsetAsync(C, 0, (size_t)M * N * 2, st));
+    return BEAM_OK;
+  }
+  beam_tile_cfg c;
+  const KernelSet* ks;
+  if ((rc = resolve_cfg(cfg, M, N, K, &c, &ks))) return rc;
+  GemmParams p = base_params(A, B, M, N, K, c);
+  p.C = C;
+  BEAM_HIP(ks->launch[dtype][kEpiStore][c.loader](p, dim3((unsigned)(p.tiles_m * p.tiles_n), 1, 1), st));
+  return BEAM_OK;
+}
+
+static int custom_fixed(int bm, int bn, int tm, int tn, const void* A, const void* B, void* C, int M,
+                        int N, int K, void* stream) {
+  beam_tile_cfg c = {bm, bn, tm, tn, 0, 0};
+  return beam_gemmrc(A, B, C, M, N, K, BEAM_F16, &c, stream);
+}
+
+int beam_custom_gemmrc_128x128(const void* A, const void* B, void* C, int M, int N, int K, void* stream) {
+  return custom_fixed(128, 128, 64, 64, A, B, C, M, N, K, stream);
+}
+int beam_custom_gemmrc_128x256(const void* A, const void* B, void* C, int M, int N, int K, void* stream) {
+  return custom_fixed(128, 256, 64, 64, A, B, C, M, N, K, stream);
+}
+int beam_custom_gemmrc_256x128(const void* A, const void* B, void* C, int M, int N, int K, void* stream) {
+  return custom_fixed(256, 128, 64, 64, A, B, C, M, N, K, stream);
+}
+
+size_t beam_splitk_workspace_bytes(int M, int N, int split_k) {
+  if (M <= 0 || N <= 0 || split_k <= 0) return 0;
+  return (size_t)split_k * (size_t)M * (size_t)N * sizeof(float);
+}
+
+static int effective_split(int M, int N, int K, const beam_tile_cfg& c, int split_k) {
+  const int ktiles = (K + kBK - 1) / kBK;
+  if (ktiles <= 1) return 1;
+  int s = split_k;
+  if (s <= 0) {
+    const int cus = g_dev.cus > 0 ? g_dev.cus : 256;
+    const long t = (long)((M + c.block_m - 1) / c.block_m) * ((N + c.block_n - 1) / c.block_n);
+    s = beam_slice_heuristic((int)(t > 1 << 20 ? 1 << 20 : t), cus);
+  }
+  if (s > ktiles) s = ktiles;
+  if (s < 1) s = 1;
+  const int per = (ktiles + s - 1) / s;
+  return (ktiles + per - 1) / per;  // drop slices that would be empty
+}
+
+int beam_splitk_effective(int M, int N, int K, const beam_tile_cfg* cfg, int split_k) {
+  beam_tile_cfg c;
+  const KernelSet* ks;
+  if (M <= 0 || N <= 0 || K < 0) return 1;
+  if (resolve_cfg(cfg, M, N, K, &c, &ks)) return -1;
+  return effective_split(M, N, K, c, split_k);
+}
+
+int beam_gemmrc_splitk(const void* A, const void* B, void* C, int M, int N, int K, int dtype,
+                       const beam_tile_cfg* cfg, int split_k, void* ws, size_t ws_bytes, void* stream) {
+  int rc = check_problem(A, B, C, M, N, K, dtype);
+  if (rc) return rc;
+  if (M == 0 || N == 0) return BEAM_OK;
+  if ((rc = beam_init())) return rc;
+  hipStream_t st = (hipStream_t)stream;
+  if (K == 0) {
+    BEAM_HIP(hipMemsetAsync(C, 0, (size_t)M * N * 2, st));
+    return BEAM_OK;
+  }
+  beam_tile_cfg c;
+  const KernelSet* ks;
+  if ((rc = resolve_cfg(cfg, M, N, K, &c, &ks))) return rc;
+  const int s = effective_split(M, N, K, c, split_k);
+  if (s == 1) {  // nothing to reduce: the plain kernel writes C directly
+    GemmParams p = base_params(A, B, M, N, K, c);
+    p.C = C;
+    BEAM_HIP(ks->launch[dtype][kEpiStore][c.loader](p, dim3((unsigned)(p.tiles_m * p.tiles_n), 1, 1), st));
+    return BEAM_OK;
+  }
+  const size_t need = beam_splitk_workspace_bytes(M, N, s);
+  if (!ws || ws_bytes < need)
+    return fail(BEAM_ERR_WORKSPACE, "split-K with %d slices needs %zu bytes of workspace, got %zu", s, need, ws_bytes);
+  if ((uintptr_t)ws & 15) return fail(BEAM_ERR_UNSUPPORTED, "workspace must be 16-byte aligned");
+  GemmParams p = base_params(A, B, M, N, K, c);
+  p.ws = (float*)ws;
+  p.k_slice = split_k_len(K, s);
+  BEAM_HIP(ks->launch[dtype][kEpiPartial][c.loader](p, dim3((unsigned)(p.tiles_m * p.tiles_n), 1, (unsigned)s), st));
+  BEAM_HIP(launch_splitk_reduce((const float*)ws, C, (size_t)M * N, s, dtype, st));
+  return BEAM_OK;
+}
+
+size_t beam_gemmrc_ln_workspace_bytes(int M, int N, const beam_tile_cfg* cfg) {
+  if (M <= 0 || N <= 0) return 0;
+  beam_tile_cfg c;
+  const KernelSet* ks;
+  if (resolve_cfg(cfg, M, N, 64, &c, &ks)) return 0;
+  const size_t tiles_n = (size_t)(N + c.block_n - 1) / c.block_n;
+  return align_up((size_t)M * N * sizeof(float), 256) + align_up((size_t)M * tiles_n * 2 * sizeof(float), 256);
+}
+
+int beam_gemmrc_ln(const void* A, const void* B, const void* gamma, const void* beta, float eps, void* Y,
+                   int M, int N, int K, int dtype, const beam_tile_cfg* cfg, void* ws, size_t ws_bytes,
+                   void* stream) {
+  int rc = check_problem(A, B, Y, M, N, K, dtype);
+  if (rc) return rc;
+  if (M == 0 || N == 0) return BEAM_OK;
+  if (!gamma || !beta) return fail(BEAM_ERR_INVALID, "null gamma/beta");
+  if (((uintptr_t)gamma | (uintptr_t)beta) & 7) return fail(BEAM_ERR_UNSUPPORTED, "gamma and beta must be 8-byte aligned");
+  if (!(eps >= 0.0f)) return fail(BEAM_ERR_INVALID, "eps must be >= 0");
+  if ((rc = beam_init())) return rc;
+  hipStream_t st = (hipStream_t)stream;
+  beam_tile_cfg c;
+  const KernelSet* ks;
+  if ((rc = resolve_cfg(cfg, M, N, K, &c, &ks))) return rc;
+  const size_t need = beam_gemmrc_ln_workspace_bytes(M, N, &c);
+  if (!ws || ws_bytes < need)
+    return fail(BEAM_ERR_WORKSPACE, "GEMM+LayerNorm needs %zu bytes of workspace, got %zu", need, ws_bytes);
+  if ((uintptr_t)ws & 255) return fail(BEAM_ERR_UNSUPPORTED, "workspace must be 256-byte aligned");
+  GemmParams p = base_params(A, B, M, N, K, c);
+  p.ws = (float*)ws;
+  p.stats = (float*)((char*)ws + align_up((size_t)M * N * sizeof(float), 256));
+  // K == 0: the kernel runs with an empty K range and produces x = 0, i.e. y = beta.
+  BEAM_HIP(ks->launch[dtype][kEpiLnStats][c.loader](p, dim3((unsigned)(p.tiles_m * p.tiles_n), 1, 1), st));
+  BEAM_HIP(launch_ln_apply(p.ws, p.stats, gamma, beta, Y, M, N, p.tiles_n, c.block_n, eps, dtype, st));
+  return BEAM_OK;
+}
+
+int beam_bench(int op, const beam_problem* q, const beam_tile_cfg* cfg, int warmup, int iters, void* stream,
+               float* avg_ms) {
+  if (!q || !avg_ms || iters < 1 || warmup < 0) return fail(BEAM_ERR_INVALID, "bad bench arguments");
+  auto once = [&]() -> int {
+    switch (op) {
+      case BEAM_OP_GEMM:
+        return beam_gemmrc(q->A, q->B, q->C, q->M, q->N, q->K, q->dtype, cfg, stream);
+      case BEAM_OP_SPLITK:
+        return beam_gemmrc_splitk(q->A, q->B, q->C, q->M, q->N, q->K, q->dtype, cfg, q->split_k, q->ws,
+                                  q->ws_bytes, stream);
+      case BEAM_OP_GEMM_LN:
+        return beam_gemmrc_ln(q->A, q->B, q->gamma, q->beta, q->eps, q->C, q->M, q->N, q->K, q->dtype, cfg,
+                              q->ws, q->ws_bytes, stream);
+      default:
+        return fail(BEAM_ERR_INVALID, "unknown op %d", op);
+    }
+  };
+  hipStream_t st = (hipStream_t)stream;
+  for (int i = 0; i < warmup; ++i) {
+    int rc = once();
+    if (rc) return rc;
+  }
+  hipEvent_t e0, e1;
+  BEAM_HIP(hipEventCreate(&e0));
+  BEAM_HIP(hipEventCreate(&e1));
+  int rc = BEAM_OK;
+  hipError_t he = hipEventRecord(e0, st);
+  for (int i = 0; i < iters && rc == BEAM_OK && he == hipSuccess; ++i) rc = once();
+  if (he == hipSuccess) he = hipEventRecord(e1, st);
+  if (he == hipSuccess) he = hipEventSynchronize(e1);
+  float ms = 0.0f;
+  if (he == hipSuccess) he = hipEventElapsedTime(&ms, e0, e1);
+  (void)hipEventDestroy(e0);
+  (void)hipEventDestroy(e1);
+  if (rc) return rc;
+  if (he != hipSuccess) return hip_fail(he, "event timing");
+  *avg_ms = ms / (float)iters;
+  return BEAM_OK;
+}
+
+int beam_event_create(void** event) {
+  if (!event) return fail(BEAM_ERR_INVALID, "null event");
+  hipEvent_t e;
+  BEAM_HIP(hipEventCreate(&e));
+  *event = (void*)e;
+  return BEAM_OK;
+}
+int beam_event_record(void* event, void* stream) {
+  if (!event) return fail(BEAM_ERR_INVALID, "null event");
+  BEAM_HIP(hipEventRecord((hipEvent_t)event, (hipStream_t)stream));
+  return BEAM_OK;
+}
+int beam_event_elapsed_ms(void* start, void* stop, float* ms) {
+  if (!start || !stop || !ms) return fail(BEAM_ERR_INVALID, "null event");
+  BEAM_HIP(hipEventSynchronize((hipEvent_t)stop));
+  BEAM_HIP(hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop));
+  return BEAM_OK;
+}
+int beam_event_destroy(void* event) {
+  if (event) BEAM_HIP(hipEventDestroy((hipEvent_t)event));
+  return BEAM_OK;
+}
+
+int beam_malloc(void** dptr, size_t bytes) {
+  if (!dptr) return fail(BEAM_ERR_INVALID, "null dptr");
+  *dptr = nullptr;
+  if (bytes == 0) return BEAM_OK;
+  BEAM_HIP(hipMalloc(dptr, bytes));
+  return BEAM_OK;
+}
+int beam_free(void* dptr) {
+  if (dptr) BEAM_HIP(hipFree(dptr));
+  return BEAM_OK;
+}
+int beam_memcpy_h2d(void* dst, const void* src_host, size_t bytes) {
+  if (bytes) BEAM_HIP(hipMemcpy(dst, src_host, bytes, hipMemcpyHostToDevice));
+  return BEAM_OK;
+}
+int beam_memcpy_d2h(void* dst_host, const void* src, size_t bytes) {
+  if (bytes) BEAM_HIP(hipMemcpy(dst_host, src, bytes, hipMemcpyDeviceToHost));
+  return BEAM_OK;
+}
+int beam_memset(void* dptr, int byte, size_t bytes) {
+  if (bytes) BEAM_HIP(hipMemset(dptr, byte, bytes));
+  return BEAM_OK;
+}
+int beam_sync(void* stream) {
+  BEAM_HIP(hipStreamSynchronize((hipStream_t)stream));
+  return BEAM_OK;
+}
+
+int beam_host_fill_uniform(void* dst_host, size_t n, int dtype, uint64_t seed, uint64_t tensor_id) {
+  if (!dst_host && n) return fail(BEAM_ERR_INVALID, "null destination");
+  if (dtype != BEAM_F16 && dtype != BEAM_BF16) return fail(BEAM_ERR_UNSUPPORTED, "dtype %d", dtype);
+  uint16_t* out = (uint16_t*)dst_host;
+  parallel_for(n, [=](size_t lo, size_t hi) {
+    for (size_t i = lo; i < hi; ++i) {
+      const uint64_t r = draw(seed, tensor_id, i);
+      const float v = (float)(r >> 40) * (1.0f / 8388608.0f) - 1.0f;  // 24 bits -> [-1, 1)
+      out[i] = dtype == BEAM_BF16 ? to_bf16_bits(v) : to_f16_bits(v);
+    }
+  });
+  return BEAM_OK;
+}
+
+int beam_host_fill_normal(void* dst_host, size_t n, int dtype, uint64_t seed, uint64_t tensor_id, float mean,
+                          float scale) {
+  if (!dst_host && n) return fail(BEAM_ERR_INVALID, "null destination");
+  if (dtype != BEAM_F16 && dtype != BEAM_BF16) return fail(BEAM_ERR_UNSUPPORTED, "dtype %d", dtype);
+  uint16_t* out = (uint16_t*)dst_host;
+  parallel_for(n, [=](size_t lo, size_t hi) {
+    for (size_t i = lo; i < hi; ++i) {
+      const uint64_t r = draw(seed, tensor_id, i);
+      const double u1 = ((double)(r >> 40) + 1.0) * (1.0 / 16777216.0);      // (0, 1]
+      const double u2 = (double)((r >> 8) & 0xffffffull) * (1.0 / 16777216.0);  // [0, 1)
+      const double z = std::sqrt(-2.0 * std::log(u1)) * std::cos(6.283185307179586476925 * u2);
+      const float v = (float)((double)mean + (double)scale * z);
+      out[i] = dtype == BEAM_BF16 ? to_bf16_bits(v) : to_f16_bits(v);
+    }
+  });
+  return BEAM_OK;
+}
+
+int beam_dbg_tile_of_workgroup(int wg, int tiles_m, int tiles_n, int group_m, int* tm, int* tn) {
+  if (tiles_m < 1 || tiles_n < 1 || group_m < 1 || wg < 0 || wg >= tiles_m * tiles_n || !tm || !tn)
+    return fail(BEAM_ERR_INVALID, "bad rasterisation query");
+  const TileCoord t = tile_of_workgroup(wg, tiles_m, tiles_n, group_m);
+  *tm = t.tm;
+  *tn = t.tn;
+  return BEAM_OK;
+}
+
+int beam_dbg_lds_offset(int row, int chunk) { return lds_offset(row, chunk); }
+
+}  // extern "C"

@@ -1,0 +1,6 @@
+// gemmrc kernels for workgroup tile 128x128, wavefront tile 64x32 (all dtypes, epilogues, loaders).
+#include "kernel_set.h"
+
+namespace beam {
+BEAM_DEFINE_SET(128, 128, 64, 32)
+}  // namespace beam

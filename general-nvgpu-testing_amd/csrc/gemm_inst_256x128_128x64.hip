@@ -1,0 +1,6 @@
+// gemmrc kernels for workgroup tile 256x128, wavefront tile 128x64 (all dtypes, epilogues, loaders).
+#include "kernel_set.h"
+
+namespace beam {
+BEAM_DEFINE_SET(256, 128, 128, 64)
+}  // namespace beam

@@ -1,0 +1,83 @@
+// Table of compiled gemmrc kernels: one KernelSet per (workgroup tile, wavefront tile),
+// holding a launcher for every (dtype, epilogue, loader) combination.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include "../../include/beam_hip.h"
+#include "gemm_kernel.h"
+
+namespace beam {
+
+typedef hipError_t (*GemmLauncher)(const GemmParams& p, dim3 grid, hipStream_t stream);
+
+struct KernelSet {
+  int block_m, block_n, wave_m, wave_n;
+  int threads;
+  int lds_bytes;
+  GemmLauncher launch[2][3][2];  // [dtype][epilogue][loader: 0 direct, 1 staged]
+};
+
+template <typename T, int BM, int BN, int WVM, int WVN, int EPI, bool DIRECT>
+hipError_t launch_gemm(const GemmParams& p, dim3 grid, hipStream_t stream) {
+  using Tile = GemmTile<T, BM, BN, WVM, WVN, EPI, DIRECT>;
+  auto kern = gemmrc_kernel<T, BM, BN, WVM, WVN, EPI, DIRECT>;
+  static bool configured = false;  // benign race: the attribute call is idempotent
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, Tile::LDS_BYTES);
+    if (e != hipSuccess) return e;
+    configured = true;
+  }
+  hipLaunchKernelGGL(kern, grid, dim3(Tile::NT), Tile::LDS_BYTES, stream, p);
+  return hipGetLastError();
+}
+
+template <int BM, int BN, int TM, int TN>
+KernelSet make_kernel_set() {
+  constexpr int WVM = BM / TM, WVN = BN / TN;
+  KernelSet k;
+  k.block_m = BM;
+  k.block_n = BN;
+  k.wave_m = TM;
+  k.wave_n = TN;
+  k.threads = WVM * WVN * 64;
+  k.lds_bytes = GemmTile<_Float16, BM, BN, WVM, WVN, kEpiStore, true>::LDS_BYTES;
+#define BEAM_FILL(D, T)                                                             \
+  k.launch[D][kEpiStore][0] = launch_gemm<T, BM, BN, WVM, WVN, kEpiStore, true>;     \
+  k.launch[D][kEpiStore][1] = launch_gemm<T, BM, BN, WVM, WVN, kEpiStore, false>;    \
+  k.launch[D][kEpiPartial][0] = launch_gemm<T, BM, BN, WVM, WVN, kEpiPartial, true>; \
+  k.launch[D][kEpiPartial][1] = launch_gemm<T, BM, BN, WVM, WVN, kEpiPartial, false>; \
+  k.launch[D][kEpiLnStats][0] = launch_gemm<T, BM, BN, WVM, WVN, kEpiLnStats, true>; \
+  k.launch[D][kEpiLnStats][1] = launch_gemm<T, BM, BN, WVM, WVN, kEpiLnStats, false>;
+  BEAM_FILL(0, _Float16)
+  BEAM_FILL(1, __bf16)
+#undef BEAM_FILL
+  return k;
+}
+
+// One definition per instantiation file (gemm_inst_*.hip).
+#define BEAM_DECLARE_SET(BM, BN, TM, TN) KernelSet kernel_set_##BM##x##BN##_##TM##x##TN();
+#define BEAM_DEFINE_SET(BM, BN, TM, TN) \
+  KernelSet kernel_set_##BM##x##BN##_##TM##x##TN() { return make_kernel_set<BM, BN, TM, TN>(); }
+
+// (workgroup tile M, N, wavefront tile M, N)
+#define BEAM_FOR_EACH_SET(X) \
+  X(256, 256, 128, 64)       \
+  X(256, 256, 64, 128)       \
+  X(256, 256, 128, 128)      \
+  X(256, 128, 64, 64)        \
+  X(256, 128, 128, 32)       \
+  X(256, 128, 32, 128)       \
+  X(256, 128, 128, 64)       \
+  X(128, 256, 64, 64)        \
+  X(128, 256, 64, 128)       \
+  X(128, 128, 64, 64)        \
+  X(128, 128, 64, 32)        \
+  X(128, 64, 64, 32)         \
+  X(64, 128, 32, 64)         \
+  X(64, 64, 32, 32)
+
+BEAM_FOR_EACH_SET(BEAM_DECLARE_SET)
+
+}  // namespace beam

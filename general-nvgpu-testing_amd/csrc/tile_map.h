@@ -1,0 +1,82 @@
+// Integer index maps shared by device kernels and host-side checks.
+//
+// Everything here is plain integer arithmetic, callable from host and device, so the
+// host can verify (by brute force) that each map is a bijection and that the LDS
+// layout is bank-conflict free before any kernel is launched.
+//
+// Reference counterparts:
+//   * workgroup -> tile rasterisation ("mtile" grouping):
+//       cuda/cute_kernels/cute_gemm_128x128.cu:22-33, cute_gemm_128x256.cu:26-37
+//   * shared-memory XOR swizzle of 16-byte chunks:
+//       cuda/cute_kernels/cute_gemm_128x128.cu:55-65  (Swizzle<3,3,3>)
+#pragma once
+
+#if defined(__HIPCC__) || defined(__CUDACC__)
+#define BEAM_HD __host__ __device__ inline
+#else
+#define BEAM_HD inline
+#endif
+
+namespace beam {
+
+// K extent (elements) of one LDS stage: 64 x 2 bytes = 128 bytes = 8 chunks of 16 bytes.
+constexpr int kBK = 64;
+constexpr int kRowBytes = kBK * 2;
+constexpr int kChunksPerRow = 8;
+// MI355X: 8 accelerator complex dies, workgroups are dispatched to them round-robin.
+constexpr int kNumXcd = 8;
+
+// XOR pattern applied to the 16-byte chunk index of an LDS row.
+// LDS has 64 banks of 4 bytes (256 bytes per bank sweep) and rows are 128 bytes, so two
+// consecutive rows share a sweep; 16 consecutive rows of the same logical chunk land on
+// 16 distinct 16-byte slots when the chunk is XORed with (row >> 1) & 7.
+BEAM_HD int swizzle_of_row(int row) { return (row >> 1) & 7; }
+
+// Byte offset inside a stage of logical (row, chunk) after swizzling.
+BEAM_HD int lds_offset(int row, int chunk) {
+  return row * kRowBytes + ((chunk ^ swizzle_of_row(row)) << 4);
+}
+
+struct TileCoord {
+  int tm;  // tile index along M
+  int tn;  // tile index along N
+};
+
+// Workgroup id -> linear tile id such that the workgroups living on one XCD (ids congruent
+// modulo 8) own one contiguous range of tile ids. Bijection on [0, total).
+BEAM_HD int xcd_remap(int wg, int total) {
+  const int base = total / kNumXcd;
+  const int rem = total % kNumXcd;
+  const int xcd = wg % kNumXcd;
+  const int local = wg / kNumXcd;
+  return xcd * base + (xcd < rem ? xcd : rem) + local;
+}
+
+// Linear tile id -> (tm, tn): groups of `group_m` tile rows, M fastest inside a group, so
+// that workgroups with neighbouring ids reuse the same B panel and a small set of A panels
+// out of the XCD-private L2.
+BEAM_HD TileCoord grouped_tile(int pid, int tiles_m, int tiles_n, int group_m) {
+  const int gsize = group_m * tiles_n;
+  const int g = pid / gsize;
+  const int first_m = g * group_m;
+  const int rows = (tiles_m - first_m) < group_m ? (tiles_m - first_m) : group_m;
+  const int within = pid - g * gsize;
+  TileCoord t;
+  t.tm = first_m + within % rows;
+  t.tn = within / rows;
+  return t;
+}
+
+BEAM_HD TileCoord tile_of_workgroup(int wg, int tiles_m, int tiles_n, int group_m) {
+  return grouped_tile(xcd_remap(wg, tiles_m * tiles_n), tiles_m, tiles_n, group_m);
+}
+
+// K range [begin, end) of split slice `z` out of `splits`: every slice gets the same whole
+// number of kBK-wide K tiles (the last ones may be short or empty). Matches the CUTLASS
+// partitioning the reference relies on (cuda/cutlass_kernels/cutlass_gemmrc_splitk.cu:95-99).
+BEAM_HD int split_k_len(int K, int splits) {
+  const int ktiles = (K + kBK - 1) / kBK;
+  return ((ktiles + splits - 1) / splits) * kBK;
+}
+
+}  // namespace beam

@@ -1,0 +1,174 @@
+/*
+ * beam_hip.h -- C ABI of the MI355X (gfx950) gemmrc library, libbeam_hip.so.
+ *
+ * gemmrc:  C[M][N] = A[M][K] . B[N][K]^T   (A, B, C row-major 16-bit; fp32 accumulation on the
+ * matrix cores; round-to-nearest-even output).  All pointers are DEVICE pointers unless the
+ * name says host.  Every entry point returns a beam_status; nothing aborts, nothing returns
+ * silently leaving C untouched.  Launches are asynchronous on the stream passed in
+ * (a hipStream_t cast to void*, NULL = the default stream).
+ *
+ * Each declaration cites the reference interface it stands in for
+ * (paths relative to the reference repository).
+ */
+#ifndef BEAM_HIP_H
+#define BEAM_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum beam_status {
+  BEAM_OK = 0,
+  BEAM_ERR_INVALID = 1,     /* bad pointer / shape / argument                                 */
+  BEAM_ERR_UNSUPPORTED = 2, /* tile / dtype / alignment combination that has no kernel        */
+  BEAM_ERR_WORKSPACE = 3,   /* workspace missing or too small                                 */
+  BEAM_ERR_HIP = 4,         /* HIP runtime error, text in beam_last_error()                   */
+  BEAM_ERR_DEVICE = 5       /* not a gfx950 device                                            */
+} beam_status;
+
+typedef enum beam_dtype { BEAM_F16 = 0, BEAM_BF16 = 1 } beam_dtype;
+
+/* One point of the tunable space.
+ * Replaces the (shape_threadblock, shape_warp) pair of
+ * cuda/cutlass_kernels/main.cc:125-142 and cuda/cutlass_kernels/cutlass_gemmrc.cu:85-110. */
+typedef struct beam_tile_cfg {
+  int block_m, block_n; /* workgroup tile of C ("shape_threadblock")                          */
+  int wave_m, wave_n;   /* wavefront tile ("shape_warp"); block/wave = wavefront grid         */
+  int loader;           /* 0 = buffer loads straight into LDS, 1 = staged through registers   */
+  int group_m;          /* rasterisation group height in tiles; 0 = library default           */
+} beam_tile_cfg;
+
+/* ---- library ------------------------------------------------------------------------- */
+
+/* Checks that device 0 is gfx950 and raises the kernels' LDS limits.  Called implicitly.
+ * Stands in for the module initialiser cuda/main.cc:51-60. */
+int beam_init(void);
+/* Text of the last error on the calling thread ("" if none). */
+const char* beam_last_error(void);
+/* name[<=len], compute units, peak engine clock (kHz), total device memory (bytes). */
+int beam_device_info(char* name, int len, int* compute_units, int* clock_khz, size_t* mem_bytes);
+
+/* ---- tunable space -------------------------------------------------------------------- */
+
+/* Number of compiled tile configurations and the i-th of them (both dtypes share the table).
+ * Replaces the hard-coded search spaces of python/beam/tuner.py:52-95. */
+int beam_num_configs(void);
+int beam_get_config(int index, beam_tile_cfg* out);
+/* Library default for a problem: writes the configuration and the split factor (1 = no
+ * split).  Replaces CUTLASS's default shapes, cuda/cutlass_kernels/cutlass_gemmrc.cu:22-24. */
+int beam_default_config(int M, int N, int K, beam_tile_cfg* cfg, int* split_k);
+
+/* ---- tiled GEMM ------------------------------------------------------------------------ */
+
+/* cfg == NULL: beam_default_config() picks the tile (never a split).
+ * Replaces entry_cutlass_gemmrc / entry_cutlass_gemmrc_spec
+ * (cuda/cutlass_kernels/main.cc:11-15, cutlass_gemmrc.cu:21-40,55-111). */
+int beam_gemmrc(const void* A, const void* B, void* C, int M, int N, int K, int dtype,
+                const beam_tile_cfg* cfg, void* stream);
+
+/* fp16 only, fixed tiles, same argument order as the reference launchers.
+ * Replace entry_custom_gemmrc_128x128 / entry_custom_gemmrc_128x256
+ * (cuda/cute_kernels/main.cc:13-18, cute_gemm_128x128.cu:193-205, cute_gemm_128x256.cu:196-208);
+ * 256x128 is the third tile the configuration list names. */
+int beam_custom_gemmrc_128x128(const void* A, const void* B, void* C, int M, int N, int K, void* stream);
+int beam_custom_gemmrc_128x256(const void* A, const void* B, void* C, int M, int N, int K, void* stream);
+int beam_custom_gemmrc_256x128(const void* A, const void* B, void* C, int M, int N, int K, void* stream);
+
+/* ---- split-K ---------------------------------------------------------------------------- */
+
+/* Slices the library would choose for `tiles` output tiles on `compute_units` CUs: the rule of
+ * get_slice_heuristic (cuda/cutlass_kernels/cutlass_gemmrc_splitk.cu:44-57) with the device's
+ * CU count in place of the hard-coded 108. */
+int beam_slice_heuristic(int tiles, int compute_units);
+/* Bytes of fp32 workspace for `split_k` partial results (replaces the hidden grow-only
+ * buffer get_the_buffer, cutlass_gemmrc_splitk.cu:31-42: the caller owns the workspace). */
+size_t beam_splitk_workspace_bytes(int M, int N, int split_k);
+/* split_k <= 0: heuristic.  The effective factor is clamped to [1, ceil(K/64)].
+ * Slice s covers K elements [s*len, (s+1)*len), len = ceil(ceil(K/64)/split_k)*64; partial
+ * sums are fp32 in ws[split][M][N]; a second kernel adds them in slice order 0,1,2,... and
+ * rounds once, so results are bit-identical from run to run.
+ * Replaces entry_cutlass_gemmrc_splitk / _spec
+ * (cuda/cutlass_kernels/main.cc:17-21, cutlass_gemmrc_splitk.cu:59-105,107-195). */
+int beam_gemmrc_splitk(const void* A, const void* B, void* C, int M, int N, int K, int dtype,
+                       const beam_tile_cfg* cfg, int split_k, void* ws, size_t ws_bytes,
+                       void* stream);
+/* The effective split factor beam_gemmrc_splitk would use for these arguments. */
+int beam_splitk_effective(int M, int N, int K, const beam_tile_cfg* cfg, int split_k);
+
+/* ---- fused GEMM + LayerNorm --------------------------------------------------------------- */
+
+/* Y[m][:] = LayerNorm_N(A.B^T)[m][:] * gamma + beta, statistics (biased variance over N) and
+ * normalisation computed from the fp32 accumulators, Y rounded once to the 16-bit dtype.
+ * gamma, beta: 16-bit [N].  The reference has no LayerNorm (its
+ * entry_cute_parallel_gemmrc_lnr, cuda/cute_kernels/main.cc:19-22 and cute_gemm_ln.cu:230-245,
+ * is a GEMM plus an unrelated SiLU); this entry takes that slot in the interface. */
+size_t beam_gemmrc_ln_workspace_bytes(int M, int N, const beam_tile_cfg* cfg);
+int beam_gemmrc_ln(const void* A, const void* B, const void* gamma, const void* beta, float eps,
+                   void* Y, int M, int N, int K, int dtype, const beam_tile_cfg* cfg, void* ws,
+                   size_t ws_bytes, void* stream);
+
+/* ---- timing ------------------------------------------------------------------------------- */
+
+/* Which operation beam_bench times. */
+typedef enum beam_op { BEAM_OP_GEMM = 0, BEAM_OP_SPLITK = 1, BEAM_OP_GEMM_LN = 2 } beam_op;
+
+typedef struct beam_problem {
+  const void* A;
+  const void* B;
+  void* C;            /* C or Y                                                     */
+  const void* gamma;  /* BEAM_OP_GEMM_LN only                                       */
+  const void* beta;
+  float eps;
+  int M, N, K, dtype;
+  int split_k;        /* BEAM_OP_SPLITK                                             */
+  void* ws;
+  size_t ws_bytes;
+} beam_problem;
+
+/* `warmup` untimed calls, then `iters` back-to-back calls bracketed by HIP events on `stream`;
+ * *avg_ms = elapsed / iters.  Replaces test_pipeline (cuda/cublas.cc:12-40) and
+ * triton.testing.do_bench as used by python/beam/tuner.py:33-44. */
+int beam_bench(int op, const beam_problem* prob, const beam_tile_cfg* cfg, int warmup, int iters,
+               void* stream, float* avg_ms);
+
+/* Events for hosts that time their own call sequences (what triton.testing.do_bench gives the
+ * reference's tuner, python/beam/tuner.py:38-39).  elapsed waits for `stop` to complete. */
+int beam_event_create(void** event);
+int beam_event_record(void* event, void* stream);
+int beam_event_elapsed_ms(void* start, void* stop, float* ms);
+int beam_event_destroy(void* event);
+
+/* ---- device memory (so that hosts need no other GPU runtime) ------------------------------ */
+
+int beam_malloc(void** dptr, size_t bytes);
+int beam_free(void* dptr);
+int beam_memcpy_h2d(void* dst, const void* src_host, size_t bytes);
+int beam_memcpy_d2h(void* dst_host, const void* src, size_t bytes);
+int beam_memset(void* dptr, int byte, size_t bytes);
+int beam_sync(void* stream);
+
+/* ---- synthetic data (host) ----------------------------------------------------------------- */
+
+/* Counter-based generator: element i of tensor `tensor_id` under `seed` depends on nothing
+ * else, so any number of threads produce the same bits.  dst_host: 16-bit [n].
+ *   uniform: value in [-1, 1) with 24 random bits, rounded RN to the dtype
+ *   normal : mean + scale * N(0,1) (Box-Muller in double), rounded RN to the dtype
+ * The reference draws unseeded torch.randn on the GPU (python/gemm_test.py:81). */
+int beam_host_fill_uniform(void* dst_host, size_t n, int dtype, uint64_t seed, uint64_t tensor_id);
+int beam_host_fill_normal(void* dst_host, size_t n, int dtype, uint64_t seed, uint64_t tensor_id,
+                          float mean, float scale);
+
+/* ---- index maps, exported for host-side verification ---------------------------------------- */
+
+/* Workgroup id -> (tile_m, tile_n) as the kernels compute it. */
+int beam_dbg_tile_of_workgroup(int wg, int tiles_m, int tiles_n, int group_m, int* tm, int* tn);
+/* Byte offset of (row, 16-byte chunk) inside an LDS stage. */
+int beam_dbg_lds_offset(int row, int chunk);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* BEAM_HIP_H */

@@ -1,0 +1,180 @@
+"""Parity of the tiled gemmrc kernels (through the C ABI) with the CPU oracle.
+
+Bound for fp16: max|C_gpu - C_ref| <= 1e-2 * sqrt(K/1024) * RMS(C_ref), C_ref being the oracle's
+un-rounded fp32 result.  bf16 output carries a half-ulp of 2^-9 relative by itself (more than
+the bound at small K), so for bf16 the error in excess of |ref|/256 is held to the same bound.
+"""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+F16, BF16 = 0, 1
+
+
+def run_gemm(beamc, a_bits, b_bits, dtype, config=None, guard_rows=4):
+    M, K = a_bits.shape
+    N = b_bits.shape[0]
+    a = beamc.DeviceArray.from_numpy(a_bits, dtype)
+    b = beamc.DeviceArray.from_numpy(b_bits, dtype)
+    # Output with guard rows behind it: a kernel writing past C is caught, not just wrong.
+    full = beamc.DeviceArray((M + guard_rows, N), dtype)
+    full.fill_bytes(0xEE)
+    c = beamc.DeviceArray.__new__(beamc.DeviceArray)
+    c.shape, c.dtype, c.itemsize, c.nbytes, c.ptr = (M, N), dtype, 2, M * N * 2, full.ptr
+    try:
+        beamc.gemmrc(a, b, c, config=config)
+        out = full.to_numpy()
+    finally:
+        c.ptr = 0
+        for x in (a, b, full):
+            x.free()
+    assert (out[M:] == 0xEEEE).all(), "kernel wrote past the end of C"
+    return out[:M]
+
+
+def assert_close(oracle, got_bits, ref32, K, dtype, what=""):
+    r = oracle.compare(got_bits, ref32, dtype)
+    tol = oracle.gemm_tolerance(K) * r["rms_ref"]
+    err = r["max_abs_err"] if dtype == F16 else r["max_bf16_excess"]
+    assert err <= tol, f"{what}: max err {err:.4g} > {tol:.4g} (rms {r['rms_ref']:.4g})"
+    return r
+
+
+def all_configs(beamc):
+    out = []
+    for cfg in beamc.list_configs():
+        out.append(cfg)
+        out.append(beamc.TileConfig(cfg.block_m, cfg.block_n, cfg.wave_m, cfg.wave_n, 1, 0))
+    return out
+
+
+def test_1024_cube_every_config(gpu, beamc, oracle):
+    """fp16 1024^3, uniform[-1,1): every compiled tile, both loaders."""
+    M = N = K = 1024
+    a = beamc.host_uniform((M, K), F16, 1, 0)
+    b = beamc.host_uniform((N, K), F16, 1, 1)
+    ref = oracle.gemmrc(a, b, F16)
+    for cfg in all_configs(beamc):
+        got = run_gemm(beamc, a, b, F16, cfg)
+        assert_close(oracle, got, ref, K, F16, cfg.name)
+
+
+@pytest.mark.parametrize("shape", [(3, 5, 16), (1, 1, 8), (130, 70, 48), (257, 129, 1000), (64, 64, 64),
+                                   (300, 500, 200), (33, 1000, 72), (1000, 31, 136)])
+def test_ragged_small_every_config(gpu, beamc, oracle, shape):
+    M, N, K = shape
+    a = beamc.host_uniform((M, K), F16, 2, 0)
+    b = beamc.host_uniform((N, K), F16, 2, 1)
+    ref = oracle.gemmrc(a, b, F16)
+    naive = oracle.gemmrc_naive_f64(a, b, F16)
+    assert np.abs(ref - naive).max() <= 1e-5 * max(1.0, np.abs(naive).max())
+    for cfg in all_configs(beamc):
+        got = run_gemm(beamc, a, b, F16, cfg)
+        assert_close(oracle, got, ref, K, F16, f"{shape} {cfg.name}")
+
+
+def test_ragged_3000x5000x2000(gpu, beamc, oracle):
+    """Edge tiles in M and N and a short last K tile (K = 31*64 + 16), fp16 and bf16."""
+    M, N, K = 3000, 5000, 2000
+    for dtype in (F16, BF16):
+        a = beamc.host_uniform((M, K), dtype, 3, 0)
+        b = beamc.host_uniform((N, K), dtype, 3, 1)
+        ref = oracle.gemmrc(a, b, dtype)
+        for cfg in [None] + [c for c in beamc.list_configs() if (c.block_m, c.block_n) in ((256, 256), (128, 128), (256, 128))]:
+            got = run_gemm(beamc, a, b, dtype, cfg)
+            assert_close(oracle, got, ref, K, dtype, f"dtype {dtype} {cfg.name if cfg else 'default'}")
+
+
+def test_closed_forms(gpu, beamc, oracle):
+    """Identity, all-ones and one-hot operands have exact answers."""
+    n = 256
+    eye = np.eye(n, dtype=np.float16).view(np.uint16)
+    b = beamc.host_uniform((384, n), F16, 4, 1)
+    got = run_gemm(beamc, eye, b, F16)            # C = I . B^T = B^T exactly
+    assert (got == b.T).all()
+    K = 2048
+    ones_a = np.ones((100, K), np.float16).view(np.uint16)
+    ones_b = np.ones((36, K), np.float16).view(np.uint16)
+    got = run_gemm(beamc, ones_a, ones_b, F16)    # every element = K, exact in fp16
+    assert (got.view(np.float16) == np.float16(K)).all()
+    # one-hot rows of A pick single columns of B: C[m][n] = B[n][k_m]
+    K = 512
+    idx = (np.arange(200) * 37) % K
+    a = np.zeros((200, K), np.float16)
+    a[np.arange(200), idx] = 1
+    b = beamc.host_uniform((300, K), F16, 4, 2)
+    got = run_gemm(beamc, a.view(np.uint16), b, F16)
+    assert (got == b[:, idx].T).all()
+
+
+def test_bf16_sweep(gpu, beamc, oracle):
+    for (M, N, K) in [(512, 512, 512), (1024, 1024, 1024), (2048, 2048, 2048)]:
+        a = beamc.host_uniform((M, K), BF16, 5, 0)
+        b = beamc.host_uniform((N, K), BF16, 5, 1)
+        ref = oracle.gemmrc(a, b, BF16)
+        for cfg in [None, beamc.TileConfig(128, 128, 64, 64), beamc.TileConfig(64, 64, 32, 32)]:
+            got = run_gemm(beamc, a, b, BF16, cfg)
+            assert_close(oracle, got, ref, K, BF16, f"{(M, N, K)}")
+
+
+@pytest.mark.parametrize("shape", [(512, 512, 512), (2048, 2048, 2048), (4096, 4096, 4096),
+                                   (4096, 11008, 4096), (4096, 4096, 11008)])
+def test_fp16_sweep(gpu, beamc, oracle, shape):
+    M, N, K = shape
+    a = beamc.host_uniform((M, K), F16, 6, 0)
+    b = beamc.host_uniform((N, K), F16, 6, 1)
+    ref = oracle.gemmrc(a, b, F16)
+    got = run_gemm(beamc, a, b, F16)
+    assert_close(oracle, got, ref, K, F16, f"{shape}")
+
+
+def test_headline_8192_cube(gpu, beamc, oracle):
+    """fp16 8192^3, N(0,1)/sqrt(K): default tile and the three named tiles, full oracle."""
+    M = N = K = 8192
+    a = beamc.host_normal((M, K), F16, 7, 0, 0.0, K ** -0.5)
+    b = beamc.host_normal((N, K), F16, 7, 1, 0.0, K ** -0.5)
+    ref = oracle.gemmrc(a, b, F16)
+    rms = float(np.sqrt(np.mean(ref.astype(np.float64) ** 2)))
+    assert abs(rms * K ** 0.5 - 1.0) < 0.05          # RMS(C) = 1/sqrt(K) for these inputs
+    for cfg in [None, beamc.TileConfig(128, 128, 64, 64), beamc.TileConfig(128, 256, 64, 64),
+                beamc.TileConfig(256, 128, 64, 64)]:
+        got = run_gemm(beamc, a, b, F16, cfg)
+        assert_close(oracle, got, ref, K, F16, cfg.name if cfg else "default")
+
+
+def test_fixed_tile_entry_points(gpu, beamc, oracle):
+    """The three reference-named launchers (fp16 only)."""
+    M, N, K = 512, 768, 1024
+    a_bits = beamc.host_uniform((M, K), F16, 8, 0)
+    b_bits = beamc.host_uniform((N, K), F16, 8, 1)
+    ref = oracle.gemmrc(a_bits, b_bits, F16)
+    a = beamc.DeviceArray.from_numpy(a_bits)
+    b = beamc.DeviceArray.from_numpy(b_bits)
+    c = beamc.DeviceArray((M, N))
+    for fn in (beamc.custom_gemmrc_128x128, beamc.custom_gemmrc_128x256, beamc.custom_gemmrc_256x128):
+        c.fill_bytes(0)
+        fn(a=a, b=b, c=c)
+        assert_close(oracle, c.to_numpy(), ref, K, F16, fn.__name__)
+
+
+def test_error_codes(gpu, beamc):
+    a = beamc.DeviceArray((64, 64))
+    b = beamc.DeviceArray((64, 64))
+    c = beamc.DeviceArray((64, 64))
+    with pytest.raises(beamc.BeamError) as e:
+        beamc.gemmrc_spec(a, b, c, shape_threadblock=[96, 96], shape_warp=[48, 48])
+    assert e.value.status == 2
+    with pytest.raises(beamc.BeamError) as e:
+        beamc.gemmrc(a, b, beamc.DeviceArray((64, 32)))
+    assert e.value.status == 1
+    a2 = beamc.DeviceArray((64, 12))
+    b2 = beamc.DeviceArray((64, 12))
+    with pytest.raises(beamc.BeamError) as e:
+        beamc.gemmrc(a2, b2, c)
+    assert e.value.status == 2      # K % 8 != 0 has no kernel: reported, never silent
+    # empty problems are no-ops, K == 0 clears C
+    beamc.gemmrc(beamc.DeviceArray((0, 64)), b, beamc.DeviceArray((0, 64)))
+    c.fill_bytes(0x55)
+    beamc.gemmrc(beamc.DeviceArray((64, 0)), beamc.DeviceArray((64, 0)), c)
+    assert (c.to_numpy() == 0).all()
