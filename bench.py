@@ -1,0 +1,171 @@
+#!/usr/bin/env python3
+"""Headline benchmark: fp16 gemmrc 8192^3 on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-extra]
+
+A step is one gemmrc launch (C = A . B^T, fp32 accumulation, fp16 output) on inputs already
+resident in HBM (N(0,1)/sqrt(K) values from the seeded host generator).  One JSON line is
+printed: whole-job TFLOP/s, the MFMA roofline fraction of the kernel measured with HIP events on
+the launch stream, and the CPU oracle timed on this host's cores beside it (a reported baseline,
+also used to check the GPU result of the timed run).  `extra` carries the two companion targets:
+split-K at 256x256x32768 (us, against the best non-split tile) and fused GEMM+LayerNorm at 4096^3
+(against the plain GEMM).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, "general-nvgpu-testing_amd"))
+
+METRIC = "fp16 GEMM TFLOP/s + % MFMA peak at 8192^3; split-K µs at 256x256x32768"
+# MI355X dense fp16 matrix-core peak: 256 CUs x 4 SIMDs x 1024 FLOP/clk x 2.4 GHz = 2516.6 TFLOP/s,
+# published as 2.5 PFLOP/s.
+PEAK_TFLOPS = 2500.0
+HBM_PEAK_GBS = 8000.0
+
+
+def time_region(_C, fn, steps):
+    """(wall seconds, HIP-event milliseconds) for `steps` calls of fn on the default stream."""
+    import ctypes
+    e0, e1 = ctypes.c_void_p(), ctypes.c_void_p()
+    _C._check(_C.lib.beam_event_create(ctypes.byref(e0)))
+    _C._check(_C.lib.beam_event_create(ctypes.byref(e1)))
+    _C.sync()
+    t0 = time.perf_counter()
+    _C._check(_C.lib.beam_event_record(e0, None))
+    for _ in range(steps):
+        fn()
+    _C._check(_C.lib.beam_event_record(e1, None))
+    ms = ctypes.c_float()
+    _C._check(_C.lib.beam_event_elapsed_ms(e0, e1, ctypes.byref(ms)))
+    _C.sync()
+    wall = time.perf_counter() - t0
+    _C.lib.beam_event_destroy(e0)
+    _C.lib.beam_event_destroy(e1)
+    return wall, ms.value
+
+
+def cpu_baseline(a_bits, b_bits, M, N, K):
+    """The oracle (test infrastructure) timed once on the full workload; returns the baseline
+    record and the fp32 result for checking the GPU output."""
+    sys.path.insert(0, os.path.join(ROOT, "oracle"))
+    import oracle as O
+    O.lib()
+    t0 = time.perf_counter()
+    ref = O.gemmrc(a_bits, b_bits, O.F16)
+    dt = time.perf_counter() - t0
+    rec = {"value": round(2.0 * M * N * K / dt / 1e12, 4), "unit": "TFLOP/s", "cores": O.num_threads(),
+           "kind": "port", "sample": f"full {M}x{N}x{K} fp16 gemmrc once, {dt:.2f} s (fp32 FMA, OpenMP, AVX2)"}
+    return rec, ref, O
+
+
+def extra_splitk(_C):
+    """split-K at 256x256x32768: best (tile, S) against the best non-split tile."""
+    M, N, K = 256, 256, 32768
+    a = _C.DeviceArray.from_numpy(_C.host_uniform((M, K), _C.F16, 11, 0))
+    b = _C.DeviceArray.from_numpy(_C.host_uniform((N, K), _C.F16, 11, 1))
+    c = _C.DeviceArray((M, N))
+    best_plain, best_split = (None, 1e30), (None, 1e30)
+    for cfg in _C.list_configs():
+        ms = _C.bench(0, a, b, c, config=cfg, warmup=3, iters=20)
+        if ms < best_plain[1]:
+            best_plain = (cfg.name, ms)
+        if cfg.block_m * cfg.block_n > 128 * 128:
+            continue
+        for s in (4, 8, 16, 32, 64):
+            ms = _C.bench(1, a, b, c, config=cfg, split_k=s, warmup=3, iters=20)
+            if ms < best_split[1]:
+                best_split = (f"{cfg.name},S={s}", ms)
+    for x in (a, b, c):
+        x.free()
+    bytes_alg = 2.0 * (M * K + N * K + M * N)
+    return {"shape": [M, N, K], "splitk_us": round(best_split[1] * 1e3, 2), "splitk_config": best_split[0],
+            "best_nonsplit_us": round(best_plain[1] * 1e3, 2), "best_nonsplit_config": best_plain[0],
+            "speedup": round(best_plain[1] / best_split[1], 2),
+            "hbm_GBs": round(bytes_alg / (best_split[1] * 1e-3) / 1e9, 1),
+            "hbm_frac": round(bytes_alg / (best_split[1] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+
+
+def extra_ln(_C):
+    """fused GEMM+LayerNorm at 4096^3 against the plain GEMM of the same tile."""
+    M = N = K = 4096
+    a = _C.DeviceArray.from_numpy(_C.host_normal((M, K), _C.F16, 22, 0, 0.0, K ** -0.5))
+    b = _C.DeviceArray.from_numpy(_C.host_normal((N, K), _C.F16, 22, 1, 0.0, K ** -0.5))
+    g = _C.DeviceArray.from_numpy(_C.host_normal((N,), _C.F16, 22, 2, 1.0, 0.1))
+    bt = _C.DeviceArray.from_numpy(_C.host_normal((N,), _C.F16, 22, 3, 0.0, 0.1))
+    c = _C.DeviceArray((M, N))
+    plain = _C.bench(0, a, b, c, warmup=5, iters=20)
+    fused = _C.bench(2, a, b, c, gamma=g, beta=bt, warmup=5, iters=20)
+    for x in (a, b, g, bt, c):
+        x.free()
+    return {"shape": [M, N, K], "gemm_us": round(plain * 1e3, 1), "gemm_ln_us": round(fused * 1e3, 1),
+            "overhead": round(fused / plain - 1.0, 4),
+            "gemm_ln_TFLOPs": round(2.0 * M * N * K / (fused * 1e-3) / 1e12, 1)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline and the result check")
+    ap.add_argument("--no-extra", action="store_true", help="skip the split-K and GEMM+LN companions")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on ONE GPU (the gemmrc path needs no exchange between GPUs; "
+                 "see DESIGN.md for how it would shard). Re-run with --gpus 1.")
+
+    from beam import _C  # fails loudly if libbeam_hip.so is missing; there is no fallback
+
+    info = _C.device_info()
+    M = N = K = 8192
+    a_bits = _C.host_normal((M, K), _C.F16, 7, 0, 0.0, K ** -0.5)
+    b_bits = _C.host_normal((N, K), _C.F16, 7, 1, 0.0, K ** -0.5)
+    a, b = _C.DeviceArray.from_numpy(a_bits), _C.DeviceArray.from_numpy(b_bits)
+    c = _C.DeviceArray((M, N))
+    c.fill_bytes(0xEE)
+    cfg, _ = _C.default_config(M, N, K)
+
+    def step():
+        _C.gemmrc(a, b, c)
+
+    for _ in range(args.warmup):
+        step()
+    wall, ev_ms = time_region(_C, step, args.steps)
+    flops = 2.0 * M * N * K
+    value = flops * args.steps / wall / 1e12
+    kern_ms = ev_ms / args.steps
+    achieved = flops / (kern_ms * 1e-3) / 1e12
+
+    out = {
+        "metric": METRIC, "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(wall / args.steps * 1e3, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+        "config": {"workload": "fp16 gemmrc M=N=K=8192, A,B ~ N(0,1)/sqrt(K) seed 7, fp32 accumulate, fp16 C",
+                   "tile": cfg.name, "device": info["name"], "compute_units": info["compute_units"]},
+        "pct_of_peak": round(100.0 * value / PEAK_TFLOPS, 2),
+        "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(achieved / PEAK_TFLOPS, 4), "traffic": None,
+                     "kernel_ms": round(kern_ms, 4)},
+    }
+    if not args.no_cpu:
+        rec, ref, O = cpu_baseline(a_bits, b_bits, M, N, K)
+        r = O.compare(c.to_numpy(), ref, O.F16)
+        tol = O.gemm_tolerance(K) * r["rms_ref"]
+        out["cpu_baseline"] = rec
+        out["check"] = {"max_abs_err": r["max_abs_err"], "bound": tol, "ok": bool(r["max_abs_err"] <= tol)}
+        del ref
+    for x in (a, b, c):
+        x.free()
+    if not args.no_extra:
+        out["extra"] = {"splitk": extra_splitk(_C), "gemm_ln": extra_ln(_C)}
+    print(json.dumps(out))
+    if "check" in out and not out["check"]["ok"]:
+        sys.exit("bench.py: GPU result outside the tolerance of the CPU oracle")
+
+
+if __name__ == "__main__":
+    main()

@@ -36,7 +36,7 @@ class BeamError(RuntimeError):
 
 class _TileCfg(ctypes.Structure):
     _fields_ = [("block_m", ctypes.c_int), ("block_n", ctypes.c_int), ("wave_m", ctypes.c_int),
-                ("wave_n", ctypes.c_int), ("loader", ctypes.c_int), ("group_m", ctypes.c_int)]
+                ("wave_n", ctypes.c_int), ("pipeline", ctypes.c_int), ("group_m", ctypes.c_int)]
 
 
 class _Problem(ctypes.Structure):
@@ -106,22 +106,22 @@ def _check(status: int) -> None:
 
 @dataclass(frozen=True)
 class TileConfig:
-    """One point of the tunable space: workgroup tile, wavefront tile, loader, raster group."""
+    """One point of the tunable space: workgroup tile, wavefront tile, pipeline depth, raster group."""
     block_m: int
     block_n: int
     wave_m: int
     wave_n: int
-    loader: int = 0
+    pipeline: int = 0
     group_m: int = 0
 
     def to_c(self) -> _TileCfg:
-        return _TileCfg(self.block_m, self.block_n, self.wave_m, self.wave_n, self.loader, self.group_m)
+        return _TileCfg(self.block_m, self.block_n, self.wave_m, self.wave_n, self.pipeline, self.group_m)
 
     @property
     def name(self) -> str:
         s = f"{self.block_m}x{self.block_n}_w{self.wave_m}x{self.wave_n}"
-        if self.loader:
-            s += "_staged"
+        if self.pipeline:
+            s += "_p22"
         if self.group_m:
             s += f"_g{self.group_m}"
         return s
@@ -132,7 +132,7 @@ def list_configs() -> List[TileConfig]:
     for idx in range(lib.beam_num_configs()):
         c = _TileCfg()
         _check(lib.beam_get_config(idx, ctypes.byref(c)))
-        out.append(TileConfig(c.block_m, c.block_n, c.wave_m, c.wave_n, c.loader, 0))
+        out.append(TileConfig(c.block_m, c.block_n, c.wave_m, c.wave_n, c.pipeline, 0))
     return out
 
 
@@ -140,7 +140,7 @@ def default_config(M: int, N: int, K: int):
     c = _TileCfg()
     s = ctypes.c_int(1)
     _check(lib.beam_default_config(M, N, K, ctypes.byref(c), ctypes.byref(s)))
-    return TileConfig(c.block_m, c.block_n, c.wave_m, c.wave_n, c.loader, c.group_m), s.value
+    return TileConfig(c.block_m, c.block_n, c.wave_m, c.wave_n, c.pipeline, c.group_m), s.value
 
 
 def device_info() -> dict:
@@ -241,13 +241,13 @@ def _problem(a, b, c):
     return pa, pb, pc, M, N, K, da, st
 
 
-def _cfg_from_shapes(shape_threadblock, shape_warp, loader=0, group_m=0) -> _TileCfg:
+def _cfg_from_shapes(shape_threadblock, shape_warp, pipeline=0, group_m=0) -> _TileCfg:
     # An empty list means "default", as in cuda/cutlass_kernels/cutlass_gemmrc.cu:73-81.
     tb = list(shape_threadblock) if shape_threadblock else [128, 128]
     wp = list(shape_warp) if shape_warp else [64, 64]
     if len(tb) != 2 or len(wp) != 2:
         raise BeamError(1, "shape_threadblock and shape_warp must have two entries")
-    return _TileCfg(tb[0], tb[1], wp[0], wp[1], loader, group_m)
+    return _TileCfg(tb[0], tb[1], wp[0], wp[1], pipeline, group_m)
 
 
 # ---------------------------------------------------------------------------- workspaces
@@ -277,12 +277,12 @@ def gemmrc(a, b, c, config: Optional[TileConfig] = None) -> None:
     _check(lib.beam_gemmrc(pa, pb, pc, M, N, K, d, cfg, st))
 
 
-def gemmrc_spec(a, b, c, shape_threadblock=(128, 128), shape_warp=(64, 64), loader: int = 0,
+def gemmrc_spec(a, b, c, shape_threadblock=(128, 128), shape_warp=(64, 64), pipeline: int = 0,
                 group_m: int = 0) -> None:
     """c = a @ b.T with an explicit workgroup tile / wavefront tile
     (reference: cutlass_gemmrc_spec, python/beam/_C/beam_C.pyi:16)."""
     pa, pb, pc, M, N, K, d, st = _problem(a, b, c)
-    cfg = _cfg_from_shapes(shape_threadblock, shape_warp, loader, group_m)
+    cfg = _cfg_from_shapes(shape_threadblock, shape_warp, pipeline, group_m)
     _check(lib.beam_gemmrc(pa, pb, pc, M, N, K, d, ctypes.byref(cfg), st))
 
 
@@ -294,10 +294,10 @@ def gemmrc_splitk(a, b, c, split_k_slices: int = 0) -> None:
 
 
 def gemmrc_splitk_spec(a, b, c, shape_threadblock=(128, 128), shape_warp=(64, 64), split_k_slices: int = 0,
-                       loader: int = 0, group_m: int = 0) -> None:
+                       pipeline: int = 0, group_m: int = 0) -> None:
     """Split-K with explicit tiles (reference: cutlass_gemmrc_splitk_spec, beam_C.pyi:20)."""
     pa, pb, pc, M, N, K, d, st = _problem(a, b, c)
-    cfg = _cfg_from_shapes(shape_threadblock, shape_warp, loader, group_m)
+    cfg = _cfg_from_shapes(shape_threadblock, shape_warp, pipeline, group_m)
     s = lib.beam_splitk_effective(M, N, K, ctypes.byref(cfg), split_k_slices)
     if s < 0:
         raise BeamError(2, lib.beam_last_error().decode())

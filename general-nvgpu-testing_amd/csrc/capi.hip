@@ -91,7 +91,7 @@ int resolve_cfg(const beam_tile_cfg* in, int M, int N, int K, beam_tile_cfg* out
     int rc = beam_default_config(M, N, K, out, &s);
     if (rc) return rc;
   }
-  if (out->loader != 0 && out->loader != 1) return fail(BEAM_ERR_UNSUPPORTED, "loader %d: 0 (direct to LDS) or 1 (register staged)", out->loader);
+  if (out->pipeline != 0 && out->pipeline != 1) return fail(BEAM_ERR_UNSUPPORTED, "pipeline %d: 0 (3 A + 2 B LDS slots) or 1 (2 + 2)", out->pipeline);
   if (out->group_m <= 0) out->group_m = kDefaultGroupM;
   *ks = find_set(*out);
   if (!*ks)
@@ -229,7 +229,7 @@ int beam_get_config(int index, beam_tile_cfg* out) {
   out->block_n = k.block_n;
   out->wave_m = k.wave_m;
   out->wave_n = k.wave_n;
-  out->loader = 0;
+  out->pipeline = 0;
   out->group_m = kDefaultGroupM;
   return BEAM_OK;
 }
@@ -298,7 +298,7 @@ int beam_gemmrc(const void* A, const void* B, void* C, int M, int N, int K, int 
   if ((rc = resolve_cfg(cfg, M, N, K, &c, &ks))) return rc;
   GemmParams p = base_params(A, B, M, N, K, c);
   p.C = C;
-  BEAM_HIP(ks->launch[dtype][kEpiStore][c.loader](p, dim3((unsigned)(p.tiles_m * p.tiles_n), 1, 1), st));
+  BEAM_HIP(ks->launch[dtype][kEpiStore][c.pipeline](p, dim3((unsigned)(p.tiles_m * p.tiles_n), 1, 1), st));
   return BEAM_OK;
 }
 
@@ -364,7 +364,7 @@ int beam_gemmrc_splitk(const void* A, const void* B, void* C, int M, int N, int 
   if (s == 1) {  // nothing to reduce: the plain kernel writes C directly
     GemmParams p = base_params(A, B, M, N, K, c);
     p.C = C;
-    BEAM_HIP(ks->launch[dtype][kEpiStore][c.loader](p, dim3((unsigned)(p.tiles_m * p.tiles_n), 1, 1), st));
+    BEAM_HIP(ks->launch[dtype][kEpiStore][c.pipeline](p, dim3((unsigned)(p.tiles_m * p.tiles_n), 1, 1), st));
     return BEAM_OK;
   }
   const size_t need = beam_splitk_workspace_bytes(M, N, s);
@@ -374,7 +374,7 @@ int beam_gemmrc_splitk(const void* A, const void* B, void* C, int M, int N, int 
   GemmParams p = base_params(A, B, M, N, K, c);
   p.ws = (float*)ws;
   p.k_slice = split_k_len(K, s);
-  BEAM_HIP(ks->launch[dtype][kEpiPartial][c.loader](p, dim3((unsigned)(p.tiles_m * p.tiles_n), 1, (unsigned)s), st));
+  BEAM_HIP(ks->launch[dtype][kEpiPartial][c.pipeline](p, dim3((unsigned)(p.tiles_m * p.tiles_n), 1, (unsigned)s), st));
   BEAM_HIP(launch_splitk_reduce((const float*)ws, C, (size_t)M * N, s, dtype, st));
   return BEAM_OK;
 }
@@ -410,7 +410,7 @@ int beam_gemmrc_ln(const void* A, const void* B, const void* gamma, const void* 
   p.ws = (float*)ws;
   p.stats = (float*)((char*)ws + align_up((size_t)M * N * sizeof(float), 256));
   // K == 0: the kernel runs with an empty K range and produces x = 0, i.e. y = beta.
-  BEAM_HIP(ks->launch[dtype][kEpiLnStats][c.loader](p, dim3((unsigned)(p.tiles_m * p.tiles_n), 1, 1), st));
+  BEAM_HIP(ks->launch[dtype][kEpiLnStats][c.pipeline](p, dim3((unsigned)(p.tiles_m * p.tiles_n), 1, 1), st));
   BEAM_HIP(launch_ln_apply(p.ws, p.stats, gamma, beta, Y, M, N, p.tiles_n, c.block_n, eps, dtype, st));
   return BEAM_OK;
 }

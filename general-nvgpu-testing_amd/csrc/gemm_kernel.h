@@ -8,29 +8,36 @@
 // cute_gemm_128x256.cu:17-194; layouts cuda/cute_kernels/main.cc:29-40; fp32 accumulate
 // :90; round-to-nearest output :183) rebuilt for 64-wide wavefronts:
 //
-//   * one workgroup owns a BM x BN tile of C, WAVES_M x WAVES_N wavefronts each own a
-//     (BM/WAVES_M) x (BN/WAVES_N) sub-tile made of 32x32 MFMA blocks
-//     (v_mfma_f32_32x32x16_{f16,bf16}: 16 K elements per instruction);
-//   * K is walked in steps of 64 elements; a stage of LDS holds BM + BN rows of 128 bytes,
-//     16-byte chunks XOR-swizzled (tile_map.h) so that both the 1 KiB-per-wavefront fills
-//     and the ds_read_b128 fragment reads are bank-conflict free;
+//   * one workgroup owns a BM x BN tile of C; WAVES_M x WAVES_N wavefronts each own a
+//     (BM/WAVES_M) x (BN/WAVES_N) sub-tile made of 16x16 MFMA blocks
+//     (v_mfma_f32_16x16x32_{f16,bf16}: 32 K elements per instruction -- on random data it
+//     draws measurably less power per flop than the 32x32x16 shape, and this part is power
+//     limited long before it is issue limited);
+//   * K is walked in tiles of 64 elements; an LDS slot holds one operand tile as rows of 128
+//     bytes whose 16-byte chunks are XOR-swizzled (tile_map.h): the 1 KiB-per-wavefront fills
+//     and the ds_read_b128 fragment reads are both bank-conflict free;
 //   * global -> LDS goes through buffer loads that write LDS directly (no VGPR staging);
 //     rows past the matrix edge are outside the buffer descriptor and never touch memory;
-//   * two LDS stages: the fill of stage s^1 is in flight while stage s feeds the MFMAs, and
-//     fragments are double-buffered in registers so LDS latency hides behind MFMA issue;
+//   * A has AST slots and B has BST slots (3 + 2 for the 256x256 tile = all 160 KiB of LDS).
+//     While tile h feeds the MFMAs, B tile h+BST-1 and A tile h+AST-1 are in flight, their
+//     loads issued one at a time between rows of MFMAs so the vector-memory path (64 B/clk)
+//     never sees a burst; one s_barrier per K tile;
+//   * fragments are software pipelined one 32-wide step ahead: A in place (a row's next
+//     fragment is fetched right after its last use), B double buffered;
 //   * the MFMA is issued with B as the first operand, so every lane ends up with 4
-//     consecutive columns of one output row per accumulator quad: rows reduce inside a
-//     lane (LayerNorm statistics) and stores are 8-byte (16-bit C) or 16-byte (fp32).
+//     consecutive columns of one output row per block: stores are 8 bytes (16-bit C) or 16
+//     bytes (fp32), and a row's statistics reduce over registers plus two lane swaps.
 #pragma once
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 #include "tile_map.h"
 
 namespace beam {
 
-typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
@@ -45,8 +52,8 @@ template <>
 struct ElemTraits<_Float16> {
   using vec8 = f16x8;
   using vec4 = f16x4;
-  static __device__ __forceinline__ f32x16 mfma(vec8 a, vec8 b, f32x16 c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  static __device__ __forceinline__ f32x4 mfma(vec8 a, vec8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
   }
 };
 
@@ -54,8 +61,8 @@ template <>
 struct ElemTraits<__bf16> {
   using vec8 = bf16x8;
   using vec4 = bf16x4;
-  static __device__ __forceinline__ f32x16 mfma(vec8 a, vec8 b, f32x16 c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  static __device__ __forceinline__ f32x4 mfma(vec8 a, vec8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
   }
 };
 
@@ -87,7 +94,24 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, un
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, kRsrcFlags);
 }
 
-template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, int EPI, bool DIRECT>
+// s_waitcnt vmcnt(N) lgkmcnt(0): at most N of this wavefront's buffer loads still in flight,
+// all of its LDS reads returned.
+template <int N>
+__device__ __forceinline__ void wait_vm_and_lds() {
+  static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+  __builtin_amdgcn_s_waitcnt(0x0070 | (N & 15) | ((N >> 4) << 14));
+}
+
+// Workgroup barrier without the memory fence of __syncthreads(): the fence would wait for
+// every outstanding LDS fill (vmcnt(0)) and serialise the pipeline.  The waits the data
+// hazards need are issued explicitly by the caller.
+__device__ __forceinline__ void bare_barrier() {
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+}
+
+template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, int EPI, int AST, int BST>
 struct GemmTile {
   using Traits = ElemTraits<T>;
   using vec8 = typename Traits::vec8;
@@ -97,24 +121,31 @@ struct GemmTile {
   static constexpr int NT = NW * 64;
   static constexpr int TM = BM / WAVES_M;  // wavefront tile
   static constexpr int TN = BN / WAVES_N;
-  static constexpr int FM = TM / 32;       // MFMA blocks per wavefront tile
-  static constexpr int FN = TN / 32;
+  static constexpr int FM = TM / 16;       // MFMA blocks per wavefront tile
+  static constexpr int FN = TN / 16;
+  static constexpr int KSTEPS = kBK / 32;  // MFMA K steps per tile (= 2)
   static constexpr int A_BYTES = BM * kRowBytes;
   static constexpr int B_BYTES = BN * kRowBytes;
-  static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
-  static constexpr int LDS_BYTES = 2 * STAGE_BYTES;
-  static constexpr int LA = (BM * kChunksPerRow) / NT;  // 16-byte chunks per thread per stage
+  static constexpr int B_REGION = AST * A_BYTES;  // A slots first, then B slots
+  static constexpr int LDS_BYTES = AST * A_BYTES + BST * B_BYTES;
+  static constexpr int LA = (BM * kChunksPerRow) / NT;  // buffer loads per wavefront per A tile
   static constexpr int LB = (BN * kChunksPerRow) / NT;
+  static constexpr int LOADS = LA + LB;
+  static constexpr int ROWS = KSTEPS * FM;                 // rows of MFMAs per K tile
+  static constexpr int PER_ROW = (LOADS + ROWS - 1) / ROWS;  // buffer loads issued after each row
+  // Loads that may still be in flight when tile h is needed: the A tiles and B tiles beyond h.
+  static constexpr int WAIT_STEADY = (AST - 2) * LA + (BST - 2) * LB;
 
-  static_assert(TM % 32 == 0 && TN % 32 == 0, "wavefront tile must be made of 32x32 blocks");
+  static_assert(KSTEPS == 2, "the step pipeline below is written for two 32-wide steps per tile");
+  static_assert(TM % 16 == 0 && TN % 16 == 0, "wavefront tile must be made of 16x16 blocks");
   static_assert((BM * kChunksPerRow) % NT == 0 && (BN * kChunksPerRow) % NT == 0,
-                "every thread must move a whole number of chunks per stage");
+                "every wavefront must move a whole number of 1 KiB chunks per tile");
+  static_assert(AST >= 2 && BST >= 2 && (AST == BST || AST == BST + 1), "slot counts");
   static_assert(LDS_BYTES <= 160 * 1024, "LDS budget of one CU");
+  static_assert(WAIT_STEADY < 64, "vmcnt range");
 
-  // ---- global -> LDS ------------------------------------------------------------------
-  // Chunk q = i * NT + tid of an operand tile lives at LDS byte q * 16 of its stage, which is
-  // row q / 8, slot q % 8; the slot holds logical chunk slot ^ swizzle_of_row(row).
-
+  // Chunk q = i * NT + tid of an operand tile lives at LDS byte q * 16 of its slot, which is
+  // row q / 8, position q % 8; the position holds logical chunk position ^ swizzle_of_row(row).
   static __device__ __forceinline__ unsigned chunk_voffset(int q, int K) {
     const int row = q >> 3;
     const int chunk = (q & 7) ^ swizzle_of_row(row);
@@ -140,7 +171,7 @@ struct GemmTile {
     if (klen < 0) klen = 0;
     const int kt_full = klen / kBK;
     const int k_tail = klen - kt_full * kBK;         // multiple of 8 (host guarantees K % 8 == 0)
-    const int n_tiles = kt_full + (k_tail ? 1 : 0);  // the short tile, if any, is processed FIRST
+    const int n_tiles = kt_full + (k_tail ? 1 : 0);  // the short tile, if any, is tile 0
 
     // Buffer descriptors cover exactly the rows of this tile that exist and the K range of
     // this slice; anything else is out of range: reads return zero and touch no memory.
@@ -159,25 +190,24 @@ struct GemmTile {
 #pragma unroll
     for (int i = 0; i < LB; ++i) voff_b[i] = chunk_voffset(i * NT + tid, K);
 
-    // Fill of one stage straight into LDS; `koff` = first K element of the tile inside the slice.
-    auto fill_direct = [&](int stage, int koff) {
-      char* sa = smem + stage * STAGE_BYTES + wave * 1024;
-      char* sb = sa + A_BYTES;
-#pragma unroll
-      for (int i = 0; i < LA; ++i)
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(
-            rsrc_a, (__attribute__((address_space(3))) void*)(sa + i * (NT * 16)), 16,
-            (int)voff_a[i], koff * 2, 0, 0);
-#pragma unroll
-      for (int i = 0; i < LB; ++i)
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(
-            rsrc_b, (__attribute__((address_space(3))) void*)(sb + i * (NT * 16)), 16,
-            (int)voff_b[i], koff * 2, 0, 0);
-    };
+    // First K element (inside the slice) of tile t: the short tile comes first.
+    auto tile_koff = [&](int t) { return k_tail ? (t == 0 ? kt_full * kBK : (t - 1) * kBK) : t * kBK; };
 
-    // Fill of one stage through registers, zero-filling chunks at or past `kvalid` elements
-    // (used for the short K tile and by the DIRECT=false variant).
-    auto fill_staged = [&](int stage, int koff, int kvalid) {
+    // ---- global -> LDS ------------------------------------------------------------------
+    // One buffer load (1 KiB per wavefront) of A tile t / B tile t into its slot.
+    auto load_a = [&](int i, int t) {
+      char* dst = smem + (t % AST) * A_BYTES + wave * 1024 + i * (NT * 16);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (__attribute__((address_space(3))) void*)dst, 16,
+                                               (int)voff_a[i], tile_koff(t) * 2, 0, 0);
+    };
+    auto load_b = [&](int i, int t) {
+      char* dst = smem + B_REGION + (t % BST) * B_BYTES + wave * 1024 + i * (NT * 16);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, (__attribute__((address_space(3))) void*)dst, 16,
+                                               (int)voff_b[i], tile_koff(t) * 2, 0, 0);
+    };
+    // The short tile goes through registers so that chunks at or past `kvalid` are zero-filled.
+    auto fill_short_tile = [&](int kvalid) {
+      const int koff = tile_koff(0);
       i32x4 ra[LA], rb[LB];
 #pragma unroll
       for (int i = 0; i < LA; ++i) {
@@ -193,8 +223,8 @@ struct GemmTile {
         const unsigned off = (chunk * 8 < kvalid) ? voff_b[i] + (unsigned)koff * 2u : kOobOffset;
         rb[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, (int)off, 0, 0);
       }
-      char* sa = smem + stage * STAGE_BYTES + tid * 16;
-      char* sb = sa + A_BYTES;
+      char* sa = smem + tid * 16;
+      char* sb = smem + B_REGION + tid * 16;
 #pragma unroll
       for (int i = 0; i < LA; ++i) *(i32x4*)(sa + i * (NT * 16)) = ra[i];
 #pragma unroll
@@ -202,239 +232,229 @@ struct GemmTile {
     };
 
     // ---- LDS -> MFMA fragments ----------------------------------------------------------
-    // 32x32x16 operand: lane l supplies row (l & 31), K elements 8*(l>>5) .. +7 of the step.
-    const int frow = lane & 31;
-    int frag_off[4];
+    // 16x16x32 operand: lane l supplies row (l & 15), K elements 8*(l>>4) .. +7 of the step.
+    int frag_off[KSTEPS];
 #pragma unroll
-    for (int kk = 0; kk < 4; ++kk) frag_off[kk] = lds_offset(frow, 2 * kk + (lane >> 5));
+    for (int kk = 0; kk < KSTEPS; ++kk) frag_off[kk] = lds_offset(lane & 15, 4 * kk + (lane >> 4));
     const int a_wave_off = wm * TM * kRowBytes;
-    const int b_wave_off = A_BYTES + wn * TN * kRowBytes;
+    const int b_wave_off = wn * TN * kRowBytes;
 
-    auto read_frags = [&](int stage, int kk, vec8 (&fa)[FM], vec8 (&fb)[FN]) {
-      const char* s = smem + stage * STAGE_BYTES + frag_off[kk];
-#pragma unroll
-      for (int i = 0; i < FM; ++i) fa[i] = *(const vec8*)(s + a_wave_off + i * 32 * kRowBytes);
-#pragma unroll
-      for (int j = 0; j < FN; ++j) fb[j] = *(const vec8*)(s + b_wave_off + j * 32 * kRowBytes);
-    };
-
-    f32x16 acc[FM][FN];
+    f32x4 acc[FM][FN];
 #pragma unroll
     for (int i = 0; i < FM; ++i)
 #pragma unroll
       for (int j = 0; j < FN; ++j)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+        for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.0f;
 
-    auto mma = [&](const vec8 (&fa)[FM], const vec8 (&fb)[FN]) {
+    // Fragments of the step being multiplied: A rows in fa, B rows in fb0 or fb1.  They start
+    // as zeros so that the very first step of the pipeline multiplies nothing.
+    vec8 fa[FM], fb0[FN], fb1[FN];
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) fa[i][e] = 0;
+#pragma unroll
+    for (int j = 0; j < FN; ++j)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        fb0[j][e] = 0;
+        fb1[j][e] = 0;
+      }
+
+    // One pipeline step: the MFMAs of the step whose fragments are in (fa, fb_cur) and, row by
+    // row, the LDS reads of the next step's fragments (A in place, B into fb_nxt) from (sa, sb)
+    // plus this row's share of the tile's buffer loads.
+    //   ISSUE: 2 = A and B loads, 1 = B loads only, 0 = none;  ROW0: first row index of the step.
+    auto step = [&](const char* sa, const char* sb, vec8(&fb_cur)[FN], vec8(&fb_nxt)[FN], int h, auto issue_tag,
+                    auto row0_tag) {
+      constexpr int ISSUE = decltype(issue_tag)::value;
+      constexpr int ROW0 = decltype(row0_tag)::value;
+#pragma unroll
+      for (int i = 0; i < FM; ++i) {
+#pragma unroll
+        for (int j = 0; j < FN; ++j) acc[i][j] = Traits::mfma(fb_cur[j], fa[i], acc[i][j]);
+        fa[i] = *(const vec8*)(sa + i * 16 * kRowBytes);
+#pragma unroll
+        for (int j = i * FN / FM; j < (i + 1) * FN / FM; ++j) fb_nxt[j] = *(const vec8*)(sb + j * 16 * kRowBytes);
+        if (ISSUE) {
+#pragma unroll
+          for (int u = 0; u < PER_ROW; ++u) {
+            const int l = (ROW0 + i) * PER_ROW + u;  // B first: it is needed one tile sooner
+            if (l < LB) load_b(l, h + BST - 1);
+            else if (l < LOADS && ISSUE == 2) load_a(l - LB, h + AST - 1);
+          }
+        }
+      }
+      // Scheduling pipeline for the compiler: per row, FN MFMAs with the row's LDS reads spread
+      // between them, then the row's buffer loads.
+#pragma unroll
+      for (int i = 0; i < FM; ++i) {
+        constexpr int R = 1 + FN / FM;                // LDS reads per row (when FN >= FM)
+        constexpr int G = FN / R > 0 ? FN / R : 1;    // MFMAs between reads
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+          __builtin_amdgcn_sched_group_barrier(0x008, G, 0);  // MFMA
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // DS read
+        }
+        if (FN - G * R > 0) __builtin_amdgcn_sched_group_barrier(0x008, FN - G * R, 0);
+        if (ISSUE) __builtin_amdgcn_sched_group_barrier(0x020, PER_ROW, 0);  // VMEM read
+      }
+    };
+
+    // One K tile h: make it visible to every wavefront, then two steps.  Step 0 multiplies the
+    // second half of tile h-1 while reading the first half of tile h; step 1 multiplies the first
+    // half of tile h while reading its second half.
+    auto tile_body = [&](int h, auto issue_tag, auto wait_tag) {
+      constexpr int WAITN = decltype(wait_tag)::value;
+      wait_vm_and_lds<WAITN>();  // my fills of tile h have landed; my reads of tile h-1 are done
+      bare_barrier();            // ... and so have everyone else's: the slots of tile h-1 are free
+      const char* sa = smem + (h % AST) * A_BYTES + a_wave_off;
+      const char* sb = smem + B_REGION + (h % BST) * B_BYTES + b_wave_off;
+      step(sa + frag_off[0], sb + frag_off[0], fb1, fb0, h, issue_tag, std::integral_constant<int, 0>{});
+      step(sa + frag_off[1], sb + frag_off[1], fb0, fb1, h, issue_tag, std::integral_constant<int, FM>{});
+    };
+
+    if (n_tiles > 0) {
+      // Prologue: A tiles 0 .. AST-2 and B tiles 0 .. BST-2.
+      if (k_tail) fill_short_tile(k_tail);
+#pragma unroll
+      for (int s = 0; s < AST - 1; ++s) {
+        if (s < n_tiles && !(s == 0 && k_tail)) {
+#pragma unroll
+          for (int i = 0; i < LA; ++i) load_a(i, s);
+        }
+        if (s < BST - 1 && s < n_tiles && !(s == 0 && k_tail)) {
+#pragma unroll
+          for (int i = 0; i < LB; ++i) load_b(i, s);
+        }
+      }
+      wait_vm_and_lds<0>();
+      int h = 0;
+      for (; h < n_tiles - (AST - 1); ++h)
+        tile_body(h, std::integral_constant<int, 2>{}, std::integral_constant<int, WAIT_STEADY>{});
+      for (; h < n_tiles - (BST - 1); ++h)
+        tile_body(h, std::integral_constant<int, 1>{}, std::integral_constant<int, WAIT_STEADY>{});
+      for (; h < n_tiles; ++h) tile_body(h, std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{});
+      // Drain: the second half of the last tile is in (fa, fb1).
 #pragma unroll
       for (int i = 0; i < FM; ++i)
 #pragma unroll
-        for (int j = 0; j < FN; ++j) acc[i][j] = Traits::mfma(fb[j], fa[i], acc[i][j]);
-    };
-
-    // K offset (inside the slice) of tile t: the short tile comes first.
-    auto tile_koff = [&](int t) { return k_tail ? (t == 0 ? kt_full * kBK : (t - 1) * kBK) : t * kBK; };
-
-    if (n_tiles > 0) {
-      if (k_tail) {
-        fill_staged(0, tile_koff(0), k_tail);
-      } else if (DIRECT) {
-        fill_direct(0, 0);
-      } else {
-        fill_staged(0, 0, kBK);
-      }
-      __builtin_amdgcn_s_waitcnt(0);  // vmcnt(0) expcnt(0) lgkmcnt(0)
-      __syncthreads();
-
-      vec8 fa0[FM], fb0[FN], fa1[FM], fb1[FN];
-      read_frags(0, 0, fa0, fb0);
-
-      for (int t = 0; t < n_tiles; ++t) {
-        const int cur = t & 1;
-        const int nxt = cur ^ 1;
-        const bool has_next = (t + 1 < n_tiles);
-        if (DIRECT) {
-          if (has_next) fill_direct(nxt, tile_koff(t + 1));
-          read_frags(cur, 1, fa1, fb1);
-          mma(fa0, fb0);
-          read_frags(cur, 2, fa0, fb0);
-          mma(fa1, fb1);
-          read_frags(cur, 3, fa1, fb1);
-          mma(fa0, fb0);
-        } else {
-          i32x4 ra[LA], rb[LB];
-          if (has_next) {
-            const int koff = tile_koff(t + 1);
-#pragma unroll
-            for (int i = 0; i < LA; ++i)
-              ra[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_a, (int)voff_a[i], koff * 2, 0);
-#pragma unroll
-            for (int i = 0; i < LB; ++i)
-              rb[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, (int)voff_b[i], koff * 2, 0);
-          }
-          read_frags(cur, 1, fa1, fb1);
-          mma(fa0, fb0);
-          read_frags(cur, 2, fa0, fb0);
-          mma(fa1, fb1);
-          read_frags(cur, 3, fa1, fb1);
-          mma(fa0, fb0);
-          if (has_next) {
-            char* sa = smem + nxt * STAGE_BYTES + tid * 16;
-            char* sb = sa + A_BYTES;
-#pragma unroll
-            for (int i = 0; i < LA; ++i) *(i32x4*)(sa + i * (NT * 16)) = ra[i];
-#pragma unroll
-            for (int i = 0; i < LB; ++i) *(i32x4*)(sb + i * (NT * 16)) = rb[i];
-          }
-        }
-        // Every wavefront has read all of stage `cur`; the fill of `nxt` has landed.
-        __builtin_amdgcn_s_waitcnt(0);
-        __syncthreads();
-        if (has_next) read_frags(nxt, 0, fa0, fb0);
-        mma(fa1, fb1);
-      }
+        for (int j = 0; j < FN; ++j) acc[i][j] = Traits::mfma(fb1[j], fa[i], acc[i][j]);
     }
 
     // ---- epilogue ---------------------------------------------------------------------
-    // acc[i][j][r]: row m = row0 + wm*TM + i*32 + (lane & 31),
-    //               col n = col0 + wn*TN + j*32 + 8*(r/4) + 4*(lane>>5) + (r%4).
-    const int m_base = row0 + wm * TM + (lane & 31);
-    const int n_base = col0 + wn * TN + 4 * (lane >> 5);
+    // acc[i][j][e]: row m = row0 + wm*TM + i*16 + (lane & 15),
+    //               col n = col0 + wn*TN + j*16 + 4*(lane>>4) + e.
+    const int m_base = row0 + wm * TM + (lane & 15);
+    const int n_base = col0 + wn * TN + 4 * (lane >> 4);
     const bool vec_ok = (N % 4) == 0;
 
     if (EPI == kEpiStore) {
       T* C = (T*)p.C;
 #pragma unroll
       for (int i = 0; i < FM; ++i) {
-        const int m = m_base + i * 32;
+        const int m = m_base + i * 16;
         if (m >= M) continue;
         T* crow = C + (size_t)m * N;
 #pragma unroll
         for (int j = 0; j < FN; ++j) {
+          const int n = n_base + j * 16;
+          vec4 v;
 #pragma unroll
-          for (int g = 0; g < 4; ++g) {
-            const int n = n_base + j * 32 + g * 8;
-            vec4 v;
+          for (int e = 0; e < 4; ++e) v[e] = (T)acc[i][j][e];
+          if (vec_ok && n + 3 < N) {
+            *(vec4*)(crow + n) = v;
+          } else {
 #pragma unroll
-            for (int e = 0; e < 4; ++e) v[e] = (T)acc[i][j][g * 4 + e];
-            if (vec_ok && n + 3 < N) {
-              *(vec4*)(crow + n) = v;
-            } else {
-#pragma unroll
-              for (int e = 0; e < 4; ++e)
-                if (n + e < N) crow[n + e] = v[e];
-            }
+            for (int e = 0; e < 4; ++e)
+              if (n + e < N) crow[n + e] = v[e];
           }
         }
       }
-    } else if (EPI == kEpiPartial) {
-      float* W = p.ws + (size_t)blockIdx.z * M * N;
+    } else {
+      if (EPI == kEpiLnStats) {
+        // Per-row statistics over the columns this workgroup owns, from the fp32 accumulators.
+        // A row's TN columns of one wavefront sit in four lanes (l, l^16, l^32, l^48): reduce in
+        // registers, swap twice across the lane groups, then combine the WAVES_N wavefronts via
+        // LDS with Chan's pairwise update, so no precision is lost to cancellation.
+        __syncthreads();            // every LDS slot is dead; reuse the space for the exchange
+        float* red = (float*)smem;  // [BM][WAVES_N][2]
+        const int cols_here = (N - col0) < BN ? (N - col0) : BN;
+#pragma unroll
+        for (int i = 0; i < FM; ++i) {
+          float s = 0.0f;
+          int cnt = 0;
+#pragma unroll
+          for (int j = 0; j < FN; ++j)
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              if (n_base + j * 16 + e < N) {
+                s += acc[i][j][e];
+                ++cnt;
+              }
+          s += __shfl_xor(s, 16);
+          s += __shfl_xor(s, 32);
+          cnt += __shfl_xor(cnt, 16);
+          cnt += __shfl_xor(cnt, 32);
+          const float mean = cnt > 0 ? s / (float)cnt : 0.0f;
+          float m2 = 0.0f;
+#pragma unroll
+          for (int j = 0; j < FN; ++j)
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              if (n_base + j * 16 + e < N) {
+                const float d = acc[i][j][e] - mean;
+                m2 += d * d;
+              }
+          m2 += __shfl_xor(m2, 16);
+          m2 += __shfl_xor(m2, 32);
+          if (lane < 16) {
+            const int rl = wm * TM + i * 16 + lane;
+            red[(rl * WAVES_N + wn) * 2 + 0] = mean;
+            red[(rl * WAVES_N + wn) * 2 + 1] = m2;
+          }
+        }
+        __syncthreads();
+        for (int rl = tid; rl < BM; rl += NT) {
+          const int m = row0 + rl;
+          if (m >= M) continue;
+          float mean = 0.0f, m2 = 0.0f, n_acc = 0.0f;
+#pragma unroll
+          for (int w = 0; w < WAVES_N; ++w) {
+            int cw = cols_here - w * TN;
+            cw = cw < 0 ? 0 : (cw > TN ? TN : cw);
+            if (cw == 0) continue;
+            const float mw = red[(rl * WAVES_N + w) * 2 + 0];
+            const float qw = red[(rl * WAVES_N + w) * 2 + 1];
+            const float nb = (float)cw;
+            const float tot = n_acc + nb;
+            const float delta = mw - mean;
+            mean += delta * (nb / tot);
+            m2 += qw + delta * delta * (n_acc * nb / tot);
+            n_acc = tot;
+          }
+          float* st = p.stats + ((size_t)m * p.tiles_n + tc.tn) * 2;
+          st[0] = mean;
+          st[1] = m2;
+        }
+      }
+      // fp32 tile: split-K partial sums of this slice, or X for the normalisation pass.
+      float* W = p.ws + (EPI == kEpiPartial ? (size_t)blockIdx.z * M * N : (size_t)0);
 #pragma unroll
       for (int i = 0; i < FM; ++i) {
-        const int m = m_base + i * 32;
+        const int m = m_base + i * 16;
         if (m >= M) continue;
         float* wrow = W + (size_t)m * N;
 #pragma unroll
         for (int j = 0; j < FN; ++j) {
+          const int n = n_base + j * 16;
+          if (vec_ok && n + 3 < N) {
+            *(f32x4*)(wrow + n) = acc[i][j];
+          } else {
 #pragma unroll
-          for (int g = 0; g < 4; ++g) {
-            const int n = n_base + j * 32 + g * 8;
-            f32x4 v;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) v[e] = acc[i][j][g * 4 + e];
-            if (vec_ok && n + 3 < N) {
-              *(f32x4*)(wrow + n) = v;
-            } else {
-#pragma unroll
-              for (int e = 0; e < 4; ++e)
-                if (n + e < N) wrow[n + e] = v[e];
-            }
-          }
-        }
-      }
-    } else {  // kEpiLnStats
-      // Per-row statistics over the columns this workgroup owns, from the fp32 accumulators.
-      // A row's TN columns of one wavefront sit in two lanes (l, l^32): reduce in registers,
-      // swap once across the half-wavefronts, then combine the WAVES_N wavefronts via LDS
-      // with Chan's pairwise update so no precision is lost to cancellation.
-      __syncthreads();  // LDS stages are dead; reuse them for the cross-wavefront exchange
-      float* red = (float*)smem;  // [BM][WAVES_N][2]
-      const int cols_here = (N - col0) < BN ? (N - col0) : BN;
-#pragma unroll
-      for (int i = 0; i < FM; ++i) {
-        float s = 0.0f;
-        int cnt = 0;
-#pragma unroll
-        for (int j = 0; j < FN; ++j)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            const int n = n_base + j * 32 + (r / 4) * 8 + (r % 4);
-            if (n < N) { s += acc[i][j][r]; ++cnt; }
-          }
-        s += __shfl_xor(s, 32);
-        cnt += __shfl_xor(cnt, 32);
-        const float mean = cnt > 0 ? s / (float)cnt : 0.0f;
-        float m2 = 0.0f;
-#pragma unroll
-        for (int j = 0; j < FN; ++j)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            const int n = n_base + j * 32 + (r / 4) * 8 + (r % 4);
-            if (n < N) { const float d = acc[i][j][r] - mean; m2 += d * d; }
-          }
-        m2 += __shfl_xor(m2, 32);
-        if (lane < 32) {
-          const int rl = wm * TM + i * 32 + lane;
-          red[(rl * WAVES_N + wn) * 2 + 0] = mean;
-          red[(rl * WAVES_N + wn) * 2 + 1] = m2;
-        }
-      }
-      __syncthreads();
-      for (int rl = tid; rl < BM; rl += NT) {
-        const int m = row0 + rl;
-        if (m >= M) continue;
-        float mean = 0.0f, m2 = 0.0f, n_acc = 0.0f;
-#pragma unroll
-        for (int w = 0; w < WAVES_N; ++w) {
-          int cw = cols_here - w * TN;
-          cw = cw < 0 ? 0 : (cw > TN ? TN : cw);
-          if (cw == 0) continue;
-          const float mw = red[(rl * WAVES_N + w) * 2 + 0];
-          const float qw = red[(rl * WAVES_N + w) * 2 + 1];
-          const float nb = (float)cw;
-          const float tot = n_acc + nb;
-          const float delta = mw - mean;
-          mean += delta * (nb / tot);
-          m2 += qw + delta * delta * (n_acc * nb / tot);
-          n_acc = tot;
-        }
-        float* st = p.stats + ((size_t)m * p.tiles_n + tc.tn) * 2;
-        st[0] = mean;
-        st[1] = m2;
-      }
-      // fp32 X for the normalisation pass.
-      float* X = p.ws;
-#pragma unroll
-      for (int i = 0; i < FM; ++i) {
-        const int m = m_base + i * 32;
-        if (m >= M) continue;
-        float* xrow = X + (size_t)m * N;
-#pragma unroll
-        for (int j = 0; j < FN; ++j) {
-#pragma unroll
-          for (int g = 0; g < 4; ++g) {
-            const int n = n_base + j * 32 + g * 8;
-            f32x4 v;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) v[e] = acc[i][j][g * 4 + e];
-            if (vec_ok && n + 3 < N) {
-              *(f32x4*)(xrow + n) = v;
-            } else {
-#pragma unroll
-              for (int e = 0; e < 4; ++e)
-                if (n + e < N) xrow[n + e] = v[e];
-            }
+            for (int e = 0; e < 4; ++e)
+              if (n + e < N) wrow[n + e] = acc[i][j][e];
           }
         }
       }
@@ -442,11 +462,11 @@ struct GemmTile {
   }
 };
 
-template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, int EPI, bool DIRECT>
+template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, int EPI, int AST, int BST>
 __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
     gemmrc_kernel(const GemmParams p) {
   extern __shared__ __attribute__((aligned(1024))) char smem[];
-  GemmTile<T, BM, BN, WAVES_M, WAVES_N, EPI, DIRECT>::run(p, smem);
+  GemmTile<T, BM, BN, WAVES_M, WAVES_N, EPI, AST, BST>::run(p, smem);
 }
 
 }  // namespace beam

@@ -1,5 +1,5 @@
 // Table of compiled gemmrc kernels: one KernelSet per (workgroup tile, wavefront tile),
-// holding a launcher for every (dtype, epilogue, loader) combination.
+// holding a launcher for every (dtype, epilogue, pipeline depth) combination.
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -15,13 +15,14 @@ struct KernelSet {
   int block_m, block_n, wave_m, wave_n;
   int threads;
   int lds_bytes;
-  GemmLauncher launch[2][3][2];  // [dtype][epilogue][loader: 0 direct, 1 staged]
+  int lds_bytes_shallow;
+  GemmLauncher launch[2][3][2];  // [dtype][epilogue][pipeline: 0 = 3 A + 2 B slots, 1 = 2 + 2]
 };
 
-template <typename T, int BM, int BN, int WVM, int WVN, int EPI, bool DIRECT>
+template <typename T, int BM, int BN, int WVM, int WVN, int EPI, int AST, int BST>
 hipError_t launch_gemm(const GemmParams& p, dim3 grid, hipStream_t stream) {
-  using Tile = GemmTile<T, BM, BN, WVM, WVN, EPI, DIRECT>;
-  auto kern = gemmrc_kernel<T, BM, BN, WVM, WVN, EPI, DIRECT>;
+  using Tile = GemmTile<T, BM, BN, WVM, WVN, EPI, AST, BST>;
+  auto kern = gemmrc_kernel<T, BM, BN, WVM, WVN, EPI, AST, BST>;
   static bool configured = false;  // benign race: the attribute call is idempotent
   if (!configured) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -42,14 +43,15 @@ KernelSet make_kernel_set() {
   k.wave_m = TM;
   k.wave_n = TN;
   k.threads = WVM * WVN * 64;
-  k.lds_bytes = GemmTile<_Float16, BM, BN, WVM, WVN, kEpiStore, true>::LDS_BYTES;
+  k.lds_bytes = GemmTile<_Float16, BM, BN, WVM, WVN, kEpiStore, 3, 2>::LDS_BYTES;
+  k.lds_bytes_shallow = GemmTile<_Float16, BM, BN, WVM, WVN, kEpiStore, 2, 2>::LDS_BYTES;
 #define BEAM_FILL(D, T)                                                             \
-  k.launch[D][kEpiStore][0] = launch_gemm<T, BM, BN, WVM, WVN, kEpiStore, true>;     \
-  k.launch[D][kEpiStore][1] = launch_gemm<T, BM, BN, WVM, WVN, kEpiStore, false>;    \
-  k.launch[D][kEpiPartial][0] = launch_gemm<T, BM, BN, WVM, WVN, kEpiPartial, true>; \
-  k.launch[D][kEpiPartial][1] = launch_gemm<T, BM, BN, WVM, WVN, kEpiPartial, false>; \
-  k.launch[D][kEpiLnStats][0] = launch_gemm<T, BM, BN, WVM, WVN, kEpiLnStats, true>; \
-  k.launch[D][kEpiLnStats][1] = launch_gemm<T, BM, BN, WVM, WVN, kEpiLnStats, false>;
+  k.launch[D][kEpiStore][0] = launch_gemm<T, BM, BN, WVM, WVN, kEpiStore, 3, 2>;     \
+  k.launch[D][kEpiStore][1] = launch_gemm<T, BM, BN, WVM, WVN, kEpiStore, 2, 2>;     \
+  k.launch[D][kEpiPartial][0] = launch_gemm<T, BM, BN, WVM, WVN, kEpiPartial, 3, 2>; \
+  k.launch[D][kEpiPartial][1] = launch_gemm<T, BM, BN, WVM, WVN, kEpiPartial, 2, 2>; \
+  k.launch[D][kEpiLnStats][0] = launch_gemm<T, BM, BN, WVM, WVN, kEpiLnStats, 3, 2>; \
+  k.launch[D][kEpiLnStats][1] = launch_gemm<T, BM, BN, WVM, WVN, kEpiLnStats, 2, 2>;
   BEAM_FILL(0, _Float16)
   BEAM_FILL(1, __bf16)
 #undef BEAM_FILL

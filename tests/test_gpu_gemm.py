@@ -50,7 +50,7 @@ def all_configs(beamc):
 
 
 def test_1024_cube_every_config(gpu, beamc, oracle):
-    """fp16 1024^3, uniform[-1,1): every compiled tile, both loaders."""
+    """fp16 1024^3, uniform[-1,1): every compiled tile, both pipeline depths."""
     M = N = K = 1024
     a = beamc.host_uniform((M, K), F16, 1, 0)
     b = beamc.host_uniform((N, K), F16, 1, 1)
