@@ -1,0 +1,152 @@
+"""Host-side logic of libbeam_hip.so that needs no GPU: index maps shared with the kernels,
+the split heuristic, workspace sizes, the synthetic-data generator and argument validation."""
+import ctypes
+
+import numpy as np
+import pytest
+
+F16, BF16 = 0, 1
+
+
+def tile_of(L, wg, tiles_m, tiles_n, g):
+    a, b = ctypes.c_int(), ctypes.c_int()
+    assert L.beam_dbg_tile_of_workgroup(wg, tiles_m, tiles_n, g, ctypes.byref(a), ctypes.byref(b)) == 0
+    return a.value, b.value
+
+
+@pytest.mark.parametrize("tiles_m,tiles_n,g", [(32, 32, 8), (1, 1, 8), (3, 5, 8), (12, 20, 8), (7, 13, 4),
+                                               (16, 16, 16), (5, 1, 8), (1, 9, 8), (33, 17, 8), (16, 43, 8)])
+def test_rasterisation_is_a_bijection(beamc, tiles_m, tiles_n, g):
+    """Every workgroup id maps to a distinct tile (reference counterpart:
+    cuda/cute_kernels/cute_gemm_128x128.cu:22-33)."""
+    seen = {tile_of(beamc.lib, wg, tiles_m, tiles_n, g) for wg in range(tiles_m * tiles_n)}
+    assert len(seen) == tiles_m * tiles_n
+    assert all(0 <= tm < tiles_m and 0 <= tn < tiles_n for tm, tn in seen)
+
+
+def test_rasterisation_is_xcd_local(beamc):
+    """Workgroups that share an XCD (ids congruent mod 8) own one contiguous band of the grouped
+    order: at 32x32 tiles, each XCD's first 32 workgroups cover an 8 x 4 block of tiles."""
+    for xcd in range(8):
+        block = {tile_of(beamc.lib, xcd + 8 * i, 32, 32, 8) for i in range(32)}
+        ms = {t[0] for t in block}
+        ns = {t[1] for t in block}
+        assert len(ms) == 8 and len(ns) == 4, (xcd, sorted(block))
+
+
+def test_lds_swizzle(beamc):
+    """(row, chunk) -> byte offset is a bijection on a slot, and every group of 16 lanes of a
+    ds_read_b128 fragment read (16x16x32 operand: lane l reads row l%16, chunk 4*kk + l/16) hits 16
+    distinct 16-byte slots of the 64-bank sweep: no bank conflicts."""
+    L = beamc.lib
+    offs = {L.beam_dbg_lds_offset(r, c) for r in range(256) for c in range(8)}
+    assert len(offs) == 256 * 8 and min(offs) == 0 and max(offs) == 256 * 128 - 16
+    for kk in range(2):
+        for base in range(0, 64, 16):
+            slots = {(L.beam_dbg_lds_offset(l & 15, 4 * kk + (l >> 4)) % 256) // 16 for l in range(base, base + 16)}
+            assert len(slots) == 16
+    # the fill side: a wavefront's 64 lanes write one contiguous KiB (8 rows x 8 positions)
+    for row0 in range(0, 256, 8):
+        span = sorted(L.beam_dbg_lds_offset(row0 + r, c) for r in range(8) for c in range(8))
+        assert span == list(range(row0 * 128, row0 * 128 + 1024, 16))
+
+
+def test_slice_heuristic_matches_reference_rule(beamc, oracle):
+    for units in (108, 256):
+        for tiles in range(1, units + 2):
+            assert beamc.lib.beam_slice_heuristic(tiles, units) == oracle.slice_heuristic(tiles, float(units))
+    assert beamc.lib.beam_slice_heuristic(4, 108) == 41
+
+
+def test_split_partition(beamc, oracle):
+    cfg = beamc.TileConfig(64, 64, 32, 32).to_c()
+    for K in (64, 200, 1000, 4104, 32768):
+        ktiles = (K + 63) // 64
+        for s in (1, 2, 3, 7, 16, 64, 1000):
+            eff = beamc.lib.beam_splitk_effective(256, 256, K, ctypes.byref(cfg), s)
+            assert 1 <= eff <= min(s, ktiles)
+            L = oracle.split_k_len(K, eff)
+            assert L * eff >= K and L * (eff - 1) < K          # no empty slice
+    assert beamc.lib.beam_splitk_workspace_bytes(256, 256, 8) == 8 * 256 * 256 * 4
+    assert beamc.lib.beam_splitk_workspace_bytes(0, 256, 8) == 0
+
+
+def _mix(x):
+    x = x + np.uint64(0x9E3779B97F4A7C15)
+    x = (x ^ (x >> np.uint64(30))) * np.uint64(0xBF58476D1CE4E5B9)
+    x = (x ^ (x >> np.uint64(27))) * np.uint64(0x94D049BB133111EB)
+    return x ^ (x >> np.uint64(31))
+
+
+def _draw(seed, tensor_id, n):
+    with np.errstate(over="ignore"):
+        base = _mix(np.uint64(seed) + np.uint64(0x632BE59BD9B4E019) * (np.uint64(tensor_id) + np.uint64(1)))
+        return _mix(base + np.arange(n, dtype=np.uint64))
+
+
+def test_generator_uniform_bit_exact(beamc, oracle):
+    n = 100_000
+    r = _draw(7, 3, n)
+    v = (r >> np.uint64(40)).astype(np.float32) * np.float32(1 / 8388608.0) - np.float32(1)
+    assert (beamc.host_uniform((n,), F16, 7, 3) == v.astype(np.float16).view(np.uint16)).all()
+    assert (beamc.host_uniform((n,), BF16, 7, 3) == oracle.from_f32(v, BF16)).all()
+    # different tensors / seeds give different streams; same arguments give the same bits
+    assert (beamc.host_uniform((n,), F16, 7, 3) == beamc.host_uniform((n,), F16, 7, 3)).all()
+    assert (beamc.host_uniform((n,), F16, 7, 4) != beamc.host_uniform((n,), F16, 7, 3)).mean() > 0.9
+    assert (beamc.host_uniform((n,), F16, 8, 3) != beamc.host_uniform((n,), F16, 7, 3)).mean() > 0.9
+    x = beamc.host_uniform((400, 500), F16, 1, 0).view(np.float16).astype(np.float64)
+    assert x.min() >= -1.0 and x.max() <= 1.0 and abs(x.mean()) < 0.01 and abs(x.std() - 3 ** -0.5) < 0.01
+
+
+def test_generator_normal(beamc):
+    n = 200_000
+    r = _draw(5, 2, n)
+    u1 = ((r >> np.uint64(40)).astype(np.float64) + 1.0) / 16777216.0
+    u2 = ((r >> np.uint64(8)) & np.uint64(0xFFFFFF)).astype(np.float64) / 16777216.0
+    z = np.sqrt(-2.0 * np.log(u1)) * np.cos(2.0 * np.pi * u2)
+    want = (1.0 + 0.1 * z).astype(np.float32).astype(np.float16)
+    got = beamc.host_normal((n,), F16, 5, 2, 1.0, 0.1).view(np.float16)
+    # libm and numpy may differ in the last bit of log/cos: allow a handful of 1-ulp flips
+    diff = np.abs(got.view(np.uint16).astype(np.int32) - want.view(np.uint16).astype(np.int32))
+    assert diff.max() <= 1 and (diff != 0).mean() < 1e-3
+    x = beamc.host_normal((n,), BF16, 9, 0, 0.0, 2.0)
+    f = (x.astype(np.uint32) << 16).view(np.float32).astype(np.float64)
+    assert abs(f.mean()) < 0.02 and abs(f.std() - 2.0) < 0.02
+
+
+def test_argument_validation_without_gpu(beamc):
+    """Checks that fail before any device call."""
+    L = beamc.lib
+    cfg = beamc.TileConfig(128, 128, 64, 64).to_c()
+    assert L.beam_gemmrc(1 << 20, 1 << 20, 1 << 20, -1, 4, 8, 0, ctypes.byref(cfg), None) == 1
+    assert L.beam_gemmrc(1 << 20, 1 << 20, 1 << 20, 4, 4, 8, 7, ctypes.byref(cfg), None) == 2      # dtype
+    assert L.beam_gemmrc(1 << 20, 1 << 20, 1 << 20, 4, 4, 12, 0, ctypes.byref(cfg), None) == 2     # K % 8
+    assert L.beam_gemmrc((1 << 20) + 2, 1 << 20, 1 << 20, 4, 4, 8, 0, ctypes.byref(cfg), None) == 2  # alignment
+    assert L.beam_gemmrc(None, 1 << 20, 1 << 20, 4, 4, 8, 0, ctypes.byref(cfg), None) == 1
+    assert b"null" in L.beam_last_error()
+    assert L.beam_gemmrc(None, None, None, 0, 4, 8, 0, None, None) == 0                             # empty: no-op
+    bad = beamc._TileCfg(96, 96, 48, 48, 0, 0)
+    assert L.beam_splitk_effective(64, 64, 64, ctypes.byref(bad), 2) == -1
+    assert b"no kernel" in L.beam_last_error()
+    out = beamc._TileCfg()
+    assert L.beam_get_config(-1, ctypes.byref(out)) == 1
+    assert L.beam_get_config(10 ** 6, ctypes.byref(out)) == 1
+
+
+def test_config_table(beamc):
+    cfgs = beamc.list_configs()
+    shapes = {(c.block_m, c.block_n, c.wave_m, c.wave_n) for c in cfgs}
+    assert len(shapes) == len(cfgs)
+    # the tiles the reference names (python/beam/tuner.py:53-59,74-80) are all present
+    for want in [(128, 128, 64, 64), (128, 256, 64, 64), (256, 128, 64, 64), (256, 128, 128, 32),
+                 (256, 128, 32, 128), (128, 64, 64, 32), (64, 128, 32, 64), (64, 64, 32, 32)]:
+        assert want in shapes
+    for c in cfgs:
+        assert c.block_m % c.wave_m == 0 and c.block_n % c.wave_n == 0
+        waves = (c.block_m // c.wave_m) * (c.block_n // c.wave_n)
+        assert waves in (4, 8)
+        assert (3 * c.block_m + 2 * c.block_n) * 128 <= 160 * 1024
+    cfg, split = beamc.default_config(8192, 8192, 8192)
+    assert (cfg.block_m, cfg.block_n) == (256, 256) and split == 1
+    cfg, split = beamc.default_config(256, 256, 32768)
+    assert split > 1
