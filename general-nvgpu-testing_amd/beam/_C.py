@@ -13,6 +13,7 @@ from __future__ import annotations
 
 import ctypes
 import os
+import sys
 from dataclasses import dataclass
 from typing import List, Optional, Sequence
 
@@ -55,6 +56,11 @@ def _load() -> ctypes.CDLL:
         raise ImportError(
             f"{_LIB_PATH} is missing: build it with `make -C {os.path.join(_PKG_DIR, 'csrc')}` "
             "(hipcc, gfx950).  There is no fallback path.")
+    # PyTorch wheels bundle their own HIP runtime.  If torch is imported first, the dynamic linker
+    # hands that same runtime to libbeam_hip.so (one runtime per process: tensors and streams can be
+    # shared).  Loaded the other way round, torch would bring a second runtime and fail to see the GPU.
+    global _TORCH_FIRST
+    _TORCH_FIRST = "torch" in sys.modules
     L = ctypes.CDLL(_LIB_PATH)
     vp, i, sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t
     cfgp = ctypes.POINTER(_TileCfg)
@@ -93,6 +99,7 @@ def _load() -> ctypes.CDLL:
     return L
 
 
+_TORCH_FIRST = False
 lib = _load()
 
 
@@ -207,6 +214,9 @@ def _describe(x):
     if isinstance(x, DeviceArray):
         return x.ptr, x.shape, x.dtype, None
     if _is_torch(x):
+        if not _TORCH_FIRST:
+            raise BeamError(1, "torch tensors need `import torch` before `import beam` (one HIP runtime per "
+                               "process); use beam.DeviceArray otherwise")
         import torch
         if not x.is_cuda:
             raise BeamError(1, "tensor is not on the GPU")

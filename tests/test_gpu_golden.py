@@ -44,38 +44,16 @@ def test_ln_fixture(gpu, beamc, path):
     assert err.max() <= 2e-3, path
 
 
-def test_reference_named_operators_on_torch_tensors(gpu, beamc, oracle):
+def test_reference_named_operators_on_torch_tensors(gpu):
     """Scripts written against the reference call f(a=, b=, c=) on CUDA tensors
-    (python/gemm_test.py:78-107); the same calls work here, on torch's current stream."""
-    import torch
-    import beam
-    M, N, K = 512, 640, 1024
-    a_bits = beamc.host_uniform((M, K), F16, 31, 0)
-    b_bits = beamc.host_uniform((N, K), F16, 31, 1)
-    ref = oracle.gemmrc(a_bits, b_bits, F16)
-    a = torch.from_numpy(a_bits.view(np.float16)).cuda()
-    b = torch.from_numpy(b_bits.view(np.float16)).cuda()
-    stream = torch.cuda.Stream()
-    with torch.cuda.stream(stream):
-        for fn, kw in [(beam.custom_gemmrc_128x128, {}), (beam.custom_gemmrc_128x256, {}),
-                       (beam.cutlass_gemmrc, {}),
-                       (beam.cutlass_gemmrc_spec, dict(shape_threadblock=[256, 128], shape_warp=[128, 32])),
-                       (beam.cutlass_gemmrc_splitk, dict(split_k_slices=3)),
-                       (beam.cutlass_gemmrc_splitk_spec, dict(shape_threadblock=[128, 64], shape_warp=[64, 32],
-                                                              split_k_slices=5))]:
-            c = torch.zeros(M, N, dtype=torch.float16, device="cuda")
-            fn(a=a, b=b, c=c, **kw)
-            stream.synchronize()
-            r = oracle.compare(c.cpu().numpy().view(np.uint16), ref, F16)
-            assert r["max_abs_err"] <= oracle.gemm_tolerance(K) * r["rms_ref"], fn.__name__
-    # unsupported inputs raise instead of returning silently
-    with pytest.raises(beam.BeamError):
-        beam.cutlass_gemmrc(a=a.float(), b=b.float(), c=torch.zeros(M, N, device="cuda"))
-    with pytest.raises(beam.BeamError):
-        beam.cutlass_gemmrc(a=a.cpu(), b=b, c=torch.zeros(M, N, dtype=torch.float16, device="cuda"))
-    with pytest.raises(beam.BeamError):
-        beam.cutlass_gemmrc_spec(a=a, b=b, c=torch.zeros(M, N, dtype=torch.float16, device="cuda"),
-                                 shape_threadblock=[48, 48])
+    (python/gemm_test.py:78-107); the same calls work here, on torch's current stream.  Runs in its own
+    process because torch must be imported before beam (they then share torch's HIP runtime)."""
+    import subprocess
+    import sys
+    script = os.path.join(os.path.dirname(os.path.abspath(__file__)), "torch_dropin_check.py")
+    r = subprocess.run([sys.executable, "-u", script], capture_output=True, text=True, timeout=600)
+    assert r.returncode == 0, r.stdout[-3000:] + r.stderr[-3000:]
+    assert "torch drop-in OK" in r.stdout
 
 
 def test_tuner_end_to_end(gpu, beamc, tmp_path):

@@ -1,0 +1,35 @@
+"""The C++ host (beam_host: test registry + CLI over the C ABI) runs its self-checks on the GPU."""
+import os
+import subprocess
+
+import pytest
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HOST = os.path.join(ROOT, "general-nvgpu-testing_amd", "beam_host")
+
+
+def run(*args, timeout=240):
+    return subprocess.run([HOST, *args], capture_output=True, text=True, timeout=timeout)
+
+
+def test_registry_runs_green(gpu):
+    assert os.path.exists(HOST), "beam_host is not built (make -C general-nvgpu-testing_amd/csrc)"
+    listed = run("--list").stdout.split()
+    assert {"identity_every_tile", "all_ones_ragged", "one_hot_k_tail", "splitk_consistency",
+            "layernorm_invariants", "error_paths"} <= set(listed)
+    r = run("--run", "all")
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert r.stdout.count("[ OK ]") == len(listed) and "FAIL" not in r.stdout
+
+
+def test_cli_bench_and_info(gpu):
+    r = run("--info")
+    assert r.returncode == 0 and "gfx950" in r.stdout
+    r = run("--bench", "--m", "1024", "--n", "1024", "--k", "1024", "--tile", "128x128", "--wave", "64x64", "--iters", "5")
+    assert r.returncode == 0 and "TFLOP/s" in r.stdout, r.stdout + r.stderr
+    r = run("--bench", "--op", "splitk", "--m", "256", "--n", "256", "--k", "8192", "--tile", "64x64", "--wave", "32x32",
+            "--splitk", "16", "--iters", "5")
+    assert r.returncode == 0 and "split 16" in r.stdout, r.stdout + r.stderr
+    r = run("--bench", "--tile", "100x100")
+    assert r.returncode != 0
