@@ -81,6 +81,12 @@ def _load() -> ctypes.CDLL:
     L.beam_gemmrc_ln_workspace_bytes.argtypes = [i, i, cfgp]
     L.beam_gemmrc_ln_workspace_bytes.restype = sz
     L.beam_gemmrc_ln.argtypes = [vp, vp, vp, vp, ctypes.c_float, vp, i, i, i, i, cfgp, vp, sz, vp]
+    L.beam_gemmrc_ln_workspace_bytes_ex.argtypes = [i, i, cfgp, i]
+    L.beam_gemmrc_ln_workspace_bytes_ex.restype = sz
+    L.beam_gemmrc_ln_ex.argtypes = [vp, vp, vp, vp, ctypes.c_float, vp, i, i, i, i, cfgp, i, vp, sz, vp]
+    L.beam_set_ln_spin_limit.argtypes = [i]
+    L.beam_gemmrc_ln_workspace_reset.argtypes = [vp]
+    L.beam_gemmrc_ln_timed_out.argtypes = [vp, vp, ctypes.POINTER(i)]
     L.beam_bench.argtypes = [i, ctypes.POINTER(_Problem), cfgp, i, i, vp, ctypes.POINTER(ctypes.c_float)]
     L.beam_event_create.argtypes = [ctypes.POINTER(vp)]
     L.beam_event_record.argtypes = [vp, vp]
@@ -96,6 +102,8 @@ def _load() -> ctypes.CDLL:
     L.beam_host_fill_normal.argtypes = [vp, sz, i, ctypes.c_uint64, ctypes.c_uint64, ctypes.c_float, ctypes.c_float]
     L.beam_dbg_tile_of_workgroup.argtypes = [i, i, i, i, ctypes.POINTER(i), ctypes.POINTER(i)]
     L.beam_dbg_lds_offset.argtypes = [i, i]
+    L.beam_dbg_band_block_tile.argtypes = [i, i, i, i, i, ctypes.POINTER(i), ctypes.POINTER(i)]
+    L.beam_dbg_band_block_grid.argtypes = [i, i, i]
     return L
 
 
@@ -263,6 +271,19 @@ def _cfg_from_shapes(shape_threadblock, shape_warp, pipeline=0, group_m=0) -> _T
 # ---------------------------------------------------------------------------- workspaces
 
 _workspace: Optional[DeviceArray] = None
+_ln_workspace: Optional[DeviceArray] = None  # fused GEMM+LayerNorm keeps state in its workspace: never shared
+
+
+def _get_ln_workspace(nbytes: int) -> DeviceArray:
+    global _ln_workspace
+    if _ln_workspace is None or _ln_workspace.nbytes < nbytes:
+        if _ln_workspace is not None:
+            _check(lib.beam_sync(None))
+            lib.beam_gemmrc_ln_workspace_reset(_ln_workspace.ptr)
+            _ln_workspace.free()
+        _ln_workspace = DeviceArray((max(nbytes, 1 << 20),), itemsize=1)
+        lib.beam_gemmrc_ln_workspace_reset(_ln_workspace.ptr)
+    return _ln_workspace
 
 
 def _get_workspace(nbytes: int) -> DeviceArray:
@@ -317,18 +338,32 @@ def gemmrc_splitk_spec(a, b, c, shape_threadblock=(128, 128), shape_warp=(64, 64
                                   ws.ptr if ws else None, ws.nbytes if ws else 0, st))
 
 
-def gemmrc_ln(a, b, c, gamma, beta, eps: float = 1e-5, config: Optional[TileConfig] = None) -> None:
-    """c = LayerNorm_N(a @ b.T) * gamma + beta, statistics from the fp32 accumulators."""
+LN_AUTO, LN_TWOPASS, LN_FUSED = 0, 1, 2
+
+
+def gemmrc_ln(a, b, c, gamma, beta, eps: float = 1e-5, config: Optional[TileConfig] = None,
+              mode: int = LN_AUTO) -> None:
+    """c = LayerNorm_N(a @ b.T) * gamma + beta, statistics from the fp32 accumulators.
+    mode: LN_AUTO (fused single kernel when N / block_n <= 64), LN_TWOPASS, LN_FUSED."""
     pa, pb, pc, M, N, K, d, st = _problem(a, b, c)
     pg, sg, dg, _ = _describe(gamma)
     pbt, sbt, dbt, _ = _describe(beta)
     if tuple(sg) != (N,) or tuple(sbt) != (N,) or dg != d or dbt != d:
         raise BeamError(1, "gamma and beta must be [N] of the same dtype as a, b, c")
     cfg = config.to_c() if config is not None else None
-    need = lib.beam_gemmrc_ln_workspace_bytes(M, N, ctypes.byref(cfg) if cfg else None)
-    ws = _get_workspace(need)
-    _check(lib.beam_gemmrc_ln(pa, pb, pg, pbt, eps, pc, M, N, K, d, ctypes.byref(cfg) if cfg else None,
-                              ws.ptr, ws.nbytes, st))
+    cfgp = ctypes.byref(cfg) if cfg else None
+    need = lib.beam_gemmrc_ln_workspace_bytes_ex(M, N, cfgp, mode)
+    ws = _get_ln_workspace(need)
+    _check(lib.beam_gemmrc_ln_ex(pa, pb, pg, pbt, eps, pc, M, N, K, d, cfgp, mode, ws.ptr, ws.nbytes, st))
+
+
+def gemmrc_ln_timed_out() -> bool:
+    """True if the last fused GEMM+LayerNorm on the shared workspace gave up waiting for a band."""
+    if _ln_workspace is None:
+        return False
+    flag = ctypes.c_int(0)
+    _check(lib.beam_gemmrc_ln_timed_out(_ln_workspace.ptr, None, ctypes.byref(flag)))
+    return bool(flag.value)
 
 
 def _fixed(fn_name: str):
@@ -375,7 +410,7 @@ def bench(op: int, a, b, c, config: Optional[TileConfig] = None, split_k: int = 
         ws = _get_workspace(max(lib.beam_splitk_workspace_bytes(M, N, s), 1))
     elif op == 2:
         q.gamma, q.beta = _describe(gamma)[0], _describe(beta)[0]
-        ws = _get_workspace(lib.beam_gemmrc_ln_workspace_bytes(M, N, cfgp))
+        ws = _get_ln_workspace(lib.beam_gemmrc_ln_workspace_bytes(M, N, cfgp))
     if ws is not None:
         q.ws, q.ws_bytes = ws.ptr, ws.nbytes
     ms = ctypes.c_float()

@@ -17,4 +17,9 @@ hipError_t launch_ln_apply(const float* X, const float* stats, const void* gamma
                            void* Y, int M, int N, int tiles_n, int block_n, float eps, int dtype,
                            hipStream_t stream);
 
+// ints[0 .. n) = 0 (a fill kernel rather than hipMemsetAsync, so that callers may capture it in a graph).
+hipError_t launch_zero_ints(int* ints, int n, hipStream_t stream);
+// floats[0 .. n) = value
+hipError_t launch_fill_floats(float* floats, size_t n, float value, hipStream_t stream);
+
 }  // namespace beam

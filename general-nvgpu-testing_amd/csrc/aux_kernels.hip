@@ -82,7 +82,25 @@ __global__ void __launch_bounds__(256) ln_apply_kernel(const float* __restrict__
   }
 }
 
+__global__ void zero_ints_kernel(int* p, int n) {
+  for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x) p[i] = 0;
+}
+
+__global__ void fill_floats_kernel(float* p, size_t n, float v) {
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) p[i] = v;
+}
+
 }  // namespace
+
+hipError_t launch_fill_floats(float* floats, size_t n, float value, hipStream_t stream) {
+  hipLaunchKernelGGL(fill_floats_kernel, dim3(256), dim3(256), 0, stream, floats, n, value);
+  return hipGetLastError();
+}
+
+hipError_t launch_zero_ints(int* ints, int n, hipStream_t stream) {
+  hipLaunchKernelGGL(zero_ints_kernel, dim3(1), dim3(256), 0, stream, ints, n);
+  return hipGetLastError();
+}
 
 hipError_t launch_splitk_reduce(const float* ws, void* C, size_t mn, int splits, int dtype,
                                 hipStream_t stream) {

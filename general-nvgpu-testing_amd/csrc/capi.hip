@@ -5,6 +5,8 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <atomic>
+#include <map>
 #include <mutex>
 #include <thread>
 #include <vector>
@@ -47,6 +49,16 @@ struct Device {
 };
 Device g_dev;
 std::mutex g_dev_mu;
+// Per workspace: tile geometry of the fused GEMM+LayerNorm launches it has seen and their number
+// (selects the statistics set).
+struct LnWorkspaceState {
+  long geometry;
+  unsigned launches;
+};
+std::map<const void*, LnWorkspaceState> g_ln_geometry;
+// polls of a band counter (about a microsecond each) before a fused LayerNorm workgroup gives up
+std::atomic<int> g_ln_spin_limit{4 << 20};
+std::mutex g_ln_mu;
 
 const std::vector<KernelSet>& kernel_sets() {
   static const std::vector<KernelSet> sets = [] {
@@ -379,39 +391,144 @@ int beam_gemmrc_splitk(const void* A, const void* B, void* C, int M, int N, int 
   return BEAM_OK;
 }
 
-size_t beam_gemmrc_ln_workspace_bytes(int M, int N, const beam_tile_cfg* cfg) {
+// Fused GEMM+LayerNorm workspace: [band counters (tiles_m) + timeout flag | statistics].
+// Fused GEMM+LayerNorm workspace: [timeout flag, 256 bytes | statistics set 0 | statistics set 1];
+// launches alternate between the sets and each marks the other one "unpublished" for its successor.
+static size_t ln_fused_header_bytes() { return 256; }
+static size_t ln_fused_set_bytes(size_t tiles_m, size_t tiles_n, int block_m) {
+  return align_up(tiles_m * tiles_n * (size_t)block_m * 2 * sizeof(float), 256);
+}
+
+static bool ln_fused_applies(const beam_tile_cfg& c, const KernelSet& ks, int N) {
+  // a band's column tiles are spread over the 8 XCDs; each XCD must hold its share (<= 32) at once,
+  // and the band's statistics ((tiles_n + 1) * block_m pairs) are gathered into the kernel's LDS
+  const int tiles_n = (N + c.block_n - 1) / c.block_n;
+  const int lds = c.pipeline ? ks.lds_bytes_shallow : ks.lds_bytes;
+  return tiles_n <= 64 && (size_t)(tiles_n + 1) * c.block_m * 8 <= (size_t)lds;
+}
+
+static int ln_resolve_mode(int mode, const beam_tile_cfg& c, const KernelSet& ks, int N) {
+  if (mode == BEAM_LN_AUTO) return ln_fused_applies(c, ks, N) ? BEAM_LN_FUSED : BEAM_LN_TWOPASS;
+  return mode;
+}
+
+size_t beam_gemmrc_ln_workspace_bytes_ex(int M, int N, const beam_tile_cfg* cfg, int mode) {
   if (M <= 0 || N <= 0) return 0;
   beam_tile_cfg c;
   const KernelSet* ks;
   if (resolve_cfg(cfg, M, N, 64, &c, &ks)) return 0;
+  const size_t tiles_m = (size_t)(M + c.block_m - 1) / c.block_m;
   const size_t tiles_n = (size_t)(N + c.block_n - 1) / c.block_n;
+  if (ln_resolve_mode(mode, c, *ks, N) == BEAM_LN_FUSED)
+    return ln_fused_header_bytes() + 2 * ln_fused_set_bytes(tiles_m, tiles_n, c.block_m);
   return align_up((size_t)M * N * sizeof(float), 256) + align_up((size_t)M * tiles_n * 2 * sizeof(float), 256);
 }
 
-int beam_gemmrc_ln(const void* A, const void* B, const void* gamma, const void* beta, float eps, void* Y,
-                   int M, int N, int K, int dtype, const beam_tile_cfg* cfg, void* ws, size_t ws_bytes,
-                   void* stream) {
+size_t beam_gemmrc_ln_workspace_bytes(int M, int N, const beam_tile_cfg* cfg) {
+  return beam_gemmrc_ln_workspace_bytes_ex(M, N, cfg, BEAM_LN_AUTO);
+}
+
+int beam_gemmrc_ln_ex(const void* A, const void* B, const void* gamma, const void* beta, float eps, void* Y,
+                      int M, int N, int K, int dtype, const beam_tile_cfg* cfg, int mode, void* ws,
+                      size_t ws_bytes, void* stream) {
   int rc = check_problem(A, B, Y, M, N, K, dtype);
   if (rc) return rc;
   if (M == 0 || N == 0) return BEAM_OK;
   if (!gamma || !beta) return fail(BEAM_ERR_INVALID, "null gamma/beta");
   if (((uintptr_t)gamma | (uintptr_t)beta) & 7) return fail(BEAM_ERR_UNSUPPORTED, "gamma and beta must be 8-byte aligned");
   if (!(eps >= 0.0f)) return fail(BEAM_ERR_INVALID, "eps must be >= 0");
+  if (mode < BEAM_LN_AUTO || mode > BEAM_LN_FUSED) return fail(BEAM_ERR_INVALID, "unknown LayerNorm mode %d", mode);
   if ((rc = beam_init())) return rc;
   hipStream_t st = (hipStream_t)stream;
   beam_tile_cfg c;
   const KernelSet* ks;
   if ((rc = resolve_cfg(cfg, M, N, K, &c, &ks))) return rc;
-  const size_t need = beam_gemmrc_ln_workspace_bytes(M, N, &c);
+  if (mode == BEAM_LN_FUSED && !ln_fused_applies(c, *ks, N))
+    return fail(BEAM_ERR_UNSUPPORTED, "fused LayerNorm: too many column tiles for this tile shape (N=%d, block_n=%d)", N, c.block_n);
+  mode = ln_resolve_mode(mode, c, *ks, N);
+  const size_t need = beam_gemmrc_ln_workspace_bytes_ex(M, N, &c, mode);
   if (!ws || ws_bytes < need)
     return fail(BEAM_ERR_WORKSPACE, "GEMM+LayerNorm needs %zu bytes of workspace, got %zu", need, ws_bytes);
   if ((uintptr_t)ws & 255) return fail(BEAM_ERR_UNSUPPORTED, "workspace must be 256-byte aligned");
   GemmParams p = base_params(A, B, M, N, K, c);
+  // K == 0: the kernels run with an empty K range and produce x = 0, i.e. y = beta.
+  if (mode == BEAM_LN_FUSED) {
+    p.C = Y;
+    // The first launch on a workspace (or after its geometry changed) marks both statistics sets
+    // unpublished; afterwards each launch finds its set prepared by the previous one.  Launches that
+    // share a workspace must be ordered (same stream): overlapping ones would race on the sets.
+    const size_t set_bytes = ln_fused_set_bytes(p.tiles_m, p.tiles_n, c.block_m);
+    const long geometry = ((long)p.tiles_m << 32) | ((long)p.tiles_n << 12) | c.block_m;
+    unsigned launches = 0;
+    {
+      std::lock_guard<std::mutex> lk(g_ln_mu);
+      auto it = g_ln_geometry.find(ws);
+      if (it != g_ln_geometry.end() && it->second.geometry == geometry) launches = it->second.launches;
+      g_ln_geometry[ws] = LnWorkspaceState{geometry, launches + 1};
+    }
+    float* sets = (float*)((char*)ws + ln_fused_header_bytes());
+    if (launches == 0) {
+      BEAM_HIP(launch_zero_ints((int*)ws, 1, st));
+      BEAM_HIP(launch_fill_floats(sets, 2 * set_bytes / sizeof(float), -1.0f, st));
+    }
+    p.stats = (float*)((char*)sets + (launches & 1u) * set_bytes);
+    p.next_stats = (float*)((char*)sets + ((launches + 1) & 1u) * set_bytes);
+    p.timeout_flag = (int*)ws;
+    p.gamma = gamma;
+    p.beta = beta;
+    p.eps = eps;
+    p.spin_limit = g_ln_spin_limit.load();
+    // band groups: XCD x owns group_n columns of group_m bands; 8 * group_n covers a whole band and
+    // group_m * group_n workgroups fit the 32 CUs of an XCD even at one workgroup per CU
+    p.group_n = (p.tiles_n + kNumXcd - 1) / kNumXcd;
+    p.group_m = 32 / p.group_n;
+    if (p.group_m > p.tiles_m) p.group_m = p.tiles_m;
+    BEAM_HIP(ks->launch[dtype][kEpiLnFused][c.pipeline](
+        p, dim3((unsigned)band_block_grid(p.tiles_m, p.group_m, p.group_n), 1, 1), st));
+    return BEAM_OK;
+  }
+  {
+    std::lock_guard<std::mutex> lk(g_ln_mu);
+    g_ln_geometry.erase(ws);  // no fused launch is pending on this workspace any more
+  }
   p.ws = (float*)ws;
   p.stats = (float*)((char*)ws + align_up((size_t)M * N * sizeof(float), 256));
-  // K == 0: the kernel runs with an empty K range and produces x = 0, i.e. y = beta.
   BEAM_HIP(ks->launch[dtype][kEpiLnStats][c.pipeline](p, dim3((unsigned)(p.tiles_m * p.tiles_n), 1, 1), st));
   BEAM_HIP(launch_ln_apply(p.ws, p.stats, gamma, beta, Y, M, N, p.tiles_n, c.block_n, eps, dtype, st));
+  return BEAM_OK;
+}
+
+int beam_gemmrc_ln(const void* A, const void* B, const void* gamma, const void* beta, float eps, void* Y,
+                   int M, int N, int K, int dtype, const beam_tile_cfg* cfg, void* ws, size_t ws_bytes,
+                   void* stream) {
+  return beam_gemmrc_ln_ex(A, B, gamma, beta, eps, Y, M, N, K, dtype, cfg, BEAM_LN_AUTO, ws, ws_bytes, stream);
+}
+
+int beam_gemmrc_ln_workspace_reset(const void* ws) {
+  std::lock_guard<std::mutex> lk(g_ln_mu);
+  g_ln_geometry.erase(ws);
+  return BEAM_OK;
+}
+
+int beam_set_ln_spin_limit(int polls) {
+  if (polls < 0) return fail(BEAM_ERR_INVALID, "spin limit must be >= 0");
+  g_ln_spin_limit.store(polls);
+  return BEAM_OK;
+}
+
+int beam_gemmrc_ln_timed_out(const void* ws, void* stream, int* timed_out) {
+  if (!ws || !timed_out) return fail(BEAM_ERR_INVALID, "null argument");
+  BEAM_HIP(hipStreamSynchronize((hipStream_t)stream));
+  {
+    std::lock_guard<std::mutex> lk(g_ln_mu);
+    if (g_ln_geometry.find(ws) == g_ln_geometry.end()) {  // no fused launch has used this workspace
+      *timed_out = 0;
+      return BEAM_OK;
+    }
+  }
+  int flag = 0;
+  BEAM_HIP(hipMemcpy(&flag, ws, sizeof(int), hipMemcpyDeviceToHost));
+  *timed_out = flag;
   return BEAM_OK;
 }
 
@@ -548,5 +665,16 @@ int beam_dbg_tile_of_workgroup(int wg, int tiles_m, int tiles_n, int group_m, in
 }
 
 int beam_dbg_lds_offset(int row, int chunk) { return lds_offset(row, chunk); }
+
+int beam_dbg_band_block_tile(int wg, int tiles_m, int tiles_n, int gb, int gc, int* tm, int* tn) {
+  if (tiles_m < 1 || tiles_n < 1 || gb < 1 || gc < 1 || wg < 0 || wg >= band_block_grid(tiles_m, gb, gc) || !tm || !tn)
+    return fail(BEAM_ERR_INVALID, "bad band-block query");
+  const TileCoord t = band_block_tile(wg, tiles_m, tiles_n, gb, gc);
+  *tm = t.tm;
+  *tn = t.tn;
+  return BEAM_OK;
+}
+
+int beam_dbg_band_block_grid(int tiles_m, int gb, int gc) { return band_block_grid(tiles_m, gb, gc); }
 
 }  // extern "C"

@@ -71,6 +71,7 @@ enum Epilogue : int {
   kEpiStore = 0,    // round to 16-bit and store C
   kEpiPartial = 1,  // store fp32 partial sums of this K slice into the split-K workspace
   kEpiLnStats = 2,  // store fp32 X and per-(row, column-tile) mean / M2 for LayerNorm
+  kEpiLnFused = 3,  // LayerNorm in the epilogue: tiles of a row band exchange statistics only
 };
 
 struct GemmParams {
@@ -79,10 +80,18 @@ struct GemmParams {
   void* C;       // 16-bit [M][N]                                  (kEpiStore)
   float* ws;     // fp32 [splits][M][N] (kEpiPartial) or fp32 [M][N] (kEpiLnStats)
   float* stats;  // fp32 [M][tiles_n][2] = (mean, M2) over the tile's columns (kEpiLnStats)
+                 // fp32 [tiles_m][tiles_n][BM][2], every M2 = -1 ("not published") on entry (kEpiLnFused)
+  float* next_stats;    // the statistics set the NEXT launch on this workspace will use: reset here
+  int* timeout_flag;    // set to 1 if a bounded wait ran out (never expected)        (kEpiLnFused)
+  const void* gamma;    // 16-bit [N]                                                   (kEpiLnFused)
+  const void* beta;     // 16-bit [N]
+  float eps;
+  int spin_limit;       // polls of one statistics slot before giving up
   int M, N, K;
   int tiles_m, tiles_n;
   int k_slice;   // K elements per blockIdx.z slice, a multiple of kBK
-  int group_m;   // rasterisation group height in tiles
+  int group_m;   // rasterisation group height in tiles (fused LayerNorm: bands per band group)
+  int group_n;   // fused LayerNorm: columns of a band group owned by one XCD
 };
 
 // Buffer descriptor word 3 for gfx9-family raw buffers: 32-bit data format, no swizzle.
@@ -159,7 +168,11 @@ struct GemmTile {
     const int wm = wave % WAVES_M;
     const int wn = wave / WAVES_M;
 
-    const TileCoord tc = tile_of_workgroup(blockIdx.x, p.tiles_m, p.tiles_n, p.group_m);
+    // Fused LayerNorm uses the band-block order, which keeps the workgroups that must exchange
+    // statistics resident together; its grid is padded and the surplus workgroups leave here.
+    const TileCoord tc = (EPI == kEpiLnFused) ? band_block_tile(blockIdx.x, p.tiles_m, p.tiles_n, p.group_m, p.group_n)
+                                              : tile_of_workgroup(blockIdx.x, p.tiles_m, p.tiles_n, p.group_m);
+    if (EPI == kEpiLnFused && tc.tm < 0) return;
     const int row0 = tc.tm * BM;
     const int col0 = tc.tn * BN;
     const int M = p.M, N = p.N, K = p.K;
@@ -343,6 +356,89 @@ struct GemmTile {
         for (int j = 0; j < FN; ++j) acc[i][j] = Traits::mfma(fb1[j], fa[i], acc[i][j]);
     }
 
+    // ---- per-row statistics of the tile (LayerNorm epilogues) -------------------------------
+    // A row's BN columns are spread over WAVES_N wavefronts x 4 lane groups (lane >> 4); every lane
+    // reduces its own FN*4 values to (mean, M2) in registers, drops the pair into LDS, and one
+    // thread per row merges the 4*WAVES_N pairs in a fixed order with Chan's update: no cross-lane
+    // shuffles (they go through the LDS crossbar one at a time) and no cancellation.
+    // Result: row_stats[rl] = (mean, M2) over the tile's valid columns, for rl in [0, BM).
+    auto tile_row_stats = [&](float* part /* [BM][4*WAVES_N][2] */, float* row_stats /* [BM][2] */) {
+      constexpr int SLOTS = 4 * WAVES_N;
+      const int n_lane0 = col0 + wn * TN + 4 * (lane >> 4);  // first column of this lane
+      const bool full = (col0 + BN <= N);
+#pragma unroll
+      for (int i = 0; i < FM; ++i) {
+        float s = 0.0f, m2 = 0.0f, mean;
+        if (full) {
+#pragma unroll
+          for (int j = 0; j < FN; ++j)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) s += acc[i][j][e];
+          mean = s * (1.0f / (float)(FN * 4));
+#pragma unroll
+          for (int j = 0; j < FN; ++j)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const float d = acc[i][j][e] - mean;
+              m2 += d * d;
+            }
+        } else {
+          int cnt = 0;
+#pragma unroll
+          for (int j = 0; j < FN; ++j)
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              if (n_lane0 + j * 16 + e < N) {
+                s += acc[i][j][e];
+                ++cnt;
+              }
+          mean = cnt > 0 ? s / (float)cnt : 0.0f;
+#pragma unroll
+          for (int j = 0; j < FN; ++j)
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              if (n_lane0 + j * 16 + e < N) {
+                const float d = acc[i][j][e] - mean;
+                m2 += d * d;
+              }
+        }
+        const int rl = wm * TM + i * 16 + (lane & 15);
+        const int slot = wn * 4 + (lane >> 4);
+        part[(rl * SLOTS + slot) * 2 + 0] = mean;
+        part[(rl * SLOTS + slot) * 2 + 1] = m2;
+      }
+      __syncthreads();
+      for (int rl = tid; rl < BM; rl += NT) {
+        float mean = 0.0f, m2 = 0.0f, n_acc = 0.0f;
+#pragma unroll
+        for (int slot = 0; slot < SLOTS; ++slot) {
+          // valid columns of this (wavefront, lane group): 4 per 16-wide block, clipped at N
+          int cnt = FN * 4;
+          if (!full) {
+            cnt = 0;
+            const int n0 = col0 + (slot >> 2) * TN + 4 * (slot & 3);
+#pragma unroll
+            for (int j = 0; j < FN; ++j) {
+              int c = N - (n0 + j * 16);
+              cnt += c < 0 ? 0 : (c > 4 ? 4 : c);
+            }
+            if (cnt == 0) continue;
+          }
+          const float mw = part[(rl * SLOTS + slot) * 2 + 0];
+          const float qw = part[(rl * SLOTS + slot) * 2 + 1];
+          const float nb = (float)cnt;
+          const float tot = n_acc + nb;
+          const float delta = mw - mean;
+          mean += delta * (nb / tot);
+          m2 += qw + delta * delta * (n_acc * nb / tot);
+          n_acc = tot;
+        }
+        row_stats[rl * 2 + 0] = mean;
+        row_stats[rl * 2 + 1] = m2;
+      }
+      __syncthreads();  // `part` may be reused by the caller from here on
+    };
+
     // ---- epilogue ---------------------------------------------------------------------
     // acc[i][j][e]: row m = row0 + wm*TM + i*16 + (lane & 15),
     //               col n = col0 + wn*TN + j*16 + 4*(lane>>4) + e.
@@ -372,71 +468,137 @@ struct GemmTile {
           }
         }
       }
+    } else if (EPI == kEpiLnFused) {
+      // gamma / beta for this lane's columns: issued now, consumed in step 5
+      const T* gamma = (const T*)p.gamma;
+      const T* beta = (const T*)p.beta;
+      vec4 gv[FN], bv[FN];
+#pragma unroll
+      for (int j = 0; j < FN; ++j) {
+        const int n = n_base + j * 16;
+        if (vec_ok && n + 3 < N) {
+          gv[j] = *(const vec4*)(gamma + n);
+          bv[j] = *(const vec4*)(beta + n);
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const int nn = (n + e < N) ? n + e : N - 1;
+            gv[j][e] = gamma[nn];
+            bv[j][e] = beta[nn];
+          }
+        }
+      }
+      // 1. per-row (mean, M2) over this tile's columns
+      __syncthreads();            // every LDS slot is dead; reuse the space
+      float* red = (float*)smem;   // [BM][2] tile statistics, later (mean, rstd) of the whole row
+      float* part = red + BM * 2;  // [BM][4*WAVES_N][2], then reused as `gathered`
+      tile_row_stats(part, red);
+      // 2. publish the tile's statistics: stats[band][tile_n][row] = (mean, M2) as one 8-byte
+      //    device-scope atomic store.  Such stores go straight through the XCD-private L2 to memory
+      //    and the device-scope loads below come straight from it, so the exchange needs no cache-wide
+      //    write-back / invalidate (a __threadfence() per workgroup costs tens of microseconds here).
+      //    A slot whose M2 is negative has not been published yet: M2 of real data is never negative.
+      const size_t my_slot = ((size_t)tc.tm * p.tiles_n + tc.tn) * BM;
+      unsigned long long* my_stats = (unsigned long long*)p.stats + my_slot;
+      unsigned long long* my_next = (unsigned long long*)p.next_stats + my_slot;
+      // (tile_row_stats left row rl's pair with the thread that publishes it: same rl = tid stride)
+      for (int rl = tid; rl < BM; rl += NT) {
+        const float mean = red[rl * 2 + 0];
+        float m2 = red[rl * 2 + 1];
+        m2 = fmaxf(m2, 0.0f);  // rounding can leave -0.0 or a tiny negative: keep the "published" sign
+        const unsigned long long pair =
+            (unsigned long long)__float_as_uint(mean) | ((unsigned long long)__float_as_uint(m2) << 32);
+        __hip_atomic_store(my_stats + rl, pair, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        // the other set is the one the next launch on this workspace reads: mark it unpublished
+        const unsigned long long unpublished = (unsigned long long)__float_as_uint(-1.0f) << 32;
+        __hip_atomic_store(my_next + rl, unpublished, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+      // 3. gather the band's statistics into LDS: one 8-byte device-scope load per (tile, row), all in
+      //    flight together, each repeated (bounded) until its tile has published
+      float* gathered = part;  // [tiles_n][BM][2]; tiles_n <= 64 keeps it within the LDS the kernel owns
+      const unsigned long long* band_stats = (const unsigned long long*)p.stats + (size_t)tc.tm * p.tiles_n * BM;
+      const int n_slots = p.tiles_n * BM;
+      for (int q0 = tid; q0 < n_slots; q0 += 8 * NT) {
+        unsigned long long v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {  // eight loads in flight per thread before the first is examined
+          const int q = q0 + u * NT;
+          v[u] = __hip_atomic_load(band_stats + (q < n_slots ? q : q0), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          const int q = q0 + u * NT;
+          if (q >= n_slots) break;
+          int polls = 0;
+          while ((long long)v[u] < 0) {  // sign bit of M2: not published yet
+            if (++polls > p.spin_limit) {
+              *p.timeout_flag = 1;
+              break;
+            }
+            __builtin_amdgcn_s_sleep(4);
+            v[u] = __hip_atomic_load(band_stats + q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          }
+          ((unsigned long long*)gathered)[q] = v[u];
+        }
+      }
+      __syncthreads();
+      // 4. merge in tile order -> (mean, rstd) per row
+      for (int rl = tid; rl < BM; rl += NT) {
+        float mean = 0.0f, m2 = 0.0f, n_acc = 0.0f;
+        for (int t = 0; t < p.tiles_n; ++t) {
+          int cw = N - t * BN;
+          cw = cw > BN ? BN : cw;
+          const float mw = gathered[((size_t)t * BM + rl) * 2 + 0];
+          const float qw = gathered[((size_t)t * BM + rl) * 2 + 1];
+          const float nb = (float)cw;
+          const float tot = n_acc + nb;
+          const float delta = mw - mean;
+          mean += delta * (nb / tot);
+          m2 += qw + delta * delta * (n_acc * nb / tot);
+          n_acc = tot;
+        }
+        red[rl * 2 + 0] = mean;
+        red[rl * 2 + 1] = 1.0f / sqrtf(m2 / (float)N + p.eps);
+      }
+      __syncthreads();
+      // 5. normalise the accumulators and store Y
+      T* Y = (T*)p.C;
+#pragma unroll
+      for (int i = 0; i < FM; ++i) {
+        const int m = m_base + i * 16;
+        if (m >= M) continue;
+        const int rl = wm * TM + i * 16 + (lane & 15);
+        const float mean = red[rl * 2 + 0];
+        const float rstd = red[rl * 2 + 1];
+        T* yrow = Y + (size_t)m * N;
+#pragma unroll
+        for (int j = 0; j < FN; ++j) {
+          const int n = n_base + j * 16;
+          vec4 v;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) v[e] = (T)((acc[i][j][e] - mean) * rstd * (float)gv[j][e] + (float)bv[j][e]);
+          if (vec_ok && n + 3 < N) {
+            *(vec4*)(yrow + n) = v;
+          } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              if (n + e < N) yrow[n + e] = v[e];
+          }
+        }
+      }
     } else {
       if (EPI == kEpiLnStats) {
         // Per-row statistics over the columns this workgroup owns, from the fp32 accumulators.
-        // A row's TN columns of one wavefront sit in four lanes (l, l^16, l^32, l^48): reduce in
-        // registers, swap twice across the lane groups, then combine the WAVES_N wavefronts via
-        // LDS with Chan's pairwise update, so no precision is lost to cancellation.
-        __syncthreads();            // every LDS slot is dead; reuse the space for the exchange
-        float* red = (float*)smem;  // [BM][WAVES_N][2]
-        const int cols_here = (N - col0) < BN ? (N - col0) : BN;
-#pragma unroll
-        for (int i = 0; i < FM; ++i) {
-          float s = 0.0f;
-          int cnt = 0;
-#pragma unroll
-          for (int j = 0; j < FN; ++j)
-#pragma unroll
-            for (int e = 0; e < 4; ++e)
-              if (n_base + j * 16 + e < N) {
-                s += acc[i][j][e];
-                ++cnt;
-              }
-          s += __shfl_xor(s, 16);
-          s += __shfl_xor(s, 32);
-          cnt += __shfl_xor(cnt, 16);
-          cnt += __shfl_xor(cnt, 32);
-          const float mean = cnt > 0 ? s / (float)cnt : 0.0f;
-          float m2 = 0.0f;
-#pragma unroll
-          for (int j = 0; j < FN; ++j)
-#pragma unroll
-            for (int e = 0; e < 4; ++e)
-              if (n_base + j * 16 + e < N) {
-                const float d = acc[i][j][e] - mean;
-                m2 += d * d;
-              }
-          m2 += __shfl_xor(m2, 16);
-          m2 += __shfl_xor(m2, 32);
-          if (lane < 16) {
-            const int rl = wm * TM + i * 16 + lane;
-            red[(rl * WAVES_N + wn) * 2 + 0] = mean;
-            red[(rl * WAVES_N + wn) * 2 + 1] = m2;
-          }
-        }
-        __syncthreads();
+        __syncthreads();  // every LDS slot is dead; reuse the space
+        float* row_stats = (float*)smem;   // [BM][2]
+        float* part = row_stats + BM * 2;  // [BM][4*WAVES_N][2]
+        tile_row_stats(part, row_stats);
         for (int rl = tid; rl < BM; rl += NT) {
           const int m = row0 + rl;
           if (m >= M) continue;
-          float mean = 0.0f, m2 = 0.0f, n_acc = 0.0f;
-#pragma unroll
-          for (int w = 0; w < WAVES_N; ++w) {
-            int cw = cols_here - w * TN;
-            cw = cw < 0 ? 0 : (cw > TN ? TN : cw);
-            if (cw == 0) continue;
-            const float mw = red[(rl * WAVES_N + w) * 2 + 0];
-            const float qw = red[(rl * WAVES_N + w) * 2 + 1];
-            const float nb = (float)cw;
-            const float tot = n_acc + nb;
-            const float delta = mw - mean;
-            mean += delta * (nb / tot);
-            m2 += qw + delta * delta * (n_acc * nb / tot);
-            n_acc = tot;
-          }
           float* st = p.stats + ((size_t)m * p.tiles_n + tc.tn) * 2;
-          st[0] = mean;
-          st[1] = m2;
+          st[0] = row_stats[rl * 2 + 0];
+          st[1] = row_stats[rl * 2 + 1];
         }
       }
       // fp32 tile: split-K partial sums of this slice, or X for the normalisation pass.

@@ -16,7 +16,7 @@ struct KernelSet {
   int threads;
   int lds_bytes;
   int lds_bytes_shallow;
-  GemmLauncher launch[2][3][2];  // [dtype][epilogue][pipeline: 0 = 3 A + 2 B slots, 1 = 2 + 2]
+  GemmLauncher launch[2][4][2];  // [dtype][epilogue][pipeline: 0 = 3 A + 2 B slots, 1 = 2 + 2]
 };
 
 template <typename T, int BM, int BN, int WVM, int WVN, int EPI, int AST, int BST>
@@ -51,7 +51,9 @@ KernelSet make_kernel_set() {
   k.launch[D][kEpiPartial][0] = launch_gemm<T, BM, BN, WVM, WVN, kEpiPartial, 3, 2>; \
   k.launch[D][kEpiPartial][1] = launch_gemm<T, BM, BN, WVM, WVN, kEpiPartial, 2, 2>; \
   k.launch[D][kEpiLnStats][0] = launch_gemm<T, BM, BN, WVM, WVN, kEpiLnStats, 3, 2>; \
-  k.launch[D][kEpiLnStats][1] = launch_gemm<T, BM, BN, WVM, WVN, kEpiLnStats, 2, 2>;
+  k.launch[D][kEpiLnStats][1] = launch_gemm<T, BM, BN, WVM, WVN, kEpiLnStats, 2, 2>; \
+  k.launch[D][kEpiLnFused][0] = launch_gemm<T, BM, BN, WVM, WVN, kEpiLnFused, 3, 2>; \
+  k.launch[D][kEpiLnFused][1] = launch_gemm<T, BM, BN, WVM, WVN, kEpiLnFused, 2, 2>;
   BEAM_FILL(0, _Float16)
   BEAM_FILL(1, __bf16)
 #undef BEAM_FILL

@@ -67,6 +67,33 @@ BEAM_HD TileCoord grouped_tile(int pid, int tiles_m, int tiles_n, int group_m) {
   return t;
 }
 
+// Order for kernels whose tiles of one row band cooperate (fused LayerNorm): a workgroup may wait for
+// the other column tiles of its band, so all of them must be resident at the same time.  The grid is
+// cut into band groups of `gb` bands; inside a band group XCD x owns the `gc` columns
+// [x*gc, (x+1)*gc) of every band, i.e. a gb x gc block of tiles (good L2 reuse of both operands), and
+// 8*gc >= tiles_n, so one band group is exactly what the 8 XCDs hold at once (gb*gc <= CUs per XCD).
+// Every XCD walks the band groups in the same order, and the hardware dispatches the workgroups of an
+// XCD in id order: the earliest unfinished band group is always fully resident, hence no deadlock.
+// The grid is padded (8 * band_groups * gb * gc workgroups); ids that fall outside the tile grid
+// return tm = -1 and the workgroup exits at once.
+BEAM_HD TileCoord band_block_tile(int wg, int tiles_m, int tiles_n, int gb, int gc) {
+  const int xcd = wg % kNumXcd;
+  const int local = wg / kNumXcd;
+  const int per_group = gb * gc;
+  const int bg = local / per_group;
+  const int within = local - bg * per_group;
+  TileCoord t;
+  t.tm = bg * gb + within % gb;
+  t.tn = xcd * gc + within / gb;
+  if (t.tm >= tiles_m || t.tn >= tiles_n) t.tm = -1;
+  return t;
+}
+
+// Number of workgroups of that padded grid.
+BEAM_HD int band_block_grid(int tiles_m, int gb, int gc) {
+  return kNumXcd * ((tiles_m + gb - 1) / gb) * gb * gc;
+}
+
 BEAM_HD TileCoord tile_of_workgroup(int wg, int tiles_m, int tiles_n, int group_m) {
   return grouped_tile(xcd_remap(wg, tiles_m * tiles_n), tiles_m, tiles_n, group_m);
 }

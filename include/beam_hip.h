@@ -110,6 +110,33 @@ int beam_gemmrc_ln(const void* A, const void* B, const void* gamma, const void* 
                    void* Y, int M, int N, int K, int dtype, const beam_tile_cfg* cfg, void* ws,
                    size_t ws_bytes, void* stream);
 
+/* The two ways the library computes it, selectable for testing and tuning:
+ *   BEAM_LN_FUSED   one kernel: each workgroup keeps its fp32 accumulators in registers, the column
+ *                   tiles of a row band exchange per-row (mean, M2) pairs through the workspace and a
+ *                   per-band arrival counter, then every workgroup normalises and stores its own tile.
+ *                   Needs all column tiles of a band resident at once: N / block_n <= 64.
+ *   BEAM_LN_TWOPASS the GEMM kernel stores fp32 X and per-tile statistics, a second kernel normalises.
+ *   BEAM_LN_AUTO    fused when it applies, else two-pass (what beam_gemmrc_ln does). */
+typedef enum beam_ln_mode { BEAM_LN_AUTO = 0, BEAM_LN_TWOPASS = 1, BEAM_LN_FUSED = 2 } beam_ln_mode;
+size_t beam_gemmrc_ln_workspace_bytes_ex(int M, int N, const beam_tile_cfg* cfg, int mode);
+int beam_gemmrc_ln_ex(const void* A, const void* B, const void* gamma, const void* beta, float eps,
+                      void* Y, int M, int N, int K, int dtype, const beam_tile_cfg* cfg, int mode,
+                      void* ws, size_t ws_bytes, void* stream);
+/* The fused path keeps state in its workspace between launches (each launch prepares the statistics
+ * slots of the next one), and the library remembers per workspace pointer that it did.  If anything
+ * else writes to a workspace that fused launches have used (or it is freed and the address reused),
+ * call this before the next fused launch; that launch then re-initialises the workspace itself.
+ * Launches sharing one workspace must be ordered on one stream. */
+int beam_gemmrc_ln_workspace_reset(const void* ws);
+/* Waits for `stream`, then *timed_out = 1 if a fused call on this workspace gave up waiting for a
+ * band (its output is then invalid).  Only possible if the device could not hold a whole band of
+ * workgroups at once, e.g. because another process occupied most of it. */
+int beam_gemmrc_ln_timed_out(const void* ws, void* stream, int* timed_out);
+/* Bound of that wait, in polls of the band counter (roughly a microsecond each; default 4 Mi).
+ * 0 makes every workgroup give up at once: the kernel still ends normally and the flag is set,
+ * which is how the failure path is exercised without hanging anything. */
+int beam_set_ln_spin_limit(int polls);
+
 /* ---- timing ------------------------------------------------------------------------------- */
 
 /* Which operation beam_bench times. */
@@ -167,6 +194,10 @@ int beam_host_fill_normal(void* dst_host, size_t n, int dtype, uint64_t seed, ui
 int beam_dbg_tile_of_workgroup(int wg, int tiles_m, int tiles_n, int group_m, int* tm, int* tn);
 /* Byte offset of (row, 16-byte chunk) inside an LDS stage. */
 int beam_dbg_lds_offset(int row, int chunk);
+/* Workgroup id -> tile of the padded band-block grid used by the fused GEMM+LayerNorm (tm = -1:
+ * the id is padding), and the size of that grid. */
+int beam_dbg_band_block_tile(int wg, int tiles_m, int tiles_n, int gb, int gc, int* tm, int* tn);
+int beam_dbg_band_block_grid(int tiles_m, int gb, int gc);
 
 #ifdef __cplusplus
 }

@@ -18,14 +18,15 @@ def make_ln_inputs(beamc, M, N, K, dtype, seed):
     return a, b, gamma, beta
 
 
-def run_ln(beamc, a, b, gamma, beta, dtype, eps=1e-5, config=None):
+def run_ln(beamc, a, b, gamma, beta, dtype, eps=1e-5, config=None, mode=0):
     M, N = a.shape[0], b.shape[0]
     da, db = beamc.DeviceArray.from_numpy(a, dtype), beamc.DeviceArray.from_numpy(b, dtype)
     dg, dbt = beamc.DeviceArray.from_numpy(gamma, dtype), beamc.DeviceArray.from_numpy(beta, dtype)
     y = beamc.DeviceArray((M, N), dtype)
     y.fill_bytes(0xEE)
-    beamc.gemmrc_ln(da, db, y, dg, dbt, eps=eps, config=config)
+    beamc.gemmrc_ln(da, db, y, dg, dbt, eps=eps, config=config, mode=mode)
     out = y.to_numpy()
+    assert not beamc.gemmrc_ln_timed_out()
     for x in (da, db, dg, dbt, y):
         x.free()
     return out
@@ -50,8 +51,9 @@ def test_ln_small(gpu, beamc, oracle, shape):
         ref = oracle.gemmrc_ln(a, b, g, bt, 1e-5, dtype)
         for cfg in [None, beamc.TileConfig(128, 128, 64, 64), beamc.TileConfig(64, 64, 32, 32),
                     beamc.TileConfig(256, 256, 128, 64)]:
-            got = run_ln(beamc, a, b, g, bt, dtype, config=cfg)
-            check_ln(oracle, got, ref, dtype, f"{shape} dtype {dtype} {cfg.name if cfg else 'default'}")
+            for mode in (beamc.LN_TWOPASS, beamc.LN_FUSED):
+                got = run_ln(beamc, a, b, g, bt, dtype, config=cfg, mode=mode)
+                check_ln(oracle, got, ref, dtype, f"{shape} dtype {dtype} {cfg.name if cfg else 'default'} mode {mode}")
 
 
 def test_ln_4096_cube(gpu, beamc, oracle):
@@ -59,8 +61,23 @@ def test_ln_4096_cube(gpu, beamc, oracle):
     M = N = K = 4096
     a, b, g, bt = make_ln_inputs(beamc, M, N, K, F16, 22)
     ref = oracle.gemmrc_ln(a, b, g, bt, 1e-5, F16)
-    got = run_ln(beamc, a, b, g, bt, F16)
-    check_ln(oracle, got, ref, F16, "4096^3")
+    for mode in (beamc.LN_TWOPASS, beamc.LN_FUSED):
+        got = run_ln(beamc, a, b, g, bt, F16, mode=mode)
+        check_ln(oracle, got, ref, F16, f"4096^3 mode {mode}")
+
+
+def test_ln_many_column_tiles(gpu, beamc, oracle):
+    """N = 11008 (43 column tiles of 256: one band spans two XCDs) and a 64-wide tile with 64 column
+    tiles (the most the fused path takes); beyond that AUTO falls back to two passes."""
+    for (M, N, K, cfg) in [(512, 11008, 256, None), (128, 4096, 128, beamc.TileConfig(64, 64, 32, 32)),
+                           (130, 4100, 136, beamc.TileConfig(64, 64, 32, 32))]:
+        a, b, g, bt = make_ln_inputs(beamc, M, N, K, F16, 24)
+        ref = oracle.gemmrc_ln(a, b, g, bt, 1e-5, F16)
+        got = run_ln(beamc, a, b, g, bt, F16, config=cfg, mode=beamc.LN_AUTO)
+        check_ln(oracle, got, ref, F16, f"{(M, N, K)} auto")
+    with pytest.raises(beamc.BeamError):
+        a, b, g, bt = make_ln_inputs(beamc, 64, 8192, 64, F16, 25)
+        run_ln(beamc, a, b, g, bt, F16, config=beamc.TileConfig(64, 64, 32, 32), mode=beamc.LN_FUSED)
 
 
 def test_ln_invariants(gpu, beamc, oracle):
@@ -84,3 +101,24 @@ def test_ln_invariants(gpu, beamc, oracle):
     got = run_ln(beamc, a2, b2, ones, zeros, F16)
     r = oracle.compare(got, ref, F16)
     assert r["max_abs_err"] <= 4e-3, r
+
+
+def test_ln_fused_timeout_is_reported_not_hung(gpu, beamc):
+    """With a zero poll budget every workgroup gives up waiting at once: the kernel still ends normally,
+    the flag is raised, and the next call with the normal budget is correct again."""
+    M, N, K = 512, 4096, 256
+    a, b, g_, bt = make_ln_inputs(beamc, M, N, K, F16, 26)
+    good = run_ln(beamc, a, b, g_, bt, F16, mode=beamc.LN_FUSED)
+    try:
+        assert beamc.lib.beam_set_ln_spin_limit(0) == 0
+        da, db = beamc.DeviceArray.from_numpy(a), beamc.DeviceArray.from_numpy(b)
+        dg, dbt = beamc.DeviceArray.from_numpy(g_), beamc.DeviceArray.from_numpy(bt)
+        y = beamc.DeviceArray((M, N))
+        beamc.gemmrc_ln(da, db, y, dg, dbt, mode=beamc.LN_FUSED)
+        beamc.sync()
+        assert beamc.gemmrc_ln_timed_out()
+    finally:
+        beamc.lib.beam_set_ln_spin_limit(4 << 20)
+    beamc.lib.beam_gemmrc_ln_workspace_reset(beamc._ln_workspace.ptr)
+    again = run_ln(beamc, a, b, g_, bt, F16, mode=beamc.LN_FUSED)
+    assert (again == good).all()

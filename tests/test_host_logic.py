@@ -34,6 +34,30 @@ def test_rasterisation_is_xcd_local(beamc):
         assert len(ms) == 8 and len(ns) == 4, (xcd, sorted(block))
 
 
+@pytest.mark.parametrize("tiles_m,tiles_n", [(16, 16), (32, 32), (2, 43), (5, 7), (1, 1), (3, 64), (40, 9)])
+def test_band_block_order(beamc, tiles_m, tiles_n):
+    """Padded band-block grid of the fused GEMM+LayerNorm: every tile exactly once, padding ids are
+    flagged, an XCD's share of a band group fits its 32 CUs, and the column tiles of any band sit in one
+    band group (so they are resident together)."""
+    L = beamc.lib
+    gc = (tiles_n + 7) // 8
+    gb = min(max(32 // gc, 1), tiles_m)
+    assert gb * gc <= 32 and 8 * gc >= tiles_n
+    grid = L.beam_dbg_band_block_grid(tiles_m, gb, gc)
+    seen = {}
+    for wg in range(grid):
+        a, b = ctypes.c_int(), ctypes.c_int()
+        assert L.beam_dbg_band_block_tile(wg, tiles_m, tiles_n, gb, gc, ctypes.byref(a), ctypes.byref(b)) == 0
+        if a.value < 0:
+            continue
+        assert (a.value, b.value) not in seen
+        seen[(a.value, b.value)] = wg
+    assert len(seen) == tiles_m * tiles_n
+    for band in range(tiles_m):
+        groups = {(seen[(band, tn)] // 8) // (gb * gc) for tn in range(tiles_n)}
+        assert len(groups) == 1
+
+
 def test_lds_swizzle(beamc):
     """(row, chunk) -> byte offset is a bijection on a slot, and every group of 16 lanes of a
     ds_read_b128 fragment read (16x16x32 operand: lane l reads row l%16, chunk 4*kk + l/16) hits 16
