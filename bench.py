@@ -75,10 +75,12 @@ def extra_splitk(_C):
             best_plain = (cfg.name, ms)
         if cfg.block_m * cfg.block_n > 128 * 128:
             continue
-        for s in (4, 8, 16, 32, 64):
-            ms = _C.bench(1, a, b, c, config=cfg, split_k=s, warmup=3, iters=20)
-            if ms < best_split[1]:
-                best_split = (f"{cfg.name},S={s}", ms)
+        for pipe in (0, 2):
+            pc = _C.TileConfig(cfg.block_m, cfg.block_n, cfg.wave_m, cfg.wave_n, pipe, 0)
+            for s in (4, 8, 16, 32, 64):
+                ms = _C.bench(1, a, b, c, config=pc, split_k=s, warmup=3, iters=20)
+                if ms < best_split[1]:
+                    best_split = (f"{pc.name},S={s}", ms)
     for x in (a, b, c):
         x.free()
     bytes_alg = 2.0 * (M * K + N * K + M * N)

@@ -136,7 +136,7 @@ class TileConfig:
     def name(self) -> str:
         s = f"{self.block_m}x{self.block_n}_w{self.wave_m}x{self.wave_n}"
         if self.pipeline:
-            s += "_p22"
+            s += {1: "_p22", 2: "_deep"}.get(self.pipeline, f"_p{self.pipeline}")
         if self.group_m:
             s += f"_g{self.group_m}"
         return s

@@ -134,12 +134,13 @@ class OperatorTuner:
         for cfg in _C.list_configs():
             if cfg.block_m * cfg.block_n > 128 * 128:
                 continue  # split-K is for problems with few output tiles
+            deep = _C.TileConfig(cfg.block_m, cfg.block_n, cfg.wave_m, cfg.wave_n, 2, 0)
             for s in SPLIT_FACTORS:
                 ret.append(Operator(
                     partial(_C.gemmrc_splitk_spec, shape_threadblock=[cfg.block_m, cfg.block_n],
-                            shape_warp=[cfg.wave_m, cfg.wave_n], split_k_slices=s),
-                    native={"op": 1, "config": cfg, "split_k": s},
-                    name=f"gemmrc_splitk_spec[{cfg.name},s{s}]"))
+                            shape_warp=[cfg.wave_m, cfg.wave_n], split_k_slices=s, pipeline=2),
+                    native={"op": 1, "config": deep, "split_k": s},
+                    name=f"gemmrc_splitk_spec[{deep.name},s{s}]"))
         return ret
 
     # -- cache -----------------------------------------------------------------------------

@@ -19,14 +19,24 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 // The fixed order is what makes split-K bit-reproducible (the reference delegates this to
 // CUTLASS's reduce kernel, cuda/cutlass_kernels/cutlass_gemmrc_splitk.cu:73-75).
 template <typename T>
-__global__ void __launch_bounds__(256) splitk_reduce_kernel(const float* __restrict__ ws,
-                                                             T* __restrict__ C, size_t mn, int splits) {
+__global__ void __launch_bounds__(64) splitk_reduce_kernel(const float* __restrict__ ws, T* __restrict__ C,
+                                                            size_t mn, int splits) {
   typedef typename Vec4Of<T>::type vec4;
   const size_t quads = mn / 4;
   const size_t stride = (size_t)gridDim.x * blockDim.x;
   for (size_t q = (size_t)blockIdx.x * blockDim.x + threadIdx.x; q < quads; q += stride) {
-    f32x4 s = *(const f32x4*)(ws + q * 4);
-    for (int z = 1; z < splits; ++z) s += *(const f32x4*)(ws + (size_t)z * mn + q * 4);
+    const float* src = ws + q * 4;
+    f32x4 s = *(const f32x4*)src;
+    int z = 1;
+    // eight independent loads in flight, added in slice order
+    for (; z + 8 <= splits; z += 8) {
+      f32x4 v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) v[u] = *(const f32x4*)(src + (size_t)(z + u) * mn);
+#pragma unroll
+      for (int u = 0; u < 8; ++u) s += v[u];
+    }
+    for (; z < splits; ++z) s += *(const f32x4*)(src + (size_t)z * mn);
     vec4 o;
 #pragma unroll
     for (int e = 0; e < 4; ++e) o[e] = (T)s[e];
@@ -104,15 +114,16 @@ hipError_t launch_zero_ints(int* ints, int n, hipStream_t stream) {
 
 hipError_t launch_splitk_reduce(const float* ws, void* C, size_t mn, int splits, int dtype,
                                 hipStream_t stream) {
+  // one wavefront per workgroup: even a 256 x 256 output spreads over 256 CUs
   size_t quads = (mn + 3) / 4;
-  size_t blocks = (quads + 255) / 256;
+  size_t blocks = (quads + 63) / 64;
   if (blocks < 1) blocks = 1;
-  if (blocks > 4096) blocks = 4096;
+  if (blocks > 16384) blocks = 16384;
   if (dtype == BEAM_BF16)
-    hipLaunchKernelGGL(splitk_reduce_kernel<__bf16>, dim3((unsigned)blocks), dim3(256), 0, stream, ws,
+    hipLaunchKernelGGL(splitk_reduce_kernel<__bf16>, dim3((unsigned)blocks), dim3(64), 0, stream, ws,
                        (__bf16*)C, mn, splits);
   else
-    hipLaunchKernelGGL(splitk_reduce_kernel<_Float16>, dim3((unsigned)blocks), dim3(256), 0, stream, ws,
+    hipLaunchKernelGGL(splitk_reduce_kernel<_Float16>, dim3((unsigned)blocks), dim3(64), 0, stream, ws,
                        (_Float16*)C, mn, splits);
   return hipGetLastError();
 }

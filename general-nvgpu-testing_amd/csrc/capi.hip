@@ -103,7 +103,7 @@ int resolve_cfg(const beam_tile_cfg* in, int M, int N, int K, beam_tile_cfg* out
     int rc = beam_default_config(M, N, K, out, &s);
     if (rc) return rc;
   }
-  if (out->pipeline != 0 && out->pipeline != 1) return fail(BEAM_ERR_UNSUPPORTED, "pipeline %d: 0 (3 A + 2 B LDS slots) or 1 (2 + 2)", out->pipeline);
+  if (out->pipeline < 0 || out->pipeline > 2) return fail(BEAM_ERR_UNSUPPORTED, "pipeline %d: 0 (3 A + 2 B LDS slots), 1 (2 + 2) or 2 (deep)", out->pipeline);
   if (out->group_m <= 0) out->group_m = kDefaultGroupM;
   *ks = find_set(*out);
   if (!*ks)
@@ -124,6 +124,7 @@ GemmParams base_params(const void* A, const void* B, int M, int N, int K, const 
   p.tiles_n = (N + c.block_n - 1) / c.block_n;
   p.k_slice = ((K + kBK - 1) / kBK) * kBK;
   if (p.k_slice == 0) p.k_slice = kBK;
+  p.splits = 1;
   p.group_m = c.group_m;
   return p;
 }
@@ -289,6 +290,7 @@ int beam_default_config(int M, int N, int K, beam_tile_cfg* cfg, int* split_k) {
       if (s > ktiles / 4) s = ktiles / 4;  // keep at least 4 K tiles per slice
       if (s < 1) s = 1;
     }
+    if (s > 1) cfg->pipeline = 2;  // few workgroups per CU: a long prefetch queue keeps HBM busy
     *split_k = s;
   }
   return BEAM_OK;
@@ -386,7 +388,8 @@ int beam_gemmrc_splitk(const void* A, const void* B, void* C, int M, int N, int 
   GemmParams p = base_params(A, B, M, N, K, c);
   p.ws = (float*)ws;
   p.k_slice = split_k_len(K, s);
-  BEAM_HIP(ks->launch[dtype][kEpiPartial][c.pipeline](p, dim3((unsigned)(p.tiles_m * p.tiles_n), 1, (unsigned)s), st));
+  p.splits = s;
+  BEAM_HIP(ks->launch[dtype][kEpiPartial][c.pipeline](p, dim3((unsigned)(p.tiles_m * p.tiles_n * s), 1, 1), st));
   BEAM_HIP(launch_splitk_reduce((const float*)ws, C, (size_t)M * N, s, dtype, st));
   return BEAM_OK;
 }
@@ -417,6 +420,7 @@ size_t beam_gemmrc_ln_workspace_bytes_ex(int M, int N, const beam_tile_cfg* cfg,
   beam_tile_cfg c;
   const KernelSet* ks;
   if (resolve_cfg(cfg, M, N, 64, &c, &ks)) return 0;
+  if (c.pipeline == 2) c.pipeline = 0;
   const size_t tiles_m = (size_t)(M + c.block_m - 1) / c.block_m;
   const size_t tiles_n = (size_t)(N + c.block_n - 1) / c.block_n;
   if (ln_resolve_mode(mode, c, *ks, N) == BEAM_LN_FUSED)
@@ -443,6 +447,7 @@ int beam_gemmrc_ln_ex(const void* A, const void* B, const void* gamma, const voi
   beam_tile_cfg c;
   const KernelSet* ks;
   if ((rc = resolve_cfg(cfg, M, N, K, &c, &ks))) return rc;
+  if (c.pipeline == 2) c.pipeline = 0;  // the deep pipeline exists for the store / split-K kernels only
   if (mode == BEAM_LN_FUSED && !ln_fused_applies(c, *ks, N))
     return fail(BEAM_ERR_UNSUPPORTED, "fused LayerNorm: too many column tiles for this tile shape (N=%d, block_n=%d)", N, c.block_n);
   mode = ln_resolve_mode(mode, c, *ks, N);

@@ -89,7 +89,8 @@ struct GemmParams {
   int spin_limit;       // polls of one statistics slot before giving up
   int M, N, K;
   int tiles_m, tiles_n;
-  int k_slice;   // K elements per blockIdx.z slice, a multiple of kBK
+  int k_slice;   // K elements per split-K slice, a multiple of kBK
+  int splits;    // number of K slices (1 = no split); the grid holds tiles_m * tiles_n * splits workgroups
   int group_m;   // rasterisation group height in tiles (fused LayerNorm: bands per band group)
   int group_n;   // fused LayerNorm: columns of a band group owned by one XCD
 };
@@ -118,6 +119,15 @@ __device__ __forceinline__ void bare_barrier() {
   asm volatile("" ::: "memory");
   __builtin_amdgcn_s_barrier();
   asm volatile("" ::: "memory");
+}
+
+// A-slot count of the "deep" pipeline of a tile shape: as many slots as 160 KiB of LDS hold with one
+// slot fewer for B, at most 8.  Small tiles get a long prefetch queue this way, which is what a
+// split-K workgroup (few tiles in flight per CU, every byte fetched exactly once) needs to keep HBM busy.
+constexpr int deep_a_slots(int BM, int BN) {
+  int a = 8;
+  while (a > 3 && (a * BM + (a - 1) * BN) * kRowBytes > 160 * 1024) --a;
+  return a;
 }
 
 template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, int EPI, int AST, int BST>
@@ -170,15 +180,27 @@ struct GemmTile {
 
     // Fused LayerNorm uses the band-block order, which keeps the workgroups that must exchange
     // statistics resident together; its grid is padded and the surplus workgroups leave here.
-    const TileCoord tc = (EPI == kEpiLnFused) ? band_block_tile(blockIdx.x, p.tiles_m, p.tiles_n, p.group_m, p.group_n)
-                                              : tile_of_workgroup(blockIdx.x, p.tiles_m, p.tiles_n, p.group_m);
-    if (EPI == kEpiLnFused && tc.tm < 0) return;
+    // Split-K walks (slice, tile) pairs slice by slice, and the XCD remap gives every XCD one
+    // contiguous range of pairs: the tiles that read the same K slice of A and B share an L2.
+    TileCoord tc;
+    int slice = 0;
+    if (EPI == kEpiLnFused) {
+      tc = band_block_tile(blockIdx.x, p.tiles_m, p.tiles_n, p.group_m, p.group_n);
+      if (tc.tm < 0) return;
+    } else if (p.splits > 1) {
+      const int tiles = p.tiles_m * p.tiles_n;
+      const int pid = xcd_remap(blockIdx.x, tiles * p.splits);
+      slice = pid / tiles;
+      tc = grouped_tile(pid - slice * tiles, p.tiles_m, p.tiles_n, p.group_m);
+    } else {
+      tc = tile_of_workgroup(blockIdx.x, p.tiles_m, p.tiles_n, p.group_m);
+    }
     const int row0 = tc.tm * BM;
     const int col0 = tc.tn * BN;
     const int M = p.M, N = p.N, K = p.K;
 
     // K range of this slice.
-    const int kb = blockIdx.z * p.k_slice;
+    const int kb = slice * p.k_slice;
     int klen = K - kb;
     if (klen > p.k_slice) klen = p.k_slice;
     if (klen < 0) klen = 0;
@@ -192,10 +214,10 @@ struct GemmTile {
     const int rows_b = (N - col0) < BN ? (N - col0) : BN;
     const T* a_base = (const T*)p.A + ((size_t)row0 * K + kb);
     const T* b_base = (const T*)p.B + ((size_t)col0 * K + kb);
-    const __amdgpu_buffer_rsrc_t rsrc_a =
-        make_rsrc(a_base, klen > 0 ? ((unsigned)(rows_a - 1) * K + klen) * 2u : 0u);
-    const __amdgpu_buffer_rsrc_t rsrc_b =
-        make_rsrc(b_base, klen > 0 ? ((unsigned)(rows_b - 1) * K + klen) * 2u : 0u);
+    const unsigned bytes_a = klen > 0 ? ((unsigned)(rows_a - 1) * K + klen) * 2u : 0u;
+    const unsigned bytes_b = klen > 0 ? ((unsigned)(rows_b - 1) * K + klen) * 2u : 0u;
+    const __amdgpu_buffer_rsrc_t rsrc_a = make_rsrc(a_base, bytes_a);
+    const __amdgpu_buffer_rsrc_t rsrc_b = make_rsrc(b_base, bytes_b);
 
     unsigned voff_a[LA], voff_b[LB];
 #pragma unroll
@@ -207,15 +229,19 @@ struct GemmTile {
     auto tile_koff = [&](int t) { return k_tail ? (t == 0 ? kt_full * kBK : (t - 1) * kBK) : t * kBK; };
 
     // ---- global -> LDS ------------------------------------------------------------------
-    // One buffer load (1 KiB per wavefront) of A tile t / B tile t into its slot.
+    // One buffer load (1 KiB per wavefront) of A tile t / B tile t into its slot.  Tiles past the end
+    // of the K range get an empty descriptor: the load is still issued and counted (the pipeline below
+    // has no special cases for its last iterations) but touches no memory.
     auto load_a = [&](int i, int t) {
       char* dst = smem + (t % AST) * A_BYTES + wave * 1024 + i * (NT * 16);
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (__attribute__((address_space(3))) void*)dst, 16,
+      const __amdgpu_buffer_rsrc_t r = make_rsrc(a_base, t < n_tiles ? bytes_a : 0u);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (__attribute__((address_space(3))) void*)dst, 16,
                                                (int)voff_a[i], tile_koff(t) * 2, 0, 0);
     };
     auto load_b = [&](int i, int t) {
       char* dst = smem + B_REGION + (t % BST) * B_BYTES + wave * 1024 + i * (NT * 16);
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, (__attribute__((address_space(3))) void*)dst, 16,
+      const __amdgpu_buffer_rsrc_t r = make_rsrc(b_base, t < n_tiles ? bytes_b : 0u);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (__attribute__((address_space(3))) void*)dst, 16,
                                                (int)voff_b[i], tile_koff(t) * 2, 0, 0);
     };
     // The short tile goes through registers so that chunks at or past `kvalid` are zero-filled.
@@ -278,10 +304,8 @@ struct GemmTile {
     // One pipeline step: the MFMAs of the step whose fragments are in (fa, fb_cur) and, row by
     // row, the LDS reads of the next step's fragments (A in place, B into fb_nxt) from (sa, sb)
     // plus this row's share of the tile's buffer loads.
-    //   ISSUE: 2 = A and B loads, 1 = B loads only, 0 = none;  ROW0: first row index of the step.
-    auto step = [&](const char* sa, const char* sb, vec8(&fb_cur)[FN], vec8(&fb_nxt)[FN], int h, auto issue_tag,
-                    auto row0_tag) {
-      constexpr int ISSUE = decltype(issue_tag)::value;
+    //   ROW0: index of the step's first row inside the tile (the loads are dealt out row by row).
+    auto step = [&](const char* sa, const char* sb, vec8(&fb_cur)[FN], vec8(&fb_nxt)[FN], int h, auto row0_tag) {
       constexpr int ROW0 = decltype(row0_tag)::value;
 #pragma unroll
       for (int i = 0; i < FM; ++i) {
@@ -290,13 +314,11 @@ struct GemmTile {
         fa[i] = *(const vec8*)(sa + i * 16 * kRowBytes);
 #pragma unroll
         for (int j = i * FN / FM; j < (i + 1) * FN / FM; ++j) fb_nxt[j] = *(const vec8*)(sb + j * 16 * kRowBytes);
-        if (ISSUE) {
 #pragma unroll
-          for (int u = 0; u < PER_ROW; ++u) {
-            const int l = (ROW0 + i) * PER_ROW + u;  // B first: it is needed one tile sooner
-            if (l < LB) load_b(l, h + BST - 1);
-            else if (l < LOADS && ISSUE == 2) load_a(l - LB, h + AST - 1);
-          }
+        for (int u = 0; u < PER_ROW; ++u) {
+          const int l = (ROW0 + i) * PER_ROW + u;  // B first: it is needed one tile sooner
+          if (l < LB) load_b(l, h + BST - 1);
+          else if (l < LOADS) load_a(l - LB, h + AST - 1);
         }
       }
       // Scheduling pipeline for the compiler: per row, FN MFMAs with the row's LDS reads spread
@@ -311,44 +333,39 @@ struct GemmTile {
           __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // DS read
         }
         if (FN - G * R > 0) __builtin_amdgcn_sched_group_barrier(0x008, FN - G * R, 0);
-        if (ISSUE) __builtin_amdgcn_sched_group_barrier(0x020, PER_ROW, 0);  // VMEM read
+        __builtin_amdgcn_sched_group_barrier(0x020, PER_ROW, 0);  // VMEM read
       }
     };
 
     // One K tile h: make it visible to every wavefront, then two steps.  Step 0 multiplies the
     // second half of tile h-1 while reading the first half of tile h; step 1 multiplies the first
     // half of tile h while reading its second half.
-    auto tile_body = [&](int h, auto issue_tag, auto wait_tag) {
-      constexpr int WAITN = decltype(wait_tag)::value;
-      wait_vm_and_lds<WAITN>();  // my fills of tile h have landed; my reads of tile h-1 are done
-      bare_barrier();            // ... and so have everyone else's: the slots of tile h-1 are free
+    auto tile_body = [&](int h) {
+      wait_vm_and_lds<WAIT_STEADY>();  // my fills of tile h have landed; my reads of tile h-1 are done
+      bare_barrier();                  // ... and so have everyone else's: the slots of tile h-1 are free
       const char* sa = smem + (h % AST) * A_BYTES + a_wave_off;
       const char* sb = smem + B_REGION + (h % BST) * B_BYTES + b_wave_off;
-      step(sa + frag_off[0], sb + frag_off[0], fb1, fb0, h, issue_tag, std::integral_constant<int, 0>{});
-      step(sa + frag_off[1], sb + frag_off[1], fb0, fb1, h, issue_tag, std::integral_constant<int, FM>{});
+      step(sa + frag_off[0], sb + frag_off[0], fb1, fb0, h, std::integral_constant<int, 0>{});
+      step(sa + frag_off[1], sb + frag_off[1], fb0, fb1, h, std::integral_constant<int, FM>{});
     };
 
     if (n_tiles > 0) {
-      // Prologue: A tiles 0 .. AST-2 and B tiles 0 .. BST-2.
+      // Prologue: A tiles 0 .. AST-2 and B tiles 0 .. BST-2, oldest first (tile 0 is what the first
+      // wait below is about).  A short tile 0 goes through registers instead.
       if (k_tail) fill_short_tile(k_tail);
 #pragma unroll
       for (int s = 0; s < AST - 1; ++s) {
-        if (s < n_tiles && !(s == 0 && k_tail)) {
+        if (!(s == 0 && k_tail)) {
 #pragma unroll
           for (int i = 0; i < LA; ++i) load_a(i, s);
         }
-        if (s < BST - 1 && s < n_tiles && !(s == 0 && k_tail)) {
+        if (s < BST - 1 && !(s == 0 && k_tail)) {
 #pragma unroll
           for (int i = 0; i < LB; ++i) load_b(i, s);
         }
       }
-      wait_vm_and_lds<0>();
-      int h = 0;
-      for (; h < n_tiles - (AST - 1); ++h)
-        tile_body(h, std::integral_constant<int, 2>{}, std::integral_constant<int, WAIT_STEADY>{});
-      for (; h < n_tiles - (BST - 1); ++h)
-        tile_body(h, std::integral_constant<int, 1>{}, std::integral_constant<int, WAIT_STEADY>{});
-      for (; h < n_tiles; ++h) tile_body(h, std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{});
+      for (int h = 0; h < n_tiles; ++h) tile_body(h);
+      wait_vm_and_lds<0>();  // the empty fills of the last iterations must be gone before LDS is reused
       // Drain: the second half of the last tile is in (fa, fb1).
 #pragma unroll
       for (int i = 0; i < FM; ++i)
@@ -602,7 +619,7 @@ struct GemmTile {
         }
       }
       // fp32 tile: split-K partial sums of this slice, or X for the normalisation pass.
-      float* W = p.ws + (EPI == kEpiPartial ? (size_t)blockIdx.z * M * N : (size_t)0);
+      float* W = p.ws + (EPI == kEpiPartial ? (size_t)slice * M * N : (size_t)0);
 #pragma unroll
       for (int i = 0; i < FM; ++i) {
         const int m = m_base + i * 16;

@@ -16,7 +16,9 @@ struct KernelSet {
   int threads;
   int lds_bytes;
   int lds_bytes_shallow;
-  GemmLauncher launch[2][4][2];  // [dtype][epilogue][pipeline: 0 = 3 A + 2 B slots, 1 = 2 + 2]
+  int lds_bytes_deep;
+  // [dtype][epilogue][pipeline: 0 = 3 A + 2 B slots, 1 = 2 + 2, 2 = deep (store / partial only)]
+  GemmLauncher launch[2][4][3];
 };
 
 template <typename T, int BM, int BN, int WVM, int WVN, int EPI, int AST, int BST>
@@ -45,11 +47,17 @@ KernelSet make_kernel_set() {
   k.threads = WVM * WVN * 64;
   k.lds_bytes = GemmTile<_Float16, BM, BN, WVM, WVN, kEpiStore, 3, 2>::LDS_BYTES;
   k.lds_bytes_shallow = GemmTile<_Float16, BM, BN, WVM, WVN, kEpiStore, 2, 2>::LDS_BYTES;
+  constexpr int DA = deep_a_slots(BM, BN);
+  k.lds_bytes_deep = GemmTile<_Float16, BM, BN, WVM, WVN, kEpiStore, DA, DA - 1>::LDS_BYTES;
 #define BEAM_FILL(D, T)                                                             \
   k.launch[D][kEpiStore][0] = launch_gemm<T, BM, BN, WVM, WVN, kEpiStore, 3, 2>;     \
   k.launch[D][kEpiStore][1] = launch_gemm<T, BM, BN, WVM, WVN, kEpiStore, 2, 2>;     \
+  k.launch[D][kEpiStore][2] = launch_gemm<T, BM, BN, WVM, WVN, kEpiStore, DA, DA - 1>; \
   k.launch[D][kEpiPartial][0] = launch_gemm<T, BM, BN, WVM, WVN, kEpiPartial, 3, 2>; \
   k.launch[D][kEpiPartial][1] = launch_gemm<T, BM, BN, WVM, WVN, kEpiPartial, 2, 2>; \
+  k.launch[D][kEpiPartial][2] = launch_gemm<T, BM, BN, WVM, WVN, kEpiPartial, DA, DA - 1>; \
+  k.launch[D][kEpiLnStats][2] = nullptr;                                               \
+  k.launch[D][kEpiLnFused][2] = nullptr;                                               \
   k.launch[D][kEpiLnStats][0] = launch_gemm<T, BM, BN, WVM, WVN, kEpiLnStats, 3, 2>; \
   k.launch[D][kEpiLnStats][1] = launch_gemm<T, BM, BN, WVM, WVN, kEpiLnStats, 2, 2>; \
   k.launch[D][kEpiLnFused][0] = launch_gemm<T, BM, BN, WVM, WVN, kEpiLnFused, 3, 2>; \

@@ -37,7 +37,8 @@ typedef enum beam_dtype { BEAM_F16 = 0, BEAM_BF16 = 1 } beam_dtype;
 typedef struct beam_tile_cfg {
   int block_m, block_n; /* workgroup tile of C ("shape_threadblock")                          */
   int wave_m, wave_n;   /* wavefront tile ("shape_warp"); block/wave = wavefront grid         */
-  int pipeline;         /* LDS slots per operand: 0 = 3 for A + 2 for B (deep), 1 = 2 + 2      */
+  int pipeline;         /* LDS slots per operand: 0 = 3 for A + 2 for B, 1 = 2 + 2,             */
+                        /* 2 = as many as fit 160 KiB, up to 8 + 7 (small tiles, split-K)       */
   int group_m;          /* rasterisation group height in tiles; 0 = library default           */
 } beam_tile_cfg;
 

@@ -46,6 +46,7 @@ def all_configs(beamc):
     for cfg in beamc.list_configs():
         out.append(cfg)
         out.append(beamc.TileConfig(cfg.block_m, cfg.block_n, cfg.wave_m, cfg.wave_n, 1, 0))
+        out.append(beamc.TileConfig(cfg.block_m, cfg.block_n, cfg.wave_m, cfg.wave_n, 2, 0))
     return out
 
 

@@ -7,14 +7,14 @@ from test_gpu_gemm import F16, BF16, assert_close
 pytestmark = pytest.mark.gpu
 
 
-def run_splitk(beamc, a_bits, b_bits, dtype, tb, wp, s):
+def run_splitk(beamc, a_bits, b_bits, dtype, tb, wp, s, pipeline=0):
     M, K = a_bits.shape
     N = b_bits.shape[0]
     a = beamc.DeviceArray.from_numpy(a_bits, dtype)
     b = beamc.DeviceArray.from_numpy(b_bits, dtype)
     c = beamc.DeviceArray((M, N), dtype)
     c.fill_bytes(0xEE)
-    beamc.gemmrc_splitk_spec(a, b, c, shape_threadblock=tb, shape_warp=wp, split_k_slices=s)
+    beamc.gemmrc_splitk_spec(a, b, c, shape_threadblock=tb, shape_warp=wp, split_k_slices=s, pipeline=pipeline)
     out = c.to_numpy()
     for x in (a, b, c):
         x.free()
@@ -35,8 +35,9 @@ def test_splitk_configs(gpu, beamc, oracle, shape):
     assert r["max_abs_ref"] < 65504                                # inside fp16 range
     for tb, wp in TILES:
         for s in (4, 8, 16, 32, 64):
-            got = run_splitk(beamc, a, b, F16, tb, wp, s)
-            assert_close(oracle, got, ref, K, F16, f"{tb} s={s}")
+            for pipe in (0, 2):
+                got = run_splitk(beamc, a, b, F16, tb, wp, s, pipe)
+                assert_close(oracle, got, ref, K, F16, f"{tb} s={s} pipeline {pipe}")
     # the oracle's own slice-ordered sum agrees with its single-pass sum to fp32 reorder noise
     ref_s = oracle.gemmrc_splitk(a, b, 16, F16)
     assert np.abs(ref_s - ref).max() <= 1e-4 * r["rms_ref"]
@@ -68,8 +69,9 @@ def test_splitk_ragged_and_clamped(gpu, beamc, oracle, shape, s):
         a = beamc.host_uniform((M, K), dtype, 13, 0)
         b = beamc.host_uniform((N, K), dtype, 13, 1)
         ref = oracle.gemmrc(a, b, dtype)
-        got = run_splitk(beamc, a, b, dtype, (64, 64), (32, 32), s)
-        assert_close(oracle, got, ref, K, dtype, f"{shape} s={s}")
+        for pipe in (0, 1, 2):
+            got = run_splitk(beamc, a, b, dtype, (64, 64), (32, 32), s, pipe)
+            assert_close(oracle, got, ref, K, dtype, f"{shape} s={s} pipeline {pipe}")
 
 
 def test_splitk_workspace_errors(gpu, beamc):
