@@ -25,6 +25,10 @@ METRIC = "fp16 GEMM TFLOP/s + % MFMA peak at 8192^3; split-K µs at 256x256x3276
 # published as 2.5 PFLOP/s.
 PEAK_TFLOPS = 2500.0
 HBM_PEAK_GBS = 8000.0
+# HBM/fabric bytes per launch of the headline kernel, from the counter runs summarised in
+# profiles/gemmrc_256x256_fp16_8192cube.txt (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000, the factors of
+# profiles/copy_256MiB_counter_calibration.txt).  Counters cannot be read from inside this script.
+PROFILED_TRAFFIC_BYTES = 1.769e9
 
 
 def time_region(_C, fn, steps):
@@ -150,7 +154,7 @@ def main():
                    "tile": cfg.name, "device": info["name"], "compute_units": info["compute_units"]},
         "pct_of_peak": round(100.0 * value / PEAK_TFLOPS, 2),
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(achieved / PEAK_TFLOPS, 4), "traffic": None,
+                     "frac": round(achieved / PEAK_TFLOPS, 4), "traffic": PROFILED_TRAFFIC_BYTES,
                      "kernel_ms": round(kern_ms, 4)},
     }
     if not args.no_cpu:

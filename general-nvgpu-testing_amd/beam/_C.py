@@ -96,6 +96,7 @@ def _load() -> ctypes.CDLL:
     L.beam_free.argtypes = [vp]
     L.beam_memcpy_h2d.argtypes = [vp, vp, sz]
     L.beam_memcpy_d2h.argtypes = [vp, vp, sz]
+    L.beam_memcpy_d2d.argtypes = [vp, vp, sz]
     L.beam_memset.argtypes = [vp, i, sz]
     L.beam_sync.argtypes = [vp]
     L.beam_host_fill_uniform.argtypes = [vp, sz, i, ctypes.c_uint64, ctypes.c_uint64]

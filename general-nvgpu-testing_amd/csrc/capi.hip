@@ -619,6 +619,10 @@ int beam_memcpy_d2h(void* dst_host, const void* src, size_t bytes) {
   if (bytes) BEAM_HIP(hipMemcpy(dst_host, src, bytes, hipMemcpyDeviceToHost));
   return BEAM_OK;
 }
+int beam_memcpy_d2d(void* dst, const void* src, size_t bytes) {
+  if (bytes) BEAM_HIP(hipMemcpy(dst, src, bytes, hipMemcpyDeviceToDevice));
+  return BEAM_OK;
+}
 int beam_memset(void* dptr, int byte, size_t bytes) {
   if (bytes) BEAM_HIP(hipMemset(dptr, byte, bytes));
   return BEAM_OK;

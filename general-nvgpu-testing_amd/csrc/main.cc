@@ -15,6 +15,7 @@
 //   beam_host --bench [--op gemm|splitk|ln] --m M --n N --k K [--dtype fp16|bf16] [--tile BMxBN]
 //             [--wave TMxTN] [--pipeline 0|1] [--group G] [--splitk S] [--iters I] [--warmup W]
 //   beam_host --tune --m M --n N --k K [--dtype fp16|bf16]
+//   beam_host --copy MiB      device-to-device copy of known size (calibrates profiler byte counters)
 #include <cmath>
 #include <cstdint>
 #include <cstdio>
@@ -459,7 +460,7 @@ int main(int argc, char** argv) {
     return 0;
   }
   if (a.kv.empty() || a.has("help")) {
-    std::printf("usage: beam_host --list | --info | --run all|<test> | --bench [...] | --tune [...]\n");
+    std::printf("usage: beam_host --list | --info | --run all|<test> | --bench [...] | --tune [...] | --copy MiB\n");
     return a.kv.empty() ? 2 : 0;
   }
   char name[256];
@@ -478,6 +479,16 @@ int main(int argc, char** argv) {
   if (a.has("run")) return run_tests(a.str("run", "all").empty() ? "all" : a.str("run", "all"));
   if (a.has("bench")) return cli_bench(a);
   if (a.has("tune")) return cli_tune(a);
+  if (a.has("copy")) {
+    const size_t bytes = (size_t)a.num("copy", 256) << 20;
+    DevBuf src(bytes), dst(bytes);
+    beam_memset(src.p, 1, bytes);
+    for (int i = 0; i < 5; ++i)
+      if (beam_memcpy_d2d(dst.p, src.p, bytes) != BEAM_OK) return 1;
+    beam_sync(nullptr);
+    std::printf("copied %zu MiB device to device, 5 times\n", bytes >> 20);
+    return 0;
+  }
   std::fprintf(stderr, "nothing to do (try --help)\n");
   return 2;
 }

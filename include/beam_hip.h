@@ -175,6 +175,7 @@ int beam_malloc(void** dptr, size_t bytes);
 int beam_free(void* dptr);
 int beam_memcpy_h2d(void* dst, const void* src_host, size_t bytes);
 int beam_memcpy_d2h(void* dst_host, const void* src, size_t bytes);
+int beam_memcpy_d2d(void* dst, const void* src, size_t bytes);
 int beam_memset(void* dptr, int byte, size_t bytes);
 int beam_sync(void* stream);
 
