@@ -103,8 +103,9 @@ def extra_ln(_C):
     g = _C.DeviceArray.from_numpy(_C.host_normal((N,), _C.F16, 22, 2, 1.0, 0.1))
     bt = _C.DeviceArray.from_numpy(_C.host_normal((N,), _C.F16, 22, 3, 0.0, 0.1))
     c = _C.DeviceArray((M, N))
-    plain = _C.bench(0, a, b, c, warmup=5, iters=20)
-    fused = _C.bench(2, a, b, c, gamma=g, beta=bt, warmup=5, iters=20)
+    for _ in range(2):  # the second round is past the clock transient of a cold start
+        plain = _C.bench(0, a, b, c, warmup=50, iters=100)
+        fused = _C.bench(2, a, b, c, gamma=g, beta=bt, warmup=50, iters=100)
     for x in (a, b, g, bt, c):
         x.free()
     return {"shape": [M, N, K], "gemm_us": round(plain * 1e3, 1), "gemm_ln_us": round(fused * 1e3, 1),
@@ -115,8 +116,11 @@ def extra_ln(_C):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    # The defaults are sized for the part's power management: after an idle period the first ~50
+    # launches of a matrix-core-bound kernel run up to 40% slower while the clock settles to its
+    # sustained value, so a short run measures the transient, not the throughput.
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline and the result check")
     ap.add_argument("--no-extra", action="store_true", help="skip the split-K and GEMM+LN companions")
     args = ap.parse_args()

@@ -22,8 +22,10 @@
 //     While tile h feeds the MFMAs, B tile h+BST-1 and A tile h+AST-1 are in flight, their
 //     loads issued one at a time between rows of MFMAs so the vector-memory path (64 B/clk)
 //     never sees a burst; one s_barrier per K tile;
-//   * fragments are software pipelined one 32-wide step ahead: A in place (a row's next
-//     fragment is fetched right after its last use), B double buffered;
+//   * fragments are software pipelined one 32-wide step ahead, both operands double buffered
+//     in registers; the reads of the next step are issued in the first rows of the current
+//     one and every row of MFMAs is closed by a scheduling fence, so the order written here
+//     is the order executed;
 //   * the MFMA is issued with B as the first operand, so every lane ends up with 4
 //     consecutive columns of one output row per block: stores are 8 bytes (16-bit C) or 16
 //     bytes (fp32), and a row's statistics reduce over registers plus two lane swaps.
@@ -286,13 +288,17 @@ struct GemmTile {
 #pragma unroll
         for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.0f;
 
-    // Fragments of the step being multiplied: A rows in fa, B rows in fb0 or fb1.  They start
-    // as zeros so that the very first step of the pipeline multiplies nothing.
-    vec8 fa[FM], fb0[FN], fb1[FN];
+    // Fragments: both operands are double-buffered in registers (set 0 / set 1).  While the MFMAs
+    // of one step consume one set, the LDS reads of the next step fill the other.  They start as
+    // zeros so that the very first step of the pipeline multiplies nothing.
+    vec8 fa0[FM], fa1[FM], fb0[FN], fb1[FN];
 #pragma unroll
     for (int i = 0; i < FM; ++i)
 #pragma unroll
-      for (int e = 0; e < 8; ++e) fa[i][e] = 0;
+      for (int e = 0; e < 8; ++e) {
+        fa0[i][e] = 0;
+        fa1[i][e] = 0;
+      }
 #pragma unroll
     for (int j = 0; j < FN; ++j)
 #pragma unroll
@@ -301,52 +307,52 @@ struct GemmTile {
         fb1[j][e] = 0;
       }
 
-    // One pipeline step: the MFMAs of the step whose fragments are in (fa, fb_cur) and, row by
-    // row, the LDS reads of the next step's fragments (A in place, B into fb_nxt) from (sa, sb)
-    // plus this row's share of the tile's buffer loads.
+    // One pipeline step = FM rows of FN MFMAs on the fragments in (fa_cur, fb_cur).  The FM + FN
+    // LDS reads of the next step's fragments (from sa, sb into fa_nxt, fb_nxt; B first, it is
+    // needed by the next step's very first MFMA) are issued at the head of the first READ_ROWS
+    // rows, so the last of them has a row or more of MFMA time to land before the step ends; each
+    // row also carries its share of the tile's buffer loads.  A scheduling fence closes every row:
+    // left alone, the compiler sinks the reads to the end of the step and re-uses fragment
+    // registers across the two sets, and the step then starts by waiting for its own reads.
     //   ROW0: index of the step's first row inside the tile (the loads are dealt out row by row).
-    auto step = [&](const char* sa, const char* sb, vec8(&fb_cur)[FN], vec8(&fb_nxt)[FN], int h, auto row0_tag) {
+    auto step = [&](const char* sa, const char* sb, vec8(&fa_cur)[FM], vec8(&fa_nxt)[FM], vec8(&fb_cur)[FN],
+                    vec8(&fb_nxt)[FN], int h, auto row0_tag) {
       constexpr int ROW0 = decltype(row0_tag)::value;
+      constexpr int READS = FM + FN;
+      constexpr int READ_ROWS = FM * FN >= 64 ? FM / 2 : (FM > 1 ? FM - 1 : 1);
+      constexpr int PER_READ_ROW = (READS + READ_ROWS - 1) / READ_ROWS;
 #pragma unroll
       for (int i = 0; i < FM; ++i) {
 #pragma unroll
-        for (int j = 0; j < FN; ++j) acc[i][j] = Traits::mfma(fb_cur[j], fa[i], acc[i][j]);
-        fa[i] = *(const vec8*)(sa + i * 16 * kRowBytes);
+        for (int u = 0; u < PER_READ_ROW; ++u) {
+          const int r = i * PER_READ_ROW + u;
+          if (i < READ_ROWS && r < READS) {
+            if (r < FN) fb_nxt[r] = *(const vec8*)(sb + r * 16 * kRowBytes);
+            else fa_nxt[r - FN] = *(const vec8*)(sa + (r - FN) * 16 * kRowBytes);
+          }
+        }
 #pragma unroll
-        for (int j = i * FN / FM; j < (i + 1) * FN / FM; ++j) fb_nxt[j] = *(const vec8*)(sb + j * 16 * kRowBytes);
+        for (int j = 0; j < FN; ++j) acc[i][j] = Traits::mfma(fb_cur[j], fa_cur[i], acc[i][j]);
 #pragma unroll
         for (int u = 0; u < PER_ROW; ++u) {
           const int l = (ROW0 + i) * PER_ROW + u;  // B first: it is needed one tile sooner
           if (l < LB) load_b(l, h + BST - 1);
           else if (l < LOADS) load_a(l - LB, h + AST - 1);
         }
-      }
-      // Scheduling pipeline for the compiler: per row, FN MFMAs with the row's LDS reads spread
-      // between them, then the row's buffer loads.
-#pragma unroll
-      for (int i = 0; i < FM; ++i) {
-        constexpr int R = 1 + FN / FM;                // LDS reads per row (when FN >= FM)
-        constexpr int G = FN / R > 0 ? FN / R : 1;    // MFMAs between reads
-#pragma unroll
-        for (int r = 0; r < R; ++r) {
-          __builtin_amdgcn_sched_group_barrier(0x008, G, 0);  // MFMA
-          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // DS read
-        }
-        if (FN - G * R > 0) __builtin_amdgcn_sched_group_barrier(0x008, FN - G * R, 0);
-        __builtin_amdgcn_sched_group_barrier(0x020, PER_ROW, 0);  // VMEM read
+        __builtin_amdgcn_sched_barrier(0);
       }
     };
 
     // One K tile h: make it visible to every wavefront, then two steps.  Step 0 multiplies the
-    // second half of tile h-1 while reading the first half of tile h; step 1 multiplies the first
-    // half of tile h while reading its second half.
+    // second half of tile h-1 (set 1) while reading the first half of tile h into set 0; step 1
+    // multiplies set 0 while reading the second half of tile h into set 1.
     auto tile_body = [&](int h) {
       wait_vm_and_lds<WAIT_STEADY>();  // my fills of tile h have landed; my reads of tile h-1 are done
       bare_barrier();                  // ... and so have everyone else's: the slots of tile h-1 are free
       const char* sa = smem + (h % AST) * A_BYTES + a_wave_off;
       const char* sb = smem + B_REGION + (h % BST) * B_BYTES + b_wave_off;
-      step(sa + frag_off[0], sb + frag_off[0], fb1, fb0, h, std::integral_constant<int, 0>{});
-      step(sa + frag_off[1], sb + frag_off[1], fb0, fb1, h, std::integral_constant<int, FM>{});
+      step(sa + frag_off[0], sb + frag_off[0], fa1, fa0, fb1, fb0, h, std::integral_constant<int, 0>{});
+      step(sa + frag_off[1], sb + frag_off[1], fa0, fa1, fb0, fb1, h, std::integral_constant<int, FM>{});
     };
 
     if (n_tiles > 0) {
@@ -366,11 +372,11 @@ struct GemmTile {
       }
       for (int h = 0; h < n_tiles; ++h) tile_body(h);
       wait_vm_and_lds<0>();  // the empty fills of the last iterations must be gone before LDS is reused
-      // Drain: the second half of the last tile is in (fa, fb1).
+      // Drain: the second half of the last tile is in set 1.
 #pragma unroll
       for (int i = 0; i < FM; ++i)
 #pragma unroll
-        for (int j = 0; j < FN; ++j) acc[i][j] = Traits::mfma(fb1[j], fa[i], acc[i][j]);
+        for (int j = 0; j < FN; ++j) acc[i][j] = Traits::mfma(fb1[j], fa1[i], acc[i][j]);
     }
 
     // ---- per-row statistics of the tile (LayerNorm epilogues) -------------------------------
