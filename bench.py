@@ -113,6 +113,25 @@ def extra_ln(_C):
             "gemm_ln_TFLOPs": round(2.0 * M * N * K / (fused * 1e-3) / 1e12, 1)}
 
 
+def extra_silu(_C):
+    """GEMM carrying a SiLU over M*N elements in its K loop, against the two as separate launches."""
+    M = N = K = 4096
+    a = _C.DeviceArray.from_numpy(_C.host_normal((M, K), _C.F16, 33, 0, 0.0, K ** -0.5))
+    b = _C.DeviceArray.from_numpy(_C.host_normal((N, K), _C.F16, 33, 1, 0.0, K ** -0.5))
+    c = _C.DeviceArray((M, N))
+    x = _C.DeviceArray.from_numpy(_C.host_normal((M * N,), _C.F16, 33, 2, 0.0, 2.0))
+    y = _C.DeviceArray((M * N,))
+    for _ in range(2):
+        gemm = _C.bench(_C.OP_GEMM, a, b, c, warmup=50, iters=100)
+        silu = _C.bench(_C.OP_SILU, a, b, c, x=x, y=y, warmup=50, iters=100)
+        pair = _C.bench(_C.OP_GEMM_SILU, a, b, c, x=x, y=y, warmup=50, iters=100)
+    for t in (a, b, c, x, y):
+        t.free()
+    return {"shape": [M, N, K], "elements": M * N, "gemm_us": round(gemm * 1e3, 1), "silu_us": round(silu * 1e3, 1),
+            "silu_GBs": round(4.0 * M * N / (silu * 1e-3) / 1e9, 1), "one_launch_us": round(pair * 1e3, 1),
+            "vs_two_launches": round(pair / (gemm + silu), 4)}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -171,7 +190,7 @@ def main():
     for x in (a, b, c):
         x.free()
     if not args.no_extra:
-        out["extra"] = {"splitk": extra_splitk(_C), "gemm_ln": extra_ln(_C)}
+        out["extra"] = {"splitk": extra_splitk(_C), "gemm_ln": extra_ln(_C), "gemm_silu": extra_silu(_C)}
     print(json.dumps(out))
     if "check" in out and not out["check"]["ok"]:
         sys.exit("bench.py: GPU result outside the tolerance of the CPU oracle")

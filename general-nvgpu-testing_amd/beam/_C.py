@@ -44,7 +44,8 @@ class _Problem(ctypes.Structure):
     _fields_ = [("A", ctypes.c_void_p), ("B", ctypes.c_void_p), ("C", ctypes.c_void_p),
                 ("gamma", ctypes.c_void_p), ("beta", ctypes.c_void_p), ("eps", ctypes.c_float),
                 ("M", ctypes.c_int), ("N", ctypes.c_int), ("K", ctypes.c_int), ("dtype", ctypes.c_int),
-                ("split_k", ctypes.c_int), ("ws", ctypes.c_void_p), ("ws_bytes", ctypes.c_size_t)]
+                ("split_k", ctypes.c_int), ("ws", ctypes.c_void_p), ("ws_bytes", ctypes.c_size_t),
+                ("side_x", ctypes.c_void_p), ("side_y", ctypes.c_void_p), ("side_count", ctypes.c_longlong)]
 
 
 def library_path() -> str:
@@ -87,6 +88,8 @@ def _load() -> ctypes.CDLL:
     L.beam_set_ln_spin_limit.argtypes = [i]
     L.beam_gemmrc_ln_workspace_reset.argtypes = [vp]
     L.beam_gemmrc_ln_timed_out.argtypes = [vp, vp, ctypes.POINTER(i)]
+    L.beam_parallel_gemmrc_silu.argtypes = [vp, vp, vp, i, i, i, vp, vp, ctypes.c_longlong, i, cfgp, vp]
+    L.beam_silu.argtypes = [vp, vp, ctypes.c_longlong, i, vp]
     L.beam_bench.argtypes = [i, ctypes.POINTER(_Problem), cfgp, i, i, vp, ctypes.POINTER(ctypes.c_float)]
     L.beam_event_create.argtypes = [ctypes.POINTER(vp)]
     L.beam_event_record.argtypes = [vp, vp]
@@ -367,6 +370,33 @@ def gemmrc_ln_timed_out() -> bool:
     return bool(flag.value)
 
 
+def _flat_pair(x, y, d=None):
+    px, sx, dx, st = _describe(x)
+    py, sy, dy, _ = _describe(y)
+    nx, ny = int(np.prod(sx, dtype=np.int64)), int(np.prod(sy, dtype=np.int64))
+    if nx != ny:
+        raise BeamError(1, f"elementwise input has {nx} elements, output {ny}")
+    if dx != dy or (d is not None and dx != d):
+        raise BeamError(2, "elementwise input and output must share the GEMM's dtype")
+    return px, py, nx, dx, st
+
+
+def silu(x, y) -> None:
+    """y = x / (1 + exp(-x)) elementwise over arrays of equal size (any shape), one streaming kernel."""
+    px, py, n, d, st = _flat_pair(x, y)
+    _check(lib.beam_silu(px, py, n, d, st))
+
+
+def parallel_gemmrc_silu(a, b, c, x, y, config: Optional[TileConfig] = None) -> None:
+    """c = a @ b.T and, in the same launch, y = silu(x): the elementwise job is streamed through the
+    GEMM's K loop.  Reference: cutlass_parallel_gemmrc_lnr(gemmA, gemmB, gemmC, lnA, lnB),
+    cuda/cute_kernels/main.cc:55-76 (python/beam/_C/beam_C.pyi:20)."""
+    pa, pb, pc, M, N, K, d, st = _problem(a, b, c)
+    px, py, n, _, _ = _flat_pair(x, y, d)
+    cfg = config.to_c() if config is not None else None
+    _check(lib.beam_parallel_gemmrc_silu(pa, pb, pc, M, N, K, px, py, n, d, ctypes.byref(cfg) if cfg else None, st))
+
+
 def _fixed(fn_name: str):
     cfn = getattr(lib, fn_name)
 
@@ -391,18 +421,24 @@ cutlass_gemmrc = gemmrc
 cutlass_gemmrc_spec = gemmrc_spec
 cutlass_gemmrc_splitk = gemmrc_splitk
 cutlass_gemmrc_splitk_spec = gemmrc_splitk_spec
+cutlass_parallel_gemmrc_lnr = parallel_gemmrc_silu
 
 
 # ---------------------------------------------------------------------------- timing / data
 
 
+OP_GEMM, OP_SPLITK, OP_GEMM_LN, OP_GEMM_SILU, OP_SILU = 0, 1, 2, 3, 4
+
+
 def bench(op: int, a, b, c, config: Optional[TileConfig] = None, split_k: int = 0, gamma=None, beta=None,
-          eps: float = 1e-5, warmup: int = 5, iters: int = 20) -> float:
+          eps: float = 1e-5, warmup: int = 5, iters: int = 20, x=None, y=None) -> float:
     """Average milliseconds per call (HIP events around `iters` back-to-back launches)."""
     pa, pb, pc, M, N, K, d, st = _problem(a, b, c)
     cfg = config.to_c() if config is not None else None
     cfgp = ctypes.byref(cfg) if cfg is not None else None
-    q = _Problem(pa, pb, pc, None, None, eps, M, N, K, d, split_k, None, 0)
+    q = _Problem(pa, pb, pc, None, None, eps, M, N, K, d, split_k, None, 0, None, None, 0)
+    if op in (OP_GEMM_SILU, OP_SILU):
+        q.side_x, q.side_y, q.side_count, _, _ = _flat_pair(x, y, d)
     ws = None
     if op == 1:
         s = lib.beam_splitk_effective(M, N, K, cfgp, split_k)

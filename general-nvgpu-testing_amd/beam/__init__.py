@@ -14,6 +14,7 @@ from ._C import (  # noqa: F401
     cutlass_gemmrc_spec,
     cutlass_gemmrc_splitk,
     cutlass_gemmrc_splitk_spec,
+    cutlass_parallel_gemmrc_lnr,
     device_info,
     gemmrc,
     gemmrc_ln,
@@ -22,5 +23,7 @@ from ._C import (  # noqa: F401
     gemmrc_splitk_spec,
     list_configs,
     library_path,
+    parallel_gemmrc_silu,
+    silu,
 )
 from .tuner import Operator, OperatorTuner  # noqa: F401

@@ -1,4 +1,4 @@
-// Launchers of the split-K reduction and the LayerNorm normalisation pass.
+// Launchers of the split-K reduction, the LayerNorm normalisation pass and the streaming SiLU.
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -16,6 +16,9 @@ hipError_t launch_splitk_reduce(const float* ws, void* C, size_t mn, int splits,
 hipError_t launch_ln_apply(const float* X, const float* stats, const void* gamma, const void* beta,
                            void* Y, int M, int N, int tiles_n, int block_n, float eps, int dtype,
                            hipStream_t stream);
+
+// y[i] (16-bit) = silu(x[i]) for i in [0, count); x and y 16-byte aligned.
+hipError_t launch_silu(const void* x, void* y, size_t count, int dtype, hipStream_t stream);
 
 // ints[0 .. n) = 0 (a fill kernel rather than hipMemsetAsync, so that callers may capture it in a graph).
 hipError_t launch_zero_ints(int* ints, int n, hipStream_t stream);

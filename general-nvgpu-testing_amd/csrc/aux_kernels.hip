@@ -2,6 +2,8 @@
 // normalisation pass.  Both stream fp32 from the workspace once and write 16-bit once.
 #include "aux_kernels.h"
 
+#include "elementwise.h"
+
 namespace beam {
 
 namespace {
@@ -92,6 +94,37 @@ __global__ void __launch_bounds__(256) ln_apply_kernel(const float* __restrict__
   }
 }
 
+// y[i] = silu(x[i]) over a flat 16-bit array: 16 bytes per lane per access, four accesses in flight,
+// then the elements after the last whole vector.
+template <typename T>
+__global__ void __launch_bounds__(256) silu_kernel(const T* __restrict__ x, T* __restrict__ y, size_t count) {
+  typedef T vec8 __attribute__((ext_vector_type(8)));
+  const size_t vecs = count / 8;
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  size_t v = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  for (; v + 3 * stride < vecs; v += 4 * stride) {
+    vec8 in[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) in[u] = *(const vec8*)(x + (v + u * stride) * 8);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      vec8 out;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) out[e] = silu_16<T>(in[u][e]);
+      *(vec8*)(y + (v + u * stride) * 8) = out;
+    }
+  }
+  for (; v < vecs; v += stride) {
+    const vec8 in = *(const vec8*)(x + v * 8);
+    vec8 out;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) out[e] = silu_16<T>(in[e]);
+    *(vec8*)(y + v * 8) = out;
+  }
+  const size_t i = vecs * 8 + (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < count) y[i] = silu_16<T>(x[i]);
+}
+
 __global__ void zero_ints_kernel(int* p, int n) {
   for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x) p[i] = 0;
 }
@@ -101,6 +134,19 @@ __global__ void fill_floats_kernel(float* p, size_t n, float v) {
 }
 
 }  // namespace
+
+hipError_t launch_silu(const void* x, void* y, size_t count, int dtype, hipStream_t stream) {
+  size_t blocks = (count / 8 + 4 * 256 - 1) / (4 * 256);
+  if (blocks < 1) blocks = 1;
+  if (blocks > 8192) blocks = 8192;
+  if (dtype == BEAM_BF16)
+    hipLaunchKernelGGL(silu_kernel<__bf16>, dim3((unsigned)blocks), dim3(256), 0, stream, (const __bf16*)x,
+                       (__bf16*)y, count);
+  else
+    hipLaunchKernelGGL(silu_kernel<_Float16>, dim3((unsigned)blocks), dim3(256), 0, stream, (const _Float16*)x,
+                       (_Float16*)y, count);
+  return hipGetLastError();
+}
 
 hipError_t launch_fill_floats(float* floats, size_t n, float value, hipStream_t stream) {
   hipLaunchKernelGGL(fill_floats_kernel, dim3(256), dim3(256), 0, stream, floats, n, value);

@@ -81,6 +81,9 @@ const KernelSet* find_set(const beam_tile_cfg& c) {
 constexpr int kDefaultGroupM = 8;
 constexpr int kMaxK = 1 << 22;
 
+// Elements of a side-job array: its byte size must stay below the out-of-range offset the kernels use.
+constexpr long long kMaxSideElems = (long long)(kOobOffset / 16) * 8;
+
 int check_problem(const void* A, const void* B, const void* C, int M, int N, int K, int dtype) {
   if (M < 0 || N < 0 || K < 0) return fail(BEAM_ERR_INVALID, "negative dimension (M=%d N=%d K=%d)", M, N, K);
   if (dtype != BEAM_F16 && dtype != BEAM_BF16) return fail(BEAM_ERR_UNSUPPORTED, "dtype %d: only fp16 (0) and bf16 (1)", dtype);
@@ -313,6 +316,51 @@ int beam_gemmrc(const void* A, const void* B, void* C, int M, int N, int K, int 
   GemmParams p = base_params(A, B, M, N, K, c);
   p.C = C;
   BEAM_HIP(ks->launch[dtype][kEpiStore][c.pipeline](p, dim3((unsigned)(p.tiles_m * p.tiles_n), 1, 1), st));
+  return BEAM_OK;
+}
+
+int beam_silu(const void* X, void* Y, long long count, int dtype, void* stream) {
+  if (count < 0) return fail(BEAM_ERR_INVALID, "negative element count %lld", count);
+  if (dtype != BEAM_F16 && dtype != BEAM_BF16) return fail(BEAM_ERR_UNSUPPORTED, "dtype %d: only fp16 (0) and bf16 (1)", dtype);
+  if (count == 0) return BEAM_OK;
+  if (!X || !Y) return fail(BEAM_ERR_INVALID, "null elementwise pointer");
+  if (((uintptr_t)X | (uintptr_t)Y) & 15) return fail(BEAM_ERR_UNSUPPORTED, "X and Y must be 16-byte aligned");
+  int rc = beam_init();
+  if (rc) return rc;
+  BEAM_HIP(launch_silu(X, Y, (size_t)count, dtype, (hipStream_t)stream));
+  return BEAM_OK;
+}
+
+int beam_parallel_gemmrc_silu(const void* A, const void* B, void* C, int M, int N, int K, const void* X, void* Y,
+                              long long count, int dtype, const beam_tile_cfg* cfg, void* stream) {
+  int rc = check_problem(A, B, C, M, N, K, dtype);
+  if (rc) return rc;
+  if (count < 0) return fail(BEAM_ERR_INVALID, "negative element count %lld", count);
+  if (count > 0) {
+    if (!X || !Y) return fail(BEAM_ERR_INVALID, "null elementwise pointer");
+    if (((uintptr_t)X | (uintptr_t)Y) & 15) return fail(BEAM_ERR_UNSUPPORTED, "X and Y must be 16-byte aligned");
+    if (count > kMaxSideElems)
+      return fail(BEAM_ERR_UNSUPPORTED, "count=%lld exceeds %lld elements (one buffer descriptor)", count, kMaxSideElems);
+  }
+  if (M == 0 || N == 0 || K == 0) {  // no K loop to hide anything in: the two halves run one after the other
+    if ((rc = beam_gemmrc(A, B, C, M, N, K, dtype, cfg, stream))) return rc;
+    return beam_silu(X, Y, count, dtype, stream);
+  }
+  if ((rc = beam_init())) return rc;
+  beam_tile_cfg c;
+  const KernelSet* ks;
+  if ((rc = resolve_cfg(cfg, M, N, K, &c, &ks))) return rc;
+  if (!cfg && c.pipeline == 2) c.pipeline = 0;  // the default for split-K-shaped problems
+  if (c.pipeline == 2) return fail(BEAM_ERR_UNSUPPORTED, "the side job runs with pipeline 0 or 1");
+  GemmParams p = base_params(A, B, M, N, K, c);
+  p.C = C;
+  p.side_x = X;
+  p.side_y = Y;
+  p.side_count = count;
+  const long long wgs = (long long)p.tiles_m * p.tiles_n;
+  const long long per_pass = wgs * ks->threads;  // vectors one pass of the whole grid covers
+  p.side_iters = (int)(((count >> 3) + per_pass - 1) / per_pass);
+  BEAM_HIP(ks->launch[dtype][kEpiStoreSide][c.pipeline](p, dim3((unsigned)wgs, 1, 1), (hipStream_t)stream));
   return BEAM_OK;
 }
 
@@ -550,6 +598,11 @@ int beam_bench(int op, const beam_problem* q, const beam_tile_cfg* cfg, int warm
       case BEAM_OP_GEMM_LN:
         return beam_gemmrc_ln(q->A, q->B, q->gamma, q->beta, q->eps, q->C, q->M, q->N, q->K, q->dtype, cfg,
                               q->ws, q->ws_bytes, stream);
+      case BEAM_OP_GEMM_SILU:
+        return beam_parallel_gemmrc_silu(q->A, q->B, q->C, q->M, q->N, q->K, q->side_x, q->side_y, q->side_count,
+                                         q->dtype, cfg, stream);
+      case BEAM_OP_SILU:
+        return beam_silu(q->side_x, q->side_y, q->side_count, q->dtype, stream);
       default:
         return fail(BEAM_ERR_INVALID, "unknown op %d", op);
     }

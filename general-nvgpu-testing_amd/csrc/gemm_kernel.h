@@ -36,6 +36,7 @@
 
 #include <type_traits>
 
+#include "elementwise.h"
 #include "tile_map.h"
 
 namespace beam {
@@ -74,7 +75,9 @@ enum Epilogue : int {
   kEpiPartial = 1,  // store fp32 partial sums of this K slice into the split-K workspace
   kEpiLnStats = 2,  // store fp32 X and per-(row, column-tile) mean / M2 for LayerNorm
   kEpiLnFused = 3,  // LayerNorm in the epilogue: tiles of a row band exchange statistics only
+  kEpiStoreSide = 4,  // kEpiStore plus an independent elementwise job (SiLU) streamed through the K loop
 };
+constexpr int kNumEpilogues = 5;
 
 struct GemmParams {
   const void* A;
@@ -95,6 +98,13 @@ struct GemmParams {
   int splits;    // number of K slices (1 = no split); the grid holds tiles_m * tiles_n * splits workgroups
   int group_m;   // rasterisation group height in tiles (fused LayerNorm: bands per band group)
   int group_n;   // fused LayerNorm: columns of a band group owned by one XCD
+  // Side job (kEpiStoreSide): y[i] = silu(x[i]) over a flat 16-bit array.  Whole 8-element
+  // vectors are dealt out in contiguous runs of side_iters * threads vectors per workgroup, one
+  // vector per thread per K tile; the last side_count % 8 elements are done by workgroup 0.
+  const void* side_x;
+  void* side_y;
+  long long side_count;  // elements
+  int side_iters;        // vectors per thread of one workgroup
 };
 
 // Buffer descriptor word 3 for gfx9-family raw buffers: 32-bit data format, no swizzle.
@@ -155,7 +165,11 @@ struct GemmTile {
   static constexpr int ROWS = KSTEPS * FM;                 // rows of MFMAs per K tile
   static constexpr int PER_ROW = (LOADS + ROWS - 1) / ROWS;  // buffer loads issued after each row
   // Loads that may still be in flight when tile h is needed: the A tiles and B tiles beyond h.
-  static constexpr int WAIT_STEADY = (AST - 2) * LA + (BST - 2) * LB;
+  // The side job adds one buffer store and one buffer load at the end of every K tile; the
+  // fills a tile waits for were issued min(AST, BST) - 1 tiles earlier.
+  static constexpr bool SIDE = (EPI == kEpiStoreSide);
+  static constexpr int WAIT_STEADY =
+      (AST - 2) * LA + (BST - 2) * LB + (SIDE ? 2 * ((AST < BST ? AST : BST) - 1) : 0);
 
   static_assert(KSTEPS == 2, "the step pipeline below is written for two 32-wide steps per tile");
   static_assert(TM % 16 == 0 && TN % 16 == 0, "wavefront tile must be made of 16x16 blocks");
@@ -307,6 +321,33 @@ struct GemmTile {
         fb1[j][e] = 0;
       }
 
+    // ---- side job: state and pieces ------------------------------------------------------
+    // side_in holds the vector loaded during the previous K tile; one element per MFMA row of
+    // step 1 is pushed through silu into side_out, which is stored at the end of the tile, right
+    // before the load of the next vector.  Vectors outside this workgroup's run get an offset
+    // outside the descriptor: the load returns zeros and the store is dropped.
+    const unsigned side_bytes = SIDE ? (unsigned)((p.side_count >> 3) << 4) : 0u;
+    const __amdgpu_buffer_rsrc_t rsrc_sx = make_rsrc(p.side_x, side_bytes);
+    const __amdgpu_buffer_rsrc_t rsrc_sy = make_rsrc(p.side_y, side_bytes);
+    const unsigned side_v0 = SIDE ? ((unsigned)blockIdx.x * (unsigned)p.side_iters * NT + tid) : 0u;
+    i32x4 side_in = {0, 0, 0, 0};
+    vec8 side_out;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) side_out[e] = 0;
+    auto side_offset = [&](int it) {
+      return (it >= 0 && it < p.side_iters) ? (side_v0 + (unsigned)it * NT) * 16u : kOobOffset;
+    };
+    auto side_load = [&](int it) {
+      side_in = __builtin_amdgcn_raw_buffer_load_b128(rsrc_sx, (int)side_offset(it), 0, 0);
+    };
+    auto side_store = [&](int it) {
+      __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(i32x4, side_out), rsrc_sy, (int)side_offset(it), 0, 0);
+    };
+    auto side_element = [&](int e) {
+      const vec8 x = __builtin_bit_cast(vec8, side_in);
+      side_out[e] = silu_16<T>(x[e]);
+    };
+
     // One pipeline step = FM rows of FN MFMAs on the fragments in (fa_cur, fb_cur).  The FM + FN
     // LDS reads of the next step's fragments (from sa, sb into fa_nxt, fb_nxt; B first, it is
     // needed by the next step's very first MFMA) are issued at the head of the first READ_ROWS
@@ -333,6 +374,14 @@ struct GemmTile {
         }
 #pragma unroll
         for (int j = 0; j < FN; ++j) acc[i][j] = Traits::mfma(fb_cur[j], fa_cur[i], acc[i][j]);
+        if constexpr (SIDE && ROW0 != 0) {  // step 1: this row's share of the side vector
+          constexpr int PER = (8 + FM - 1) / FM;
+          if (h < p.side_iters) {  // uniform: tiles past the workgroup's run carry nothing
+#pragma unroll
+            for (int u = 0; u < PER; ++u)
+              if (i * PER + u < 8) side_element(i * PER + u);
+          }
+        }
 #pragma unroll
         for (int u = 0; u < PER_ROW; ++u) {
           const int l = (ROW0 + i) * PER_ROW + u;  // B first: it is needed one tile sooner
@@ -353,6 +402,10 @@ struct GemmTile {
       const char* sb = smem + B_REGION + (h % BST) * B_BYTES + b_wave_off;
       step(sa + frag_off[0], sb + frag_off[0], fa1, fa0, fb1, fb0, h, std::integral_constant<int, 0>{});
       step(sa + frag_off[1], sb + frag_off[1], fa0, fa1, fb0, fb1, h, std::integral_constant<int, FM>{});
+      if constexpr (SIDE) {
+        side_store(h);
+        side_load(h + 1);
+      }
     };
 
     if (n_tiles > 0) {
@@ -369,6 +422,10 @@ struct GemmTile {
 #pragma unroll
           for (int i = 0; i < LB; ++i) load_b(i, s);
         }
+      }
+      if constexpr (SIDE) {
+        side_store(-1);  // dropped; keeps the number of side operations per tile uniform
+        side_load(0);
       }
       for (int h = 0; h < n_tiles; ++h) tile_body(h);
       wait_vm_and_lds<0>();  // the empty fills of the last iterations must be gone before LDS is reused
@@ -469,7 +526,7 @@ struct GemmTile {
     const int n_base = col0 + wn * TN + 4 * (lane >> 4);
     const bool vec_ok = (N % 4) == 0;
 
-    if (EPI == kEpiStore) {
+    if (EPI == kEpiStore || EPI == kEpiStoreSide) {
       T* C = (T*)p.C;
 #pragma unroll
       for (int i = 0; i < FM; ++i) {
@@ -489,6 +546,22 @@ struct GemmTile {
             for (int e = 0; e < 4; ++e)
               if (n + e < N) crow[n + e] = v[e];
           }
+        }
+      }
+      if constexpr (SIDE) {
+        // Side vectors beyond the K tiles of this workgroup (a short K loop or a long array), then
+        // the elements after the last whole vector.
+        for (int it = n_tiles; it < p.side_iters; ++it) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) side_element(e);
+          side_store(it);
+          side_load(it + 1);
+        }
+        const long long done = (p.side_count >> 3) << 3;
+        if (blockIdx.x == 0 && done + tid < p.side_count) {
+          const T* x = (const T*)p.side_x;
+          T* y = (T*)p.side_y;
+          y[done + tid] = silu_16<T>(x[done + tid]);
         }
       }
     } else if (EPI == kEpiLnFused) {

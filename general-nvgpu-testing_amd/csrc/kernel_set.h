@@ -18,7 +18,7 @@ struct KernelSet {
   int lds_bytes_shallow;
   int lds_bytes_deep;
   // [dtype][epilogue][pipeline: 0 = 3 A + 2 B slots, 1 = 2 + 2, 2 = deep (store / partial only)]
-  GemmLauncher launch[2][4][3];
+  GemmLauncher launch[2][kNumEpilogues][3];
 };
 
 template <typename T, int BM, int BN, int WVM, int WVN, int EPI, int AST, int BST>
@@ -61,7 +61,10 @@ KernelSet make_kernel_set() {
   k.launch[D][kEpiLnStats][0] = launch_gemm<T, BM, BN, WVM, WVN, kEpiLnStats, 3, 2>; \
   k.launch[D][kEpiLnStats][1] = launch_gemm<T, BM, BN, WVM, WVN, kEpiLnStats, 2, 2>; \
   k.launch[D][kEpiLnFused][0] = launch_gemm<T, BM, BN, WVM, WVN, kEpiLnFused, 3, 2>; \
-  k.launch[D][kEpiLnFused][1] = launch_gemm<T, BM, BN, WVM, WVN, kEpiLnFused, 2, 2>;
+  k.launch[D][kEpiLnFused][1] = launch_gemm<T, BM, BN, WVM, WVN, kEpiLnFused, 2, 2>; \
+  k.launch[D][kEpiStoreSide][0] = launch_gemm<T, BM, BN, WVM, WVN, kEpiStoreSide, 3, 2>; \
+  k.launch[D][kEpiStoreSide][1] = launch_gemm<T, BM, BN, WVM, WVN, kEpiStoreSide, 2, 2>; \
+  k.launch[D][kEpiStoreSide][2] = nullptr;
   BEAM_FILL(0, _Float16)
   BEAM_FILL(1, __bf16)
 #undef BEAM_FILL

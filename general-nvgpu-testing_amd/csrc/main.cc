@@ -12,8 +12,9 @@
 //   beam_host --list
 //   beam_host --info
 //   beam_host --run all | <test name>
-//   beam_host --bench [--op gemm|splitk|ln] --m M --n N --k K [--dtype fp16|bf16] [--tile BMxBN]
+//   beam_host --bench [--op gemm|splitk|ln|silu] --m M --n N --k K [--dtype fp16|bf16] [--tile BMxBN]
 //             [--wave TMxTN] [--pipeline 0|1] [--group G] [--splitk S] [--iters I] [--warmup W]
+//             [--count ELEMENTS]   (silu: GEMM, SiLU alone and GEMM with the SiLU in its K loop)
 //   beam_host --tune --m M --n N --k K [--dtype fp16|bf16]
 //   beam_host --copy MiB      device-to-device copy of known size (calibrates profiler byte counters)
 #include <cmath>
@@ -259,6 +260,33 @@ BEAM_TEST(splitk_consistency) {
   return c;
 }
 
+// GEMM with the SiLU side job: C equals the plain GEMM bit for bit, Y equals the standalone kernel,
+// silu(0) = 0 and silu(x) = x for x >= 20 (fp16), for an array longer than the K loops can carry.
+BEAM_TEST(gemm_silu_side_job) {
+  Check c;
+  const int M = 384, N = 320, K = 200;
+  const long long count = 300007;
+  std::vector<uint16_t> a = normal16((size_t)M * K, BEAM_F16, 8, 0, 0.0f, 0.1f),
+                        b = normal16((size_t)N * K, BEAM_F16, 8, 1, 0.0f, 0.1f),
+                        x = normal16((size_t)count, BEAM_F16, 8, 2, 0.0f, 3.0f);
+  x[0] = 0;
+  x[1] = small_to_16(20.0f, BEAM_F16);
+  x[count - 1] = small_to_16(64.0f, BEAM_F16);
+  DevBuf da(a.size() * 2), db(b.size() * 2), dc((size_t)M * N * 2), dc2((size_t)M * N * 2), dx(x.size() * 2),
+      dy(x.size() * 2), dy2(x.size() * 2);
+  da.upload(a);
+  db.upload(b);
+  dx.upload(x);
+  BEAM_REQUIRE(c, beam_parallel_gemmrc_silu(da.p, db.p, dc.p, M, N, K, dx.p, dy.p, count, BEAM_F16, nullptr, nullptr));
+  BEAM_REQUIRE(c, beam_gemmrc(da.p, db.p, dc2.p, M, N, K, BEAM_F16, nullptr, nullptr));
+  BEAM_REQUIRE(c, beam_silu(dx.p, dy2.p, count, BEAM_F16, nullptr));
+  if (dc.download16() != dc2.download16()) c.fail("C differs from the plain GEMM");
+  std::vector<uint16_t> y = dy.download16();
+  if (y != dy2.download16()) c.fail("Y differs from the standalone SiLU");
+  if ((y[0] & 0x7fff) != 0 || y[1] != x[1] || y[count - 1] != x[count - 1]) c.fail("closed forms of silu");
+  return c;
+}
+
 // LayerNorm invariants: gamma = 1, beta = 0 gives rows of mean 0 and variance 1; x = 0 gives beta.
 BEAM_TEST(layernorm_invariants) {
   Check c;
@@ -387,6 +415,41 @@ int time_op(int op, Problem& p, const beam_tile_cfg* cfg, int split_k, int warmu
   return beam_bench(op, &q, cfg, warmup, iters, nullptr, ms);
 }
 
+// GEMM alone, SiLU alone and the GEMM carrying the SiLU, interleaved over several rounds.
+int cli_bench_silu(const Args& a, Problem& p, const beam_tile_cfg& cfg) {
+  const long long count = a.has("count") ? std::atoll(a.str("count", "0").c_str()) : (long long)p.M * p.N;
+  DevBuf x((size_t)count * 2 + 16), y((size_t)count * 2 + 16);
+  x.upload(normal16((size_t)count, p.dtype, 7, 4, 0.0f, 2.0f));
+  beam_problem q;
+  std::memset(&q, 0, sizeof q);
+  q.A = p.a.p;
+  q.B = p.b.p;
+  q.C = p.c.p;
+  q.M = p.M;
+  q.N = p.N;
+  q.K = p.K;
+  q.dtype = p.dtype;
+  q.side_x = x.p;
+  q.side_y = y.p;
+  q.side_count = count;
+  const int warmup = a.num("warmup", 50), iters = a.num("iters", 100);
+  float gemm = 0, silu = 0, pair = 0;
+  for (int round = 0; round < 3; ++round) {
+    if (beam_bench(BEAM_OP_GEMM, &q, &cfg, warmup, iters, nullptr, &gemm) ||
+        beam_bench(BEAM_OP_SILU, &q, &cfg, warmup, iters, nullptr, &silu) ||
+        beam_bench(BEAM_OP_GEMM_SILU, &q, &cfg, warmup, iters, nullptr, &pair)) {
+      std::fprintf(stderr, "bench failed: %s\n", beam_last_error());
+      return 1;
+    }
+  }
+  std::printf("silu %dx%dx%d %s tile %dx%d wave %dx%d pipeline %d, %lld elements: gemm %.1f us, silu alone %.1f us "
+              "(%.0f GB/s), gemm+silu in one launch %.1f us = %.3f of the two launches, %.1f TFLOP/s\n",
+              p.M, p.N, p.K, p.dtype ? "bf16" : "fp16", cfg.block_m, cfg.block_n, cfg.wave_m, cfg.wave_n, cfg.pipeline,
+              count, gemm * 1e3, silu * 1e3, 4.0 * count / silu / 1e6, pair * 1e3, pair / (gemm + silu),
+              2.0 * p.M * p.N * p.K / pair / 1e9);
+  return 0;
+}
+
 int cli_bench(const Args& a) {
   const int M = a.num("m", 8192), N = a.num("n", 8192), K = a.num("k", 8192);
   const int dtype = a.str("dtype", "fp16") == "bf16" ? BEAM_BF16 : BEAM_F16;
@@ -401,6 +464,10 @@ int cli_bench(const Args& a) {
   cfg.group_m = a.num("group", cfg.group_m);
   split = a.num("splitk", op == BEAM_OP_SPLITK ? 0 : split);
   Problem p(M, N, K, dtype);
+  if (opname == "silu") {
+    if (cfg.pipeline == 2) cfg.pipeline = 0;
+    return cli_bench_silu(a, p, cfg);
+  }
   float ms = 0;
   int rc = time_op(op, p, &cfg, split, a.num("warmup", 5), a.num("iters", 20), &ms);
   if (rc != BEAM_OK) {

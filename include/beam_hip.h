@@ -138,10 +138,37 @@ int beam_gemmrc_ln_timed_out(const void* ws, void* stream, int* timed_out);
  * which is how the failure path is exercised without hanging anything. */
 int beam_set_ln_spin_limit(int polls);
 
+/* ---- GEMM with an independent elementwise job hidden in its K loop ------------------------ */
+
+/* C = A . B^T as beam_gemmrc and, in the same launch, Y[i] = silu(X[i]) = X[i] / (1 + exp(-X[i]))
+ * for i in [0, count): 16-bit in, fp32 arithmetic, round-to-nearest 16-bit out.  The array is dealt
+ * out over the GEMM's workgroups and streamed one 16-byte vector per thread per K tile, so the
+ * elementwise traffic rides in the memory-side slack of the matrix-core-bound loop.  Replaces
+ * entry_cute_parallel_gemmrc_lnr (cuda/cute_kernels/cute_gemm_ln.cu:230-245, kernel :24-228, bound
+ * as cutlass_parallel_gemmrc_lnr in cuda/cute_kernels/main.cc), whose lnA/lnB are X/Y here and whose
+ * lnM*lnN is `count`.  Unlike the reference, which gives the job to a quarter of the workgroups and
+ * drops whatever does not fit their K loops, every element is processed exactly once for any
+ * count and any GEMM shape.  X, Y: device pointers, 16-byte aligned, count <= 1 073 741 696;
+ * Y may be X (in place) but must not overlap it otherwise; neither may overlap C.
+ * cfg->pipeline must be 0 or 1. */
+int beam_parallel_gemmrc_silu(const void* A, const void* B, void* C, int M, int N, int K, const void* X,
+                              void* Y, long long count, int dtype, const beam_tile_cfg* cfg, void* stream);
+
+/* The elementwise job alone (one streaming kernel): the baseline beam_parallel_gemmrc_silu is
+ * measured against, and what it falls back on when the GEMM is empty (M, N or K = 0).  The
+ * reference has no separate entry for it (the formula is cuda/cute_kernels/cute_gemm_ln.cu:191-192). */
+int beam_silu(const void* X, void* Y, long long count, int dtype, void* stream);
+
 /* ---- timing ------------------------------------------------------------------------------- */
 
 /* Which operation beam_bench times. */
-typedef enum beam_op { BEAM_OP_GEMM = 0, BEAM_OP_SPLITK = 1, BEAM_OP_GEMM_LN = 2 } beam_op;
+typedef enum beam_op {
+  BEAM_OP_GEMM = 0,
+  BEAM_OP_SPLITK = 1,
+  BEAM_OP_GEMM_LN = 2,
+  BEAM_OP_GEMM_SILU = 3, /* beam_parallel_gemmrc_silu */
+  BEAM_OP_SILU = 4       /* beam_silu alone            */
+} beam_op;
 
 typedef struct beam_problem {
   const void* A;
@@ -154,6 +181,9 @@ typedef struct beam_problem {
   int split_k;        /* BEAM_OP_SPLITK                                             */
   void* ws;
   size_t ws_bytes;
+  const void* side_x;   /* BEAM_OP_GEMM_SILU, BEAM_OP_SILU                            */
+  void* side_y;
+  long long side_count;
 } beam_problem;
 
 /* `warmup` untimed calls, then `iters` back-to-back calls bracketed by HIP events on `stream`;

@@ -24,10 +24,14 @@
  *                        SiLU).  Textbook LayerNorm over N on the fp32 GEMM result:
  *                        y = (x - mean) / sqrt(var + eps) * gamma + beta, biased variance.
  *
+ *   oracle_silu          y = x / (1 + exp(-x)) in fp32 on the widened 16-bit input, RN 16-bit out:
+ *                        the side job of cuda/cute_kernels/cute_gemm_ln.cu:186-197 (formula :191-192)
+ *
  * Pinning (see tests/test_oracle.py): float64 numpy fixtures under tests/golden, closed forms
  * (identity, all-ones, one-hot), brute-force triple loops on tiny and ragged shapes, numpy's
  * own float16 conversion for the software converters, the worked example tiles=4 -> 41 slices
- * for the heuristic.  oracle_gemmrc_ln and oracle_gemmrc_splitk have no counterpart the
+ * for the heuristic; oracle_silu over all 65536 fp16 inputs against x * scipy.special.expit(x) in
+ * float64, the identity silu(x) - silu(-x) = x and the known minimum.  oracle_gemmrc_ln and oracle_gemmrc_splitk have no counterpart the
  * reference's own tests hold: they are pinned by the mathematics only.
  */
 #include <math.h>
@@ -356,6 +360,17 @@ void oracle_compare(const uint16_t* got, const float* ref, size_t n, int dtype, 
 
 /* cuda/cutlass_kernels/cutlass_gemmrc_splitk.cu:44-57 with the SM count as a parameter
  * (the reference hard-codes 108).  Float arithmetic on purpose: it is what the reference does. */
+/* y32[i] = silu(float(x[i])) in fp32 (may be NULL), y16[i] = its RN 16-bit rounding (may be NULL). */
+void oracle_silu(const uint16_t* x, uint16_t* y16, float* y32, size_t n, int dtype) {
+#pragma omp parallel for schedule(static)
+  for (long long i = 0; i < (long long)n; ++i) {
+    const float v = dtype == 1 ? oracle_bf16_bits_to_f32(x[i]) : oracle_f16_bits_to_f32(x[i]);
+    const float r = v / (1.0f + expf(-v));
+    if (y32) y32[i] = r;
+    if (y16) y16[i] = dtype == 1 ? oracle_f32_to_bf16_bits(r) : oracle_f32_to_f16_bits(r);
+  }
+}
+
 int oracle_slice_heuristic(int tiles, float units) {
   int split_k_slices = 1;
   if ((float)tiles < units) {

@@ -59,6 +59,8 @@ def lib() -> ctypes.CDLL:
         L.oracle_tflops.argtypes = [ctypes.c_double] * 4
         L.oracle_tflops.restype = ctypes.c_double
         L.oracle_num_threads.restype = i
+        L.oracle_silu.argtypes = [u16p, u16p, f32p, ctypes.c_size_t, i]
+        L.oracle_silu.restype = None
         _lib = L
     return _lib
 
@@ -130,6 +132,15 @@ def gemmrc_ln(a_bits, b_bits, gamma_bits, beta_bits, eps: float = 1e-5, dtype: i
     if rc != 0:
         raise MemoryError("oracle_gemmrc_ln failed")
     return y32
+
+
+def silu(x_bits: np.ndarray, dtype: int = F16):
+    """(fp32 values, RN 16-bit bit patterns) of x / (1 + exp(-x)) on a flat 16-bit array."""
+    x = np.ascontiguousarray(x_bits, dtype=np.uint16).ravel()
+    y32 = np.empty(x.size, dtype=np.float32)
+    y16 = np.empty(x.size, dtype=np.uint16)
+    lib().oracle_silu(_u16(x), _u16(y16), _f32(y32), x.size, dtype)
+    return y32.reshape(x_bits.shape), y16.reshape(x_bits.shape)
 
 
 def compare(got_bits: np.ndarray, ref32: np.ndarray, dtype: int = F16) -> dict:

@@ -17,7 +17,7 @@ def test_registry_runs_green(gpu):
     assert os.path.exists(HOST), "beam_host is not built (make -C general-nvgpu-testing_amd/csrc)"
     listed = run("--list").stdout.split()
     assert {"identity_every_tile", "all_ones_ragged", "one_hot_k_tail", "splitk_consistency",
-            "layernorm_invariants", "error_paths"} <= set(listed)
+            "layernorm_invariants", "gemm_silu_side_job", "error_paths"} <= set(listed)
     r = run("--run", "all")
     assert r.returncode == 0, r.stdout + r.stderr
     assert r.stdout.count("[ OK ]") == len(listed) and "FAIL" not in r.stdout
@@ -31,5 +31,8 @@ def test_cli_bench_and_info(gpu):
     r = run("--bench", "--op", "splitk", "--m", "256", "--n", "256", "--k", "8192", "--tile", "64x64", "--wave", "32x32",
             "--splitk", "16", "--iters", "5")
     assert r.returncode == 0 and "split 16" in r.stdout, r.stdout + r.stderr
+    r = run("--bench", "--op", "silu", "--m", "1024", "--n", "1024", "--k", "1024", "--count", "1048579", "--iters", "5",
+            "--warmup", "2")
+    assert r.returncode == 0 and "gemm+silu in one launch" in r.stdout, r.stdout + r.stderr
     r = run("--bench", "--tile", "100x100")
     assert r.returncode != 0

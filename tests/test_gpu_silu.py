@@ -1,0 +1,193 @@
+"""The elementwise side job: standalone streaming kernel and the GEMM that carries it in its K loop.
+
+Bars: C of beam_parallel_gemmrc_silu is bit-identical to beam_gemmrc with the same tile (same
+accumulation order); its Y is bit-identical to beam_silu's (same device function); beam_silu
+agrees with the CPU oracle to one unit in the last place of the 16-bit format on every input
+pattern (the device uses the hardware exp2 / reciprocal, the oracle libm's expf and a division),
+with NaN where the oracle has NaN.
+"""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+F16, BF16 = 0, 1
+
+
+def ordered(bits):
+    """16-bit sign-magnitude patterns -> integers ordered like the values (so ulp distance = difference)."""
+    b = bits.astype(np.int32)
+    return np.where(b & 0x8000, -(b & 0x7FFF), b & 0x7FFF)
+
+
+def is_nan(bits, dtype):
+    if dtype == F16:
+        return ((bits & 0x7C00) == 0x7C00) & ((bits & 0x03FF) != 0)
+    return ((bits & 0x7F80) == 0x7F80) & ((bits & 0x007F) != 0)
+
+
+def assert_silu_close(got, want, dtype, what=""):
+    gn, wn = is_nan(got, dtype), is_nan(want, dtype)
+    assert (gn == wn).all(), f"{what}: NaN pattern differs"
+    d = np.abs(ordered(got)[~wn] - ordered(want)[~wn])
+    assert d.max(initial=0) <= 1, f"{what}: {int((d > 1).sum())} outputs differ by more than 1 ulp (max {int(d.max())})"
+    assert (d == 0).mean() > 0.97, f"{what}: only {(d == 0).mean():.3f} of the outputs match exactly"
+
+
+def assert_same_bits(got, want, x, what=""):
+    bad = np.flatnonzero(got != want)
+    assert bad.size == 0, (f"{what}: {bad.size} of {got.size} outputs differ; first at {bad[:8].tolist()}: "
+                           f"x={[hex(int(v)) for v in x.ravel()[bad[:8]]]} got={[hex(int(v)) for v in got[bad[:8]]]} "
+                           f"want={[hex(int(v)) for v in want[bad[:8]]]}")
+
+
+def run_silu(beamc, x_bits, dtype, guard=64, in_place=False):
+    n = x_bits.size
+    x = beamc.DeviceArray.from_numpy(np.concatenate([x_bits.ravel(), np.full(guard, 0x3C00, np.uint16)]), dtype)
+    if in_place:
+        y = x
+    else:
+        y = beamc.DeviceArray((n + guard,), dtype)
+        y.fill_bytes(0xEE)
+    xv = beamc.DeviceArray.__new__(beamc.DeviceArray)
+    xv.shape, xv.dtype, xv.itemsize, xv.nbytes, xv.ptr = (n,), dtype, 2, n * 2, x.ptr
+    yv = beamc.DeviceArray.__new__(beamc.DeviceArray)
+    yv.shape, yv.dtype, yv.itemsize, yv.nbytes, yv.ptr = (n,), dtype, 2, n * 2, y.ptr
+    try:
+        beamc.silu(xv, yv)
+        out = y.to_numpy()
+    finally:
+        xv.ptr = yv.ptr = 0
+        x.free()
+        if not in_place:
+            y.free()
+    tail = 0x3C00 if in_place else 0xEEEE
+    assert (out[n:] == tail).all(), "kernel wrote past the end of Y"
+    return out[:n]
+
+
+@pytest.mark.parametrize("dtype", [F16, BF16])
+def test_silu_every_input_pattern(gpu, beamc, oracle, dtype):
+    allbits = np.arange(65536, dtype=np.uint16)
+    x = np.tile(allbits, 3)[: 3 * 65536 - 5]  # not a multiple of 8: the scalar tail runs too
+    _, want = oracle.silu(x, dtype)
+    assert_silu_close(run_silu(beamc, x, dtype), want, dtype, "silu")
+    assert (run_silu(beamc, x, dtype, in_place=True) == run_silu(beamc, x, dtype)).all()
+
+
+def test_silu_sizes(gpu, beamc, oracle):
+    for n in (0, 1, 7, 8, 9, 1023, 8 * 4 * 256 * 3 + 1, 1 << 21):
+        x = beamc.host_normal((max(n, 1),), F16, 5, n, 0.0, 3.0)[:n]
+        if n == 0:
+            beamc._check(beamc.lib.beam_silu(None, None, 0, F16, None))
+            continue
+        _, want = oracle.silu(x, F16)
+        assert_silu_close(run_silu(beamc, x, F16), want, F16, f"n={n}")
+
+
+def run_pair(beamc, a_bits, b_bits, x_bits, dtype, config=None, guard=4096):
+    """(C, Y) of parallel_gemmrc_silu, with guards behind both outputs."""
+    M, K = a_bits.shape
+    N = b_bits.shape[0]
+    n = x_bits.size
+    a = beamc.DeviceArray.from_numpy(a_bits, dtype)
+    b = beamc.DeviceArray.from_numpy(b_bits, dtype)
+    cfull = beamc.DeviceArray((M + 4, N), dtype)
+    cfull.fill_bytes(0xEE)
+    c = beamc.DeviceArray.__new__(beamc.DeviceArray)
+    c.shape, c.dtype, c.itemsize, c.nbytes, c.ptr = (M, N), dtype, 2, M * N * 2, cfull.ptr
+    x = beamc.DeviceArray.from_numpy(np.concatenate([x_bits.ravel(), np.full(guard, 0x3C00, np.uint16)]), dtype)
+    yfull = beamc.DeviceArray((n + guard,), dtype)
+    yfull.fill_bytes(0xEE)
+    xv = beamc.DeviceArray.__new__(beamc.DeviceArray)
+    xv.shape, xv.dtype, xv.itemsize, xv.nbytes, xv.ptr = (n,), dtype, 2, n * 2, x.ptr
+    yv = beamc.DeviceArray.__new__(beamc.DeviceArray)
+    yv.shape, yv.dtype, yv.itemsize, yv.nbytes, yv.ptr = (n,), dtype, 2, n * 2, yfull.ptr
+    try:
+        beamc.parallel_gemmrc_silu(a, b, c, xv, yv, config=config)
+        cout, yout = cfull.to_numpy(), yfull.to_numpy()
+        cfull.fill_bytes(0xEE)
+        beamc.gemmrc(a, b, c, config=config)
+        cplain = cfull.to_numpy()
+    finally:
+        c.ptr = xv.ptr = yv.ptr = 0
+        for t in (a, b, cfull, x, yfull):
+            t.free()
+    assert (cout[M:] == 0xEEEE).all(), "kernel wrote past the end of C"
+    assert (yout[n:] == 0xEEEE).all(), "kernel wrote past the end of Y"
+    assert (cout[:M] == cplain[:M]).all(), "C differs from the plain gemmrc of the same tile"
+    return cout[:M], yout[:n]
+
+
+def test_pair_every_config(gpu, beamc, oracle):
+    """Ragged 300 x 200 x 136 GEMM (K tail of 8) with side arrays shorter than, equal to and far longer
+    than what the K loops can carry; every tile, pipelines 0 and 1."""
+    M, N, K = 300, 200, 136
+    a = beamc.host_uniform((M, K), F16, 2, 0)
+    b = beamc.host_uniform((N, K), F16, 2, 1)
+    ref = oracle.gemmrc(a, b, F16)
+    for cfg in beamc.list_configs():
+        for pipe in (0, 1):
+            c = beamc.TileConfig(cfg.block_m, cfg.block_n, cfg.wave_m, cfg.wave_n, pipe, 0)
+            for n in (0, 5, 4096, 100003):
+                x = beamc.host_normal((max(n, 1),), F16, 9, n, 0.0, 2.5)[:n]
+                cgot, ygot = run_pair(beamc, a, b, x, F16, c)
+                r = oracle.compare(cgot, ref, F16)
+                assert r["max_abs_err"] <= oracle.gemm_tolerance(K) * r["rms_ref"], (c.name, n)
+                if n:
+                    assert_same_bits(ygot, run_silu(beamc, x, F16), x, f"{c.name} n={n}")
+
+
+@pytest.mark.parametrize("dtype", [F16, BF16])
+def test_pair_1024_cube(gpu, beamc, oracle, dtype):
+    M = N = K = 1024
+    a = beamc.host_uniform((M, K), dtype, 1, 0)
+    b = beamc.host_uniform((N, K), dtype, 1, 1)
+    ref = oracle.gemmrc(a, b, dtype)
+    n = 3 * 1024 * 1024 + 3
+    x = np.tile(np.arange(65536, dtype=np.uint16), n // 65536 + 1)[:n]
+    _, want = oracle.silu(x, dtype)
+    cgot, ygot = run_pair(beamc, a, b, x, dtype)
+    r = oracle.compare(cgot, ref, dtype)
+    err = r["max_abs_err"] if dtype == F16 else r["max_bf16_excess"]
+    assert err <= oracle.gemm_tolerance(K) * r["rms_ref"]
+    assert_silu_close(ygot, want, dtype, "pair Y")
+
+
+def test_pair_full_size_properties(gpu, beamc):
+    """4096^3 with 32 Mi side elements: C equals the plain GEMM (checked inside run_pair), Y equals the
+    standalone kernel, and silu(x) - silu(-x) = x holds to the rounding of the two outputs."""
+    M = N = K = 4096
+    a = beamc.host_normal((M, K), F16, 22, 0, 0.0, K ** -0.5)
+    b = beamc.host_normal((N, K), F16, 22, 1, 0.0, K ** -0.5)
+    n = 32 * 1024 * 1024
+    x = beamc.host_normal((n,), F16, 22, 2, 0.0, 2.0)
+    _, y = run_pair(beamc, a, b, x, F16)
+    assert_same_bits(y, run_silu(beamc, x, F16), x, "pair against standalone")
+    _, yneg = run_pair(beamc, a[:256], b[:256], x ^ np.uint16(0x8000), F16)
+    xf, yf, ynf = (t.view(np.float16).astype(np.float32) for t in (x, y, yneg))
+    assert np.abs((yf - ynf) - xf).max() <= 2.0 ** -10 * np.abs(xf).max()
+
+
+def test_pair_error_paths(gpu, beamc):
+    a = beamc.DeviceArray((256, 64), F16)
+    b = beamc.DeviceArray((256, 64), F16)
+    c = beamc.DeviceArray((256, 256), F16)
+    x = beamc.DeviceArray((64,), F16)
+    y = beamc.DeviceArray((32,), F16)
+    with pytest.raises(beamc.BeamError):
+        beamc.parallel_gemmrc_silu(a, b, c, x, y)  # sizes differ
+    y2 = beamc.DeviceArray((64,), BF16)
+    with pytest.raises(beamc.BeamError):
+        beamc.parallel_gemmrc_silu(a, b, c, x, y2)  # dtype differs
+    deep = beamc.TileConfig(128, 128, 64, 64, 2, 0)
+    y3 = beamc.DeviceArray((64,), F16)
+    with pytest.raises(beamc.BeamError) as e:
+        beamc.parallel_gemmrc_silu(a, b, c, x, y3, config=deep)
+    assert e.value.status == 2
+    rc = beamc.lib.beam_parallel_gemmrc_silu(a.ptr, b.ptr, c.ptr, 256, 256, 64, x.ptr + 2, y3.ptr, 8, F16, None, None)
+    assert rc == 2  # misaligned X
+    rc = beamc.lib.beam_parallel_gemmrc_silu(a.ptr, b.ptr, c.ptr, 256, 256, 64, x.ptr, y3.ptr, -1, F16, None, None)
+    assert rc == 1
+    for t in (a, b, c, x, y, y2, y3):
+        t.free()

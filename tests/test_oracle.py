@@ -202,3 +202,48 @@ def test_metric_and_compare(oracle):
     assert r["max_abs_ref"] == 3.0
     assert oracle.gemm_tolerance(1024) == pytest.approx(1e-2)
     assert oracle.gemm_tolerance(4096) == pytest.approx(2e-2)
+
+
+def _bf16_to_f32(bits):
+    return (bits.astype(np.uint32) << 16).view(np.float32)
+
+
+def test_silu_exhaustive_against_library_sigmoid(oracle):
+    """Every fp16 and every bf16 input: the fp32 oracle against x * expit(x) evaluated in float64 by
+    scipy, and its 16-bit rounding against numpy's / the bit-level RN rounding of the float64 value."""
+    from scipy.special import expit
+    allbits = np.arange(65536, dtype=np.uint16)
+    for dtype in (oracle.F16, oracle.BF16):
+        x = allbits.view(np.float16).astype(np.float64) if dtype == oracle.F16 else _bf16_to_f32(allbits).astype(np.float64)
+        y32, y16 = oracle.silu(allbits, dtype)
+        fin = np.isfinite(x)
+        with np.errstate(over="ignore", invalid="ignore"):
+            want = x * expit(x)
+        # Below x = -88.7 exp(-x) overflows in fp32 and the formula returns -0 where the exact value
+        # is a denormal of magnitude up to 1.2e-36: that flush belongs to the reference's formula.
+        assert np.allclose(y32[fin], want[fin], rtol=4e-7, atol=2e-36)
+        assert np.isnan(y32[np.isnan(x)]).all()
+        assert y32[x == np.inf][0] == np.inf
+        got = y16.view(np.float16).astype(np.float64) if dtype == oracle.F16 else _bf16_to_f32(y16).astype(np.float64)
+        ulp = 2.0 ** -10 if dtype == oracle.F16 else 2.0 ** -7
+        tiny = 2.0 ** -24 if dtype == oracle.F16 else 4e-36
+        assert (np.abs(got[fin] - want[fin]) <= 0.5001 * ulp * np.abs(want[fin]) + 0.5001 * tiny).all()
+
+
+def test_silu_identities(oracle):
+    """silu(x) - silu(-x) = x; silu(0) = 0; silu(x) -> x for large x; the global minimum
+    -0.27846454 at x = -1.27846454 (root of 1 + e^x + x = 0 ... i.e. x = -(1 + e^x))."""
+    rng = np.random.default_rng(3)
+    x = (rng.standard_normal(4096) * 4).astype(np.float16)
+    pos, _ = oracle.silu(x.view(np.uint16), oracle.F16)
+    neg, _ = oracle.silu((-x).view(np.uint16), oracle.F16)
+    assert np.allclose(pos - neg, x.astype(np.float32), rtol=0, atol=3e-6)
+    z32, z16 = oracle.silu(np.array([0x0000, 0x8000], dtype=np.uint16), oracle.F16)
+    assert (z32 == 0).all() and (z16 & 0x7FFF == 0).all()
+    big = np.array([20.0, 100.0, 60000.0], dtype=np.float16)
+    b32, b16 = oracle.silu(big.view(np.uint16), oracle.F16)
+    assert (b16 == big.view(np.uint16)).all()
+    grid = np.arange(-2.0, 0.0, 2.0 ** -10, dtype=np.float16)  # exactly representable steps
+    g32, _ = oracle.silu(grid.view(np.uint16), oracle.F16)
+    k = int(np.argmin(g32))
+    assert abs(float(grid[k]) + 1.27846454) < 2.0 ** -10 and abs(float(g32[k]) + 0.27846454) < 1e-6
