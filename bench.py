@@ -132,6 +132,18 @@ def extra_silu(_C):
             "vs_two_launches": round(pair / (gemm + silu), 4)}
 
 
+def extra_nn(_C):
+    """The headline shape with B stored [K][N] (transposed on the way from LDS to registers)."""
+    M = N = K = 8192
+    a = _C.DeviceArray.from_numpy(_C.host_normal((M, K), _C.F16, 7, 0, 0.0, K ** -0.5))
+    b = _C.DeviceArray.from_numpy(_C.host_normal((K, N), _C.F16, 7, 1, 0.0, K ** -0.5))
+    c = _C.DeviceArray((M, N))
+    ms = _C.bench(_C.OP_MATMUL_NN, a, b, c, warmup=100, iters=200)
+    for t in (a, b, c):
+        t.free()
+    return {"shape": [M, N, K], "us": round(ms * 1e3, 1), "TFLOPs": round(2.0 * M * N * K / (ms * 1e-3) / 1e12, 1)}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -190,7 +202,8 @@ def main():
     for x in (a, b, c):
         x.free()
     if not args.no_extra:
-        out["extra"] = {"splitk": extra_splitk(_C), "gemm_ln": extra_ln(_C), "gemm_silu": extra_silu(_C)}
+        out["extra"] = {"splitk": extra_splitk(_C), "gemm_ln": extra_ln(_C), "gemm_silu": extra_silu(_C),
+                        "matmul_nn": extra_nn(_C)}
     print(json.dumps(out))
     if "check" in out and not out["check"]["ok"]:
         sys.exit("bench.py: GPU result outside the tolerance of the CPU oracle")

@@ -90,6 +90,7 @@ def _load() -> ctypes.CDLL:
     L.beam_gemmrc_ln_timed_out.argtypes = [vp, vp, ctypes.POINTER(i)]
     L.beam_parallel_gemmrc_silu.argtypes = [vp, vp, vp, i, i, i, vp, vp, ctypes.c_longlong, i, cfgp, vp]
     L.beam_silu.argtypes = [vp, vp, ctypes.c_longlong, i, vp]
+    L.beam_matmul_nn.argtypes = [vp, vp, vp, i, i, i, i, cfgp, vp]
     L.beam_bench.argtypes = [i, ctypes.POINTER(_Problem), cfgp, i, i, vp, ctypes.POINTER(ctypes.c_float)]
     L.beam_event_create.argtypes = [ctypes.POINTER(vp)]
     L.beam_event_record.argtypes = [vp, vp]
@@ -370,6 +371,31 @@ def gemmrc_ln_timed_out() -> bool:
     return bool(flag.value)
 
 
+def matmul(a, b, c=None, config: Optional[TileConfig] = None):
+    """c = a @ b with a [M, K] and b [K, N], both row-major; returns c (allocated like the inputs when
+    not given).  Reference: matmul(a, b) of python/beam/triton_kernels/gemm.py:78-99."""
+    pa, sa, da, st = _describe(a)
+    pb, sb, db, _ = _describe(b)
+    if len(sa) != 2 or len(sb) != 2 or sa[1] != sb[0]:
+        raise BeamError(1, "Incompatible dimensions")
+    if da != db:
+        raise BeamError(2, "a and b must share one dtype (fp16 or bf16)")
+    M, K = sa
+    N = sb[1]
+    if c is None:
+        if _is_torch(a):
+            import torch
+            c = torch.empty((M, N), device=a.device, dtype=a.dtype)
+        else:
+            c = DeviceArray((M, N), da)
+    pc, sc, dc, _ = _describe(c)
+    if tuple(sc) != (M, N) or dc != da:
+        raise BeamError(1, f"c must be {(M, N)} of the inputs' dtype")
+    cfg = config.to_c() if config is not None else None
+    _check(lib.beam_matmul_nn(pa, pb, pc, M, N, K, da, ctypes.byref(cfg) if cfg else None, st))
+    return c
+
+
 def _flat_pair(x, y, d=None):
     px, sx, dx, st = _describe(x)
     py, sy, dy, _ = _describe(y)
@@ -427,13 +453,20 @@ cutlass_parallel_gemmrc_lnr = parallel_gemmrc_silu
 # ---------------------------------------------------------------------------- timing / data
 
 
-OP_GEMM, OP_SPLITK, OP_GEMM_LN, OP_GEMM_SILU, OP_SILU = 0, 1, 2, 3, 4
+OP_GEMM, OP_SPLITK, OP_GEMM_LN, OP_GEMM_SILU, OP_SILU, OP_MATMUL_NN = 0, 1, 2, 3, 4, 5
 
 
 def bench(op: int, a, b, c, config: Optional[TileConfig] = None, split_k: int = 0, gamma=None, beta=None,
           eps: float = 1e-5, warmup: int = 5, iters: int = 20, x=None, y=None) -> float:
     """Average milliseconds per call (HIP events around `iters` back-to-back launches)."""
-    pa, pb, pc, M, N, K, d, st = _problem(a, b, c)
+    if op == OP_MATMUL_NN:  # b is [K, N]
+        pa, (M, K), d, st = _describe(a)
+        pb, (kb, N), _, _ = _describe(b)
+        pc = _describe(c)[0]
+        if kb != K or tuple(_describe(c)[1]) != (M, N):
+            raise BeamError(1, "Incompatible dimensions")
+    else:
+        pa, pb, pc, M, N, K, d, st = _problem(a, b, c)
     cfg = config.to_c() if config is not None else None
     cfgp = ctypes.byref(cfg) if cfg is not None else None
     q = _Problem(pa, pb, pc, None, None, eps, M, N, K, d, split_k, None, 0, None, None, 0)

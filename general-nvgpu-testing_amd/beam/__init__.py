@@ -23,6 +23,7 @@ from ._C import (  # noqa: F401
     gemmrc_splitk_spec,
     list_configs,
     library_path,
+    matmul,
     parallel_gemmrc_silu,
     silu,
 )

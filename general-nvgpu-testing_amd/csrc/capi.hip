@@ -319,6 +319,29 @@ int beam_gemmrc(const void* A, const void* B, void* C, int M, int N, int K, int 
   return BEAM_OK;
 }
 
+int beam_matmul_nn(const void* A, const void* B, void* C, int M, int N, int K, int dtype, const beam_tile_cfg* cfg,
+                   void* stream) {
+  int rc = check_problem(A, B, C, M, N, K, dtype);
+  if (rc) return rc;
+  if (M == 0 || N == 0) return BEAM_OK;
+  if (N % 8 != 0) return fail(BEAM_ERR_UNSUPPORTED, "N=%d: rows of B must be multiples of 16 bytes (N %% 8 == 0)", N);
+  if ((rc = beam_init())) return rc;
+  hipStream_t st = (hipStream_t)stream;
+  if (K == 0) {
+    BEAM_HIP(hipMemsetAsync(C, 0, (size_t)M * N * 2, st));
+    return BEAM_OK;
+  }
+  beam_tile_cfg c;
+  const KernelSet* ks;
+  if ((rc = resolve_cfg(cfg, M, N, K, &c, &ks))) return rc;
+  if (!cfg && c.pipeline == 2) c.pipeline = 0;
+  if (c.pipeline == 2) return fail(BEAM_ERR_UNSUPPORTED, "the [K][N] layout runs with pipeline 0 or 1");
+  GemmParams p = base_params(A, B, M, N, K, c);
+  p.C = C;
+  BEAM_HIP(ks->launch_kmajor[dtype][c.pipeline](p, dim3((unsigned)(p.tiles_m * p.tiles_n), 1, 1), st));
+  return BEAM_OK;
+}
+
 int beam_silu(const void* X, void* Y, long long count, int dtype, void* stream) {
   if (count < 0) return fail(BEAM_ERR_INVALID, "negative element count %lld", count);
   if (dtype != BEAM_F16 && dtype != BEAM_BF16) return fail(BEAM_ERR_UNSUPPORTED, "dtype %d: only fp16 (0) and bf16 (1)", dtype);
@@ -601,6 +624,8 @@ int beam_bench(int op, const beam_problem* q, const beam_tile_cfg* cfg, int warm
       case BEAM_OP_GEMM_SILU:
         return beam_parallel_gemmrc_silu(q->A, q->B, q->C, q->M, q->N, q->K, q->side_x, q->side_y, q->side_count,
                                          q->dtype, cfg, stream);
+      case BEAM_OP_MATMUL_NN:
+        return beam_matmul_nn(q->A, q->B, q->C, q->M, q->N, q->K, q->dtype, cfg, stream);
       case BEAM_OP_SILU:
         return beam_silu(q->side_x, q->side_y, q->side_count, q->dtype, stream);
       default:

@@ -124,6 +124,13 @@ __device__ __forceinline__ void wait_vm_and_lds() {
   __builtin_amdgcn_s_waitcnt(0x0070 | (N & 15) | ((N >> 4) << 14));
 }
 
+// s_waitcnt lgkmcnt(N): at most N of this wavefront's LDS reads still in flight.
+template <int N>
+__device__ __forceinline__ void wait_lds() {
+  static_assert(N >= 0 && N < 16, "lgkmcnt is a 4-bit counter");
+  __builtin_amdgcn_s_waitcnt(0xC07F | (N << 8));
+}
+
 // Workgroup barrier without the memory fence of __syncthreads(): the fence would wait for
 // every outstanding LDS fill (vmcnt(0)) and serialise the pipeline.  The waits the data
 // hazards need are issued explicitly by the caller.
@@ -142,7 +149,7 @@ constexpr int deep_a_slots(int BM, int BN) {
   return a;
 }
 
-template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, int EPI, int AST, int BST>
+template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, int EPI, int AST, int BST, bool B_KMAJOR = false>
 struct GemmTile {
   using Traits = ElemTraits<T>;
   using vec8 = typename Traits::vec8;
@@ -229,7 +236,9 @@ struct GemmTile {
     const int rows_a = (M - row0) < BM ? (M - row0) : BM;
     const int rows_b = (N - col0) < BN ? (N - col0) : BN;
     const T* a_base = (const T*)p.A + ((size_t)row0 * K + kb);
-    const T* b_base = (const T*)p.B + ((size_t)col0 * K + kb);
+    // B as [N][K] (rows of K): like A.  B as [K][N] (B_KMAJOR): the tile's columns start at col0 of
+    // row kb; a descriptor is made per K tile (load_b) so that it ends with the tile's last row.
+    const T* b_base = B_KMAJOR ? (const T*)p.B + ((size_t)kb * N + col0) : (const T*)p.B + ((size_t)col0 * K + kb);
     const unsigned bytes_a = klen > 0 ? ((unsigned)(rows_a - 1) * K + klen) * 2u : 0u;
     const unsigned bytes_b = klen > 0 ? ((unsigned)(rows_b - 1) * K + klen) * 2u : 0u;
     const __amdgpu_buffer_rsrc_t rsrc_a = make_rsrc(a_base, bytes_a);
@@ -239,7 +248,18 @@ struct GemmTile {
 #pragma unroll
     for (int i = 0; i < LA; ++i) voff_a[i] = chunk_voffset(i * NT + tid, K);
 #pragma unroll
-    for (int i = 0; i < LB; ++i) voff_b[i] = chunk_voffset(i * NT + tid, K);
+    for (int i = 0; i < LB; ++i) {
+      if (B_KMAJOR) {
+        // LDS position q of the stage: row k = q / CPR, and the chunk that lives there is position ^ swizzle
+        constexpr int CPR = BN / 8;
+        const int q = i * NT + tid;
+        const int k = q / CPR;
+        const int chunk = (q % CPR) ^ kmajor_swizzle(k, BN);
+        voff_b[i] = ((unsigned)k * (unsigned)N + (unsigned)chunk * 8u) * 2u;
+      } else {
+        voff_b[i] = chunk_voffset(i * NT + tid, K);
+      }
+    }
 
     // First K element (inside the slice) of tile t: the short tile comes first.
     auto tile_koff = [&](int t) { return k_tail ? (t == 0 ? kt_full * kBK : (t - 1) * kBK) : t * kBK; };
@@ -256,11 +276,25 @@ struct GemmTile {
     };
     auto load_b = [&](int i, int t) {
       char* dst = smem + B_REGION + (t % BST) * B_BYTES + wave * 1024 + i * (NT * 16);
-      const __amdgpu_buffer_rsrc_t r = make_rsrc(b_base, t < n_tiles ? bytes_b : 0u);
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (__attribute__((address_space(3))) void*)dst, 16,
-                                               (int)voff_b[i], tile_koff(t) * 2, 0, 0);
+      if (B_KMAJOR) {
+        // Rows koff .. koff + kBK of the slice, as many as exist: rows past the end of K and the
+        // columns past the last row's end are out of range and read as zeros.  (Columns past N in
+        // earlier rows read the next row's data; they only feed output columns that do not exist.)
+        const int koff = tile_koff(t);
+        int rows = klen - koff;
+        if (rows > kBK) rows = kBK;
+        const unsigned bytes = (t < n_tiles && rows > 0) ? ((unsigned)(rows - 1) * N + rows_b) * 2u : 0u;
+        const __amdgpu_buffer_rsrc_t r = make_rsrc(b_base + (size_t)koff * N, bytes);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (__attribute__((address_space(3))) void*)dst, 16,
+                                                 (int)voff_b[i], 0, 0, 0);
+      } else {
+        const __amdgpu_buffer_rsrc_t r = make_rsrc(b_base, t < n_tiles ? bytes_b : 0u);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (__attribute__((address_space(3))) void*)dst, 16,
+                                                 (int)voff_b[i], tile_koff(t) * 2, 0, 0);
+      }
     };
     // The short tile goes through registers so that chunks at or past `kvalid` are zero-filled.
+    // (A K-major B needs none of this: its rows past the end of K are out of range by themselves.)
     auto fill_short_tile = [&](int kvalid) {
       const int koff = tile_koff(0);
       i32x4 ra[LA], rb[LB];
@@ -271,19 +305,23 @@ struct GemmTile {
         const unsigned off = (chunk * 8 < kvalid) ? voff_a[i] + (unsigned)koff * 2u : kOobOffset;
         ra[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_a, (int)off, 0, 0);
       }
+      if (!B_KMAJOR) {
 #pragma unroll
-      for (int i = 0; i < LB; ++i) {
-        const int q = i * NT + tid;
-        const int chunk = (q & 7) ^ swizzle_of_row(q >> 3);
-        const unsigned off = (chunk * 8 < kvalid) ? voff_b[i] + (unsigned)koff * 2u : kOobOffset;
-        rb[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, (int)off, 0, 0);
+        for (int i = 0; i < LB; ++i) {
+          const int q = i * NT + tid;
+          const int chunk = (q & 7) ^ swizzle_of_row(q >> 3);
+          const unsigned off = (chunk * 8 < kvalid) ? voff_b[i] + (unsigned)koff * 2u : kOobOffset;
+          rb[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, (int)off, 0, 0);
+        }
       }
       char* sa = smem + tid * 16;
       char* sb = smem + B_REGION + tid * 16;
 #pragma unroll
       for (int i = 0; i < LA; ++i) *(i32x4*)(sa + i * (NT * 16)) = ra[i];
+      if (!B_KMAJOR) {
 #pragma unroll
-      for (int i = 0; i < LB; ++i) *(i32x4*)(sb + i * (NT * 16)) = rb[i];
+        for (int i = 0; i < LB; ++i) *(i32x4*)(sb + i * (NT * 16)) = rb[i];
+      }
     };
 
     // ---- LDS -> MFMA fragments ----------------------------------------------------------
@@ -292,7 +330,32 @@ struct GemmTile {
 #pragma unroll
     for (int kk = 0; kk < KSTEPS; ++kk) frag_off[kk] = lds_offset(lane & 15, 4 * kk + (lane >> 4));
     const int a_wave_off = wm * TM * kRowBytes;
-    const int b_wave_off = wn * TN * kRowBytes;
+    const int b_wave_off = B_KMAJOR ? 0 : wn * TN * kRowBytes;
+    // K-major B: a fragment (16 columns x 32 rows of k) is two transposing 8-byte reads.  In the
+    // 16-lane group g = lane >> 4, lane 4*e + q points at row k = 8*g + e (+4 for the second read),
+    // columns 4*q .. 4*q + 3 of the block; the read hands lane i of the group column i of rows
+    // 8*g .. 8*g + 3: the same register contents as the 16-byte read of the [N][K] layout.
+    int bfrag_off[FN];
+    if (B_KMAJOR) {
+#pragma unroll
+      for (int j = 0; j < FN; ++j)
+        bfrag_off[j] = kmajor_lds_offset(8 * (lane >> 4) + ((lane >> 2) & 3), wn * TN + j * 16 + 4 * (lane & 3), BN);
+    }
+    // The transposing reads are inline assembly: given the intrinsic, the compiler orders every
+    // LDS read it can see behind all outstanding global->LDS fills (vmcnt(0)), which would
+    // serialise the pipeline.  Results of inline assembly are not tracked by the compiler's
+    // wait-count insertion, so the step below waits for them explicitly.
+    auto read_b_fragment = [&](const char* sb, int j) -> vec8 {
+      if constexpr (B_KMAJOR) {
+        const unsigned addr = (unsigned)(size_t)(__attribute__((address_space(3))) const char*)(sb + bfrag_off[j]);
+        vec4 lo, hi;
+        asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(lo) : "v"(addr));
+        asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(hi) : "v"(addr), "n"(4 * BN * 2));
+        return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+      } else {
+        return *(const vec8*)(sb + j * 16 * kRowBytes);
+      }
+    };
 
     f32x4 acc[FM][FN];
 #pragma unroll
@@ -368,8 +431,20 @@ struct GemmTile {
         for (int u = 0; u < PER_READ_ROW; ++u) {
           const int r = i * PER_READ_ROW + u;
           if (i < READ_ROWS && r < READS) {
-            if (r < FN) fb_nxt[r] = *(const vec8*)(sb + r * 16 * kRowBytes);
+            if (r < FN) fb_nxt[r] = read_b_fragment(sb, r);
             else fa_nxt[r - FN] = *(const vec8*)(sa + (r - FN) * 16 * kRowBytes);
+          }
+        }
+        if constexpr (B_KMAJOR) {
+          // Row 0: everything the previous step read must have arrived; only the LDS reads issued
+          // just above (two per B fragment, one per A fragment) may still be in flight.
+          if (i == 0) {
+            constexpr int B_NOW = PER_READ_ROW < FN ? PER_READ_ROW : FN;
+            constexpr int NOW = (PER_READ_ROW < READS ? PER_READ_ROW : READS) + B_NOW;
+            wait_lds<(NOW < 15 ? NOW : 15)>();
+            // ... and the MFMAs must not be moved above that wait: tie their B operands to it.
+#pragma unroll
+            for (int j = 0; j < FN; ++j) asm volatile("" : "+v"(fb_cur[j]));
           }
         }
 #pragma unroll
@@ -400,8 +475,11 @@ struct GemmTile {
       bare_barrier();                  // ... and so have everyone else's: the slots of tile h-1 are free
       const char* sa = smem + (h % AST) * A_BYTES + a_wave_off;
       const char* sb = smem + B_REGION + (h % BST) * B_BYTES + b_wave_off;
-      step(sa + frag_off[0], sb + frag_off[0], fa1, fa0, fb1, fb0, h, std::integral_constant<int, 0>{});
-      step(sa + frag_off[1], sb + frag_off[1], fa0, fa1, fb0, fb1, h, std::integral_constant<int, FM>{});
+      // per-step offset of the B fragments: a swizzled chunk of the row, or 32 rows of k
+      const int sb0 = B_KMAJOR ? 0 : frag_off[0];
+      const int sb1 = B_KMAJOR ? 32 * BN * 2 : frag_off[1];
+      step(sa + frag_off[0], sb + sb0, fa1, fa0, fb1, fb0, h, std::integral_constant<int, 0>{});
+      step(sa + frag_off[1], sb + sb1, fa0, fa1, fb0, fb1, h, std::integral_constant<int, FM>{});
       if constexpr (SIDE) {
         side_store(h);
         side_load(h + 1);
@@ -418,7 +496,7 @@ struct GemmTile {
 #pragma unroll
           for (int i = 0; i < LA; ++i) load_a(i, s);
         }
-        if (s < BST - 1 && !(s == 0 && k_tail)) {
+        if (s < BST - 1 && (B_KMAJOR || !(s == 0 && k_tail))) {
 #pragma unroll
           for (int i = 0; i < LB; ++i) load_b(i, s);
         }
@@ -430,6 +508,10 @@ struct GemmTile {
       for (int h = 0; h < n_tiles; ++h) tile_body(h);
       wait_vm_and_lds<0>();  // the empty fills of the last iterations must be gone before LDS is reused
       // Drain: the second half of the last tile is in set 1.
+      if constexpr (B_KMAJOR) {
+#pragma unroll
+        for (int j = 0; j < FN; ++j) asm volatile("" : "+v"(fb1[j]));
+      }
 #pragma unroll
       for (int i = 0; i < FM; ++i)
 #pragma unroll
@@ -720,11 +802,11 @@ struct GemmTile {
   }
 };
 
-template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, int EPI, int AST, int BST>
+template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, int EPI, int AST, int BST, bool B_KMAJOR = false>
 __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64)
     gemmrc_kernel(const GemmParams p) {
   extern __shared__ __attribute__((aligned(1024))) char smem[];
-  GemmTile<T, BM, BN, WAVES_M, WAVES_N, EPI, AST, BST>::run(p, smem);
+  GemmTile<T, BM, BN, WAVES_M, WAVES_N, EPI, AST, BST, B_KMAJOR>::run(p, smem);
 }
 
 }  // namespace beam

@@ -19,12 +19,14 @@ struct KernelSet {
   int lds_bytes_deep;
   // [dtype][epilogue][pipeline: 0 = 3 A + 2 B slots, 1 = 2 + 2, 2 = deep (store / partial only)]
   GemmLauncher launch[2][kNumEpilogues][3];
+  // B stored [K][N] instead of [N][K], kEpiStore only: [dtype][pipeline 0 or 1]
+  GemmLauncher launch_kmajor[2][2];
 };
 
-template <typename T, int BM, int BN, int WVM, int WVN, int EPI, int AST, int BST>
+template <typename T, int BM, int BN, int WVM, int WVN, int EPI, int AST, int BST, bool B_KMAJOR = false>
 hipError_t launch_gemm(const GemmParams& p, dim3 grid, hipStream_t stream) {
-  using Tile = GemmTile<T, BM, BN, WVM, WVN, EPI, AST, BST>;
-  auto kern = gemmrc_kernel<T, BM, BN, WVM, WVN, EPI, AST, BST>;
+  using Tile = GemmTile<T, BM, BN, WVM, WVN, EPI, AST, BST, B_KMAJOR>;
+  auto kern = gemmrc_kernel<T, BM, BN, WVM, WVN, EPI, AST, BST, B_KMAJOR>;
   static bool configured = false;  // benign race: the attribute call is idempotent
   if (!configured) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -64,7 +66,9 @@ KernelSet make_kernel_set() {
   k.launch[D][kEpiLnFused][1] = launch_gemm<T, BM, BN, WVM, WVN, kEpiLnFused, 2, 2>; \
   k.launch[D][kEpiStoreSide][0] = launch_gemm<T, BM, BN, WVM, WVN, kEpiStoreSide, 3, 2>; \
   k.launch[D][kEpiStoreSide][1] = launch_gemm<T, BM, BN, WVM, WVN, kEpiStoreSide, 2, 2>; \
-  k.launch[D][kEpiStoreSide][2] = nullptr;
+  k.launch[D][kEpiStoreSide][2] = nullptr; \
+  k.launch_kmajor[D][0] = launch_gemm<T, BM, BN, WVM, WVN, kEpiStore, 3, 2, true>; \
+  k.launch_kmajor[D][1] = launch_gemm<T, BM, BN, WVM, WVN, kEpiStore, 2, 2, true>;
   BEAM_FILL(0, _Float16)
   BEAM_FILL(1, __bf16)
 #undef BEAM_FILL

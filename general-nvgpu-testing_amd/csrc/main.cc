@@ -12,7 +12,7 @@
 //   beam_host --list
 //   beam_host --info
 //   beam_host --run all | <test name>
-//   beam_host --bench [--op gemm|splitk|ln|silu] --m M --n N --k K [--dtype fp16|bf16] [--tile BMxBN]
+//   beam_host --bench [--op gemm|splitk|ln|silu|nn] --m M --n N --k K [--dtype fp16|bf16] [--tile BMxBN]
 //             [--wave TMxTN] [--pipeline 0|1] [--group G] [--splitk S] [--iters I] [--warmup W]
 //             [--count ELEMENTS]   (silu: GEMM, SiLU alone and GEMM with the SiLU in its K loop)
 //   beam_host --tune --m M --n N --k K [--dtype fp16|bf16]
@@ -260,6 +260,40 @@ BEAM_TEST(splitk_consistency) {
   return c;
 }
 
+// B stored [K][N]: C = I . B reproduces B, and a random problem matches beam_gemmrc on the transposed
+// copy of B bit for bit (the two kernels add the same products in the same order), every tile.
+BEAM_TEST(matmul_nn_every_tile) {
+  Check c;
+  const int M = 200, N = 328, K = 264;
+  for (int dtype = 0; dtype < 2; ++dtype) {
+    std::vector<uint16_t> a = uniform16((size_t)M * K, dtype, 5, 0), b = uniform16((size_t)K * N, dtype, 5, 1);
+    std::vector<uint16_t> bt((size_t)N * K);
+    for (int k = 0; k < K; ++k)
+      for (int n = 0; n < N; ++n) bt[(size_t)n * K + k] = b[(size_t)k * N + n];
+    std::vector<uint16_t> eye((size_t)K * K, 0);
+    for (int i = 0; i < K; ++i) eye[(size_t)i * K + i] = small_to_16(1.0f, dtype);
+    DevBuf da(a.size() * 2), db(b.size() * 2), dbt(bt.size() * 2), de(eye.size() * 2), dc((size_t)M * N * 2),
+        dc2((size_t)M * N * 2), dci((size_t)K * N * 2);
+    da.upload(a);
+    db.upload(b);
+    dbt.upload(bt);
+    de.upload(eye);
+    for (int k = 0; k < beam_num_configs() && c.ok; ++k) {
+      beam_tile_cfg cfg;
+      BEAM_REQUIRE(c, beam_get_config(k, &cfg));
+      BEAM_REQUIRE(c, beam_matmul_nn(da.p, db.p, dc.p, M, N, K, dtype, &cfg, nullptr));
+      BEAM_REQUIRE(c, beam_gemmrc(da.p, dbt.p, dc2.p, M, N, K, dtype, &cfg, nullptr));
+      if (dc.download16() != dc2.download16())
+        c.fail("tile " + std::to_string(cfg.block_m) + "x" + std::to_string(cfg.block_n) + ": differs from gemmrc on B^T");
+      BEAM_REQUIRE(c, beam_matmul_nn(de.p, db.p, dci.p, K, N, K, dtype, &cfg, nullptr));
+      std::vector<uint16_t> got = dci.download16();
+      for (size_t i = 0; i < got.size() && c.ok; ++i)
+        if (got[i] != b[i] && to_float(got[i], dtype) != to_float(b[i], dtype)) c.fail("I . B != B");
+    }
+  }
+  return c;
+}
+
 // GEMM with the SiLU side job: C equals the plain GEMM bit for bit, Y equals the standalone kernel,
 // silu(0) = 0 and silu(x) = x for x >= 20 (fp16), for an array longer than the K loops can carry.
 BEAM_TEST(gemm_silu_side_job) {
@@ -454,7 +488,10 @@ int cli_bench(const Args& a) {
   const int M = a.num("m", 8192), N = a.num("n", 8192), K = a.num("k", 8192);
   const int dtype = a.str("dtype", "fp16") == "bf16" ? BEAM_BF16 : BEAM_F16;
   const std::string opname = a.str("op", "gemm");
-  const int op = opname == "splitk" ? BEAM_OP_SPLITK : (opname == "ln" ? BEAM_OP_GEMM_LN : BEAM_OP_GEMM);
+  const int op = opname == "splitk" ? BEAM_OP_SPLITK
+                 : opname == "ln"   ? BEAM_OP_GEMM_LN
+                 : opname == "nn"   ? BEAM_OP_MATMUL_NN  // B read as [K][N]
+                                    : BEAM_OP_GEMM;
   beam_tile_cfg cfg;
   int split = 1;
   if (beam_default_config(M, N, K, &cfg, &split) != BEAM_OK) return 2;
@@ -464,6 +501,7 @@ int cli_bench(const Args& a) {
   cfg.group_m = a.num("group", cfg.group_m);
   split = a.num("splitk", op == BEAM_OP_SPLITK ? 0 : split);
   Problem p(M, N, K, dtype);
+  if (op == BEAM_OP_MATMUL_NN && cfg.pipeline == 2) cfg.pipeline = 0;
   if (opname == "silu") {
     if (cfg.pipeline == 2) cfg.pipeline = 0;
     return cli_bench_silu(a, p, cfg);

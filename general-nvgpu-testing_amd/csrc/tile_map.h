@@ -37,6 +37,22 @@ BEAM_HD int lds_offset(int row, int chunk) {
   return row * kRowBytes + ((chunk ^ swizzle_of_row(row)) << 4);
 }
 
+// B stored K-major ("NN" layout, B[K][N]): a stage holds kBK rows of block_n 16-bit columns
+// (block_n / 8 chunks of 16 bytes per row).  Fragments are fetched with the transposing read
+// ds_read_b64_tr_b16: in one 32-lane pass the lanes touch 8 different rows k (k & 3 and bit 3 of
+// k vary), 32 contiguous bytes in each, so the 32-byte segment index is XORed with a 3-bit code
+// of exactly those bits of k (2 bits when a row is only 128 bytes and two rows share a bank sweep).
+// The XOR is applied to the chunk index, shifted left by one.
+BEAM_HD int kmajor_swizzle(int k, int block_n) {
+  const int code = block_n >= 128 ? ((k & 3) | (((k >> 3) & 1) << 2)) : (((k >> 1) & 1) | (((k >> 3) & 1) << 1));
+  return code << 1;
+}
+
+// Byte offset inside a K-major stage of element (k, n), n a multiple of 4.
+BEAM_HD int kmajor_lds_offset(int k, int n, int block_n) {
+  return k * block_n * 2 + ((((n >> 3) ^ kmajor_swizzle(k, block_n))) << 4) + ((n & 7) << 1);
+}
+
 struct TileCoord {
   int tm;  // tile index along M
   int tn;  // tile index along N

@@ -159,6 +159,17 @@ int beam_parallel_gemmrc_silu(const void* A, const void* B, void* C, int M, int 
  * reference has no separate entry for it (the formula is cuda/cute_kernels/cute_gemm_ln.cu:191-192). */
 int beam_silu(const void* X, void* Y, long long count, int dtype, void* stream);
 
+/* ---- B stored [K][N] ----------------------------------------------------------------------- */
+
+/* C[M][N] = A[M][K] . B[K][N], all row-major: the layout of the reference's Triton matmul(a, b)
+ * (python/beam/triton_kernels/gemm.py:78-99, kernel :10-76), which torch.matmul callers use.  Same
+ * arithmetic as beam_gemmrc (fp32 accumulation, one rounding to 16 bits); same tile space.  B tiles
+ * are staged in LDS as they lie in memory and transposed on their way into registers
+ * (ds_read_b64_tr_b16), so no transposed copy of B is made.  Requirements beyond beam_gemmrc's:
+ * N % 8 == 0; cfg->pipeline 0 or 1. */
+int beam_matmul_nn(const void* A, const void* B, void* C, int M, int N, int K, int dtype, const beam_tile_cfg* cfg,
+                   void* stream);
+
 /* ---- timing ------------------------------------------------------------------------------- */
 
 /* Which operation beam_bench times. */
@@ -167,7 +178,8 @@ typedef enum beam_op {
   BEAM_OP_SPLITK = 1,
   BEAM_OP_GEMM_LN = 2,
   BEAM_OP_GEMM_SILU = 3, /* beam_parallel_gemmrc_silu */
-  BEAM_OP_SILU = 4       /* beam_silu alone            */
+  BEAM_OP_SILU = 4,      /* beam_silu alone            */
+  BEAM_OP_MATMUL_NN = 5  /* beam_matmul_nn             */
 } beam_op;
 
 typedef struct beam_problem {

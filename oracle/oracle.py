@@ -134,6 +134,12 @@ def gemmrc_ln(a_bits, b_bits, gamma_bits, beta_bits, eps: float = 1e-5, dtype: i
     return y32
 
 
+def matmul_nn(a_bits: np.ndarray, b_kn_bits: np.ndarray, dtype: int = F16) -> np.ndarray:
+    """fp32 C = A . B for B stored [K][N]: the same sum as gemmrc on the transposed copy of B
+    (layout of python/beam/triton_kernels/gemm.py:78-99)."""
+    return gemmrc(a_bits, np.ascontiguousarray(np.asarray(b_kn_bits).T), dtype)
+
+
 def silu(x_bits: np.ndarray, dtype: int = F16):
     """(fp32 values, RN 16-bit bit patterns) of x / (1 + exp(-x)) on a flat 16-bit array."""
     x = np.ascontiguousarray(x_bits, dtype=np.uint16).ravel()

@@ -17,7 +17,7 @@ def test_registry_runs_green(gpu):
     assert os.path.exists(HOST), "beam_host is not built (make -C general-nvgpu-testing_amd/csrc)"
     listed = run("--list").stdout.split()
     assert {"identity_every_tile", "all_ones_ragged", "one_hot_k_tail", "splitk_consistency",
-            "layernorm_invariants", "gemm_silu_side_job", "error_paths"} <= set(listed)
+            "layernorm_invariants", "gemm_silu_side_job", "matmul_nn_every_tile", "error_paths"} <= set(listed)
     r = run("--run", "all")
     assert r.returncode == 0, r.stdout + r.stderr
     assert r.stdout.count("[ OK ]") == len(listed) and "FAIL" not in r.stdout
@@ -34,5 +34,7 @@ def test_cli_bench_and_info(gpu):
     r = run("--bench", "--op", "silu", "--m", "1024", "--n", "1024", "--k", "1024", "--count", "1048579", "--iters", "5",
             "--warmup", "2")
     assert r.returncode == 0 and "gemm+silu in one launch" in r.stdout, r.stdout + r.stderr
+    r = run("--bench", "--op", "nn", "--m", "512", "--n", "1024", "--k", "768", "--iters", "5")
+    assert r.returncode == 0 and r.stdout.startswith("nn 512x1024x768"), r.stdout + r.stderr
     r = run("--bench", "--tile", "100x100")
     assert r.returncode != 0

@@ -174,3 +174,22 @@ def test_config_table(beamc):
     assert (cfg.block_m, cfg.block_n) == (256, 256) and split == 1
     cfg, split = beamc.default_config(256, 256, 32768)
     assert split > 1
+
+
+def test_roofline_calculator():
+    """gemm_flops.py's worked example (A100, fp16, 4096^3 in 512 x 512 x 1024 jobs, C counted twice):
+    flops = 2 * 4096^3 -> 137.44 GFLOP / 312 TFLOP/s = 0.4405 ms; 8 * 8 * 4 = 256 jobs x (512*512 +
+    512*1024 + 2*512*1024) halves x 2 B / 1555 GB/s = 0.6042 ms.  And the MI355X row: the headline shape is
+    matrix-bound by 2731 FLOP/B against a ridge of 315."""
+    from beam import roofline as R
+    r = R.gemm_bound(R.GPU_NAME_SPEC_MAP["A100_{PCIe,SXM}_HBM2"], "fp16", 4096, 4096, 4096, 512, 512, 1024, c_traffic=2)
+    assert r["jobs"] == 256
+    assert abs(r["compute_ms"] - 2 * 4096 ** 3 / 312e12 * 1e3) < 1e-9 and abs(r["compute_ms"] - 0.4405) < 1e-4
+    assert abs(r["memory_ms"] - 0.6042) < 1e-4 and abs(r["memory_ms"] - 256 * (512 * 512 + 512 * 1024 + 2 * 512 * 1024) * 2 / 1555e9 * 1e3) < 1e-9
+    mi = R.GPU_NAME_SPEC_MAP["MI355X"]
+    whole = R.gemm_bound(mi, "fp16", 8192, 8192, 8192, 8192, 8192, 8192)
+    assert abs(whole["intensity"] - 8192 / 3) < 1e-6 and 314 < whole["ridge"] < 316 and whole["ratio"] > 8
+    split = R.gemm_bound(mi, "fp16", 256, 32768, 256, 256, 32768, 256)
+    assert split["ratio"] < 1 and abs(split["memory_ms"] * 1e3 - 4.21) < 0.01  # the 4.2 us HBM floor
+    with pytest.raises(ValueError):
+        R.gemm_bound(mi, "tf32", 64, 64, 64, 64, 64, 64)
