@@ -107,6 +107,7 @@ def _load() -> ctypes.CDLL:
     L.beam_host_fill_normal.argtypes = [vp, sz, i, ctypes.c_uint64, ctypes.c_uint64, ctypes.c_float, ctypes.c_float]
     L.beam_dbg_tile_of_workgroup.argtypes = [i, i, i, i, ctypes.POINTER(i), ctypes.POINTER(i)]
     L.beam_dbg_lds_offset.argtypes = [i, i]
+    L.beam_dbg_kmajor_lds_offset.argtypes = [i, i, i]
     L.beam_dbg_band_block_tile.argtypes = [i, i, i, i, i, ctypes.POINTER(i), ctypes.POINTER(i)]
     L.beam_dbg_band_block_grid.argtypes = [i, i, i]
     return L

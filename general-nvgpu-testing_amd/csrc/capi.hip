@@ -753,6 +753,8 @@ int beam_dbg_tile_of_workgroup(int wg, int tiles_m, int tiles_n, int group_m, in
 
 int beam_dbg_lds_offset(int row, int chunk) { return lds_offset(row, chunk); }
 
+int beam_dbg_kmajor_lds_offset(int k, int n, int block_n) { return kmajor_lds_offset(k, n, block_n); }
+
 int beam_dbg_band_block_tile(int wg, int tiles_m, int tiles_n, int gb, int gc, int* tm, int* tn) {
   if (tiles_m < 1 || tiles_n < 1 || gb < 1 || gc < 1 || wg < 0 || wg >= band_block_grid(tiles_m, gb, gc) || !tm || !tn)
     return fail(BEAM_ERR_INVALID, "bad band-block query");

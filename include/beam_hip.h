@@ -238,6 +238,9 @@ int beam_host_fill_normal(void* dst_host, size_t n, int dtype, uint64_t seed, ui
 int beam_dbg_tile_of_workgroup(int wg, int tiles_m, int tiles_n, int group_m, int* tm, int* tn);
 /* Byte offset of (row, 16-byte chunk) inside an LDS stage. */
 int beam_dbg_lds_offset(int row, int chunk);
+/* Byte offset of element (k, n), n a multiple of 4, inside a K-major LDS stage of block_n columns
+ * (B stored [K][N], beam_matmul_nn). */
+int beam_dbg_kmajor_lds_offset(int k, int n, int block_n);
 /* Workgroup id -> tile of the padded band-block grid used by the fused GEMM+LayerNorm (tm = -1:
  * the id is padding), and the size of that grid. */
 int beam_dbg_band_block_tile(int wg, int tiles_m, int tiles_n, int gb, int gc, int* tm, int* tn);

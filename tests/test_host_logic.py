@@ -75,6 +75,34 @@ def test_lds_swizzle(beamc):
         assert span == list(range(row0 * 128, row0 * 128 + 1024, 16))
 
 
+def test_kmajor_lds_layout_is_bijective_and_conflict_free(beamc):
+    """B stored [K][N]: 64 rows of block_n columns per stage.  The transposing fragment read
+    (ds_read_b64_tr_b16, 8 bytes per lane) is served 32 lanes at a time; lane 16*g + 4*e + q points at row
+    8*g + e (+4 for the second read, +32 for the second K step), columns 4*q .. 4*q+3 of a 16-column
+    block: every such pass must touch each of the 64 banks exactly once.  And the fill side: 64
+    consecutive 16-byte positions hold whole rows' worth of chunks (a permutation within each row), so a
+    wavefront's fill reads whole contiguous row segments from memory."""
+    L = beamc.lib
+    for bn in (64, 128, 256):
+        cpr = bn // 8
+        offs = {L.beam_dbg_kmajor_lds_offset(k, c * 8, bn) for k in range(64) for c in range(cpr)}
+        assert offs == set(range(0, 64 * bn * 2, 16))
+        for k in range(64):
+            row = sorted(L.beam_dbg_kmajor_lds_offset(k, c * 8, bn) for c in range(cpr))
+            assert row == list(range(k * bn * 2, (k + 1) * bn * 2, 16))
+            assert all(L.beam_dbg_kmajor_lds_offset(k, c * 8 + 4, bn) == L.beam_dbg_kmajor_lds_offset(k, c * 8, bn) + 8
+                       for c in range(cpr))
+        for n0 in range(0, bn, 16):
+            for kbase in (0, 4, 32, 36):
+                for half in (0, 32):
+                    banks = []
+                    for lane in range(half, half + 32):
+                        g, e, q = lane >> 4, (lane >> 2) & 3, lane & 3
+                        o = L.beam_dbg_kmajor_lds_offset(kbase + 8 * g + e, n0 + 4 * q, bn)
+                        banks += [(o // 4) % 64, (o // 4 + 1) % 64]
+                    assert sorted(banks) == list(range(64)), (bn, n0, kbase, half)
+
+
 def test_slice_heuristic_matches_reference_rule(beamc, oracle):
     for units in (108, 256):
         for tiles in range(1, units + 2):
