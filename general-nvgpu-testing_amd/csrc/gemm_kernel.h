@@ -185,6 +185,7 @@ struct GemmTile {
   static_assert(AST >= 2 && BST >= 2 && (AST == BST || AST == BST + 1), "slot counts");
   static_assert(LDS_BYTES <= 160 * 1024, "LDS budget of one CU");
   static_assert(WAIT_STEADY < 64, "vmcnt range");
+  static_assert(BM * 8 * (4 * WAVES_N + 2) <= LDS_BYTES, "row statistics scratch of the LayerNorm epilogues");
 
   // Chunk q = i * NT + tid of an operand tile lives at LDS byte q * 16 of its slot, which is
   // row q / 8, position q % 8; the position holds logical chunk position ^ swizzle_of_row(row).
@@ -524,8 +525,12 @@ struct GemmTile {
     // thread per row merges the 4*WAVES_N pairs in a fixed order with Chan's update: no cross-lane
     // shuffles (they go through the LDS crossbar one at a time) and no cancellation.
     // Result: row_stats[rl] = (mean, M2) over the tile's valid columns, for rl in [0, BM).
-    auto tile_row_stats = [&](float* part /* [BM][4*WAVES_N][2] */, float* row_stats /* [BM][2] */) {
+    // A row of `part` is padded by one pair: its stride in 4-byte words is then twice an odd number, so
+    // the 32 lanes of a pass (consecutive rows, one 8-byte pair each) fall on 32 different bank pairs,
+    // both when the lanes drop their pairs and when one thread per row walks its row.
+    auto tile_row_stats = [&](float* part /* [BM][4*WAVES_N + 1][2] */, float* row_stats /* [BM][2] */) {
       constexpr int SLOTS = 4 * WAVES_N;
+      constexpr int PITCH = SLOTS + 1;  // pairs per row of `part`
       const int n_lane0 = col0 + wn * TN + 4 * (lane >> 4);  // first column of this lane
       const bool full = (col0 + BN <= N);
 #pragma unroll
@@ -566,8 +571,8 @@ struct GemmTile {
         }
         const int rl = wm * TM + i * 16 + (lane & 15);
         const int slot = wn * 4 + (lane >> 4);
-        part[(rl * SLOTS + slot) * 2 + 0] = mean;
-        part[(rl * SLOTS + slot) * 2 + 1] = m2;
+        part[(rl * PITCH + slot) * 2 + 0] = mean;
+        part[(rl * PITCH + slot) * 2 + 1] = m2;
       }
       __syncthreads();
       for (int rl = tid; rl < BM; rl += NT) {
@@ -586,8 +591,8 @@ struct GemmTile {
             }
             if (cnt == 0) continue;
           }
-          const float mw = part[(rl * SLOTS + slot) * 2 + 0];
-          const float qw = part[(rl * SLOTS + slot) * 2 + 1];
+          const float mw = part[(rl * PITCH + slot) * 2 + 0];
+          const float qw = part[(rl * PITCH + slot) * 2 + 1];
           const float nb = (float)cnt;
           const float tot = n_acc + nb;
           const float delta = mw - mean;
@@ -669,7 +674,7 @@ struct GemmTile {
       // 1. per-row (mean, M2) over this tile's columns
       __syncthreads();            // every LDS slot is dead; reuse the space
       float* red = (float*)smem;   // [BM][2] tile statistics, later (mean, rstd) of the whole row
-      float* part = red + BM * 2;  // [BM][4*WAVES_N][2], then reused as `gathered`
+      float* part = red + BM * 2;  // [BM][4*WAVES_N + 1][2], then reused as `gathered`
       tile_row_stats(part, red);
       // 2. publish the tile's statistics: stats[band][tile_n][row] = (mean, M2) as one 8-byte
       //    device-scope atomic store.  Such stores go straight through the XCD-private L2 to memory
@@ -769,7 +774,7 @@ struct GemmTile {
         // Per-row statistics over the columns this workgroup owns, from the fp32 accumulators.
         __syncthreads();  // every LDS slot is dead; reuse the space
         float* row_stats = (float*)smem;   // [BM][2]
-        float* part = row_stats + BM * 2;  // [BM][4*WAVES_N][2]
+        float* part = row_stats + BM * 2;  // [BM][4*WAVES_N + 1][2]
         tile_row_stats(part, row_stats);
         for (int rl = tid; rl < BM; rl += NT) {
           const int m = row0 + rl;
