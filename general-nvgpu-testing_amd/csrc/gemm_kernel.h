@@ -450,9 +450,11 @@ struct GemmTile {
         }
 #pragma unroll
         for (int jj = 0; jj < FN; ++jj) {
-          // boustrophedon: consecutive MFMAs always share one operand (fewer input toggles: about 2%
-          // more throughput under the power cap in a register-only loop)
-          const int j = (i & 1) ? FN - 1 - jj : jj;
+          // With two wavefronts per SIMD the rows walk the B fragments boustrophedon: consecutive
+          // MFMAs then always share one operand (fewer input toggles: about 2% more throughput under
+          // the power cap in a register-only loop, 1% here).  A wavefront that has its SIMD to itself
+          // loses 5-7% that way (measured), so 4-wavefront tiles keep the plain order.
+          const int j = (NW >= 8 && (i & 1)) ? FN - 1 - jj : jj;
           acc[i][j] = Traits::mfma(fb_cur[j], fa_cur[i], acc[i][j]);
         }
         if constexpr (SIDE && ROW0 != 0) {  // step 1: this row's share of the side vector
