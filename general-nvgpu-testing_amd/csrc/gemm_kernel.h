@@ -584,6 +584,26 @@ struct GemmTile {
       __syncthreads();
       for (int rl = tid; rl < BM; rl += NT) {
         float mean = 0.0f, m2 = 0.0f, n_acc = 0.0f;
+        if (full) {
+          // every slot covers FN * 4 columns: the mean of the slot means, then M2 about it -- the same
+          // merge as below for equal counts, in the same fixed order, without its divisions
+          float mw[SLOTS], qw[SLOTS];
+#pragma unroll
+          for (int slot = 0; slot < SLOTS; ++slot) {
+            mw[slot] = part[(rl * PITCH + slot) * 2 + 0];
+            qw[slot] = part[(rl * PITCH + slot) * 2 + 1];
+            mean += mw[slot];
+          }
+          mean *= 1.0f / (float)SLOTS;
+#pragma unroll
+          for (int slot = 0; slot < SLOTS; ++slot) {
+            const float d = mw[slot] - mean;
+            m2 += qw[slot] + (float)(FN * 4) * d * d;
+          }
+          row_stats[rl * 2 + 0] = mean;
+          row_stats[rl * 2 + 1] = m2;
+          continue;
+        }
 #pragma unroll
         for (int slot = 0; slot < SLOTS; ++slot) {
           // valid columns of this (wavefront, lane group): 4 per 16-wide block, clipped at N
@@ -733,8 +753,20 @@ struct GemmTile {
       }
       __syncthreads();
       // 4. merge in tile order -> (mean, rstd) per row
+      const bool even_tiles = (N % BN) == 0;  // every column tile is full: equal weights
       for (int rl = tid; rl < BM; rl += NT) {
         float mean = 0.0f, m2 = 0.0f, n_acc = 0.0f;
+        if (even_tiles) {
+          for (int t = 0; t < p.tiles_n; ++t) mean += gathered[((size_t)t * BM + rl) * 2 + 0];
+          mean *= 1.0f / (float)p.tiles_n;
+          for (int t = 0; t < p.tiles_n; ++t) {
+            const float d = gathered[((size_t)t * BM + rl) * 2 + 0] - mean;
+            m2 += gathered[((size_t)t * BM + rl) * 2 + 1] + (float)BN * d * d;
+          }
+          red[rl * 2 + 0] = mean;
+          red[rl * 2 + 1] = __builtin_amdgcn_rsqf(m2 * (1.0f / (float)N) + p.eps);
+          continue;
+        }
         for (int t = 0; t < p.tiles_n; ++t) {
           int cw = N - t * BN;
           cw = cw > BN ? BN : cw;
