@@ -156,8 +156,8 @@ def main():
     ap.add_argument("--no-extra", action="store_true", help="skip the split-K and GEMM+LN companions")
     args = ap.parse_args()
     if args.gpus != 1:
-        sys.exit("bench.py: this build runs on ONE GPU (the gemmrc path needs no exchange between GPUs; "
-                 "see DESIGN.md for how it would shard). Re-run with --gpus 1.")
+        sys.exit("bench.py: this build runs on ONE GPU (the gemmrc path needs no exchange between GPUs: rows of A "
+                 "and C would be sharded, B replicated). Re-run with --gpus 1.")
 
     from beam import _C  # fails loudly if libbeam_hip.so is missing; there is no fallback
 

@@ -79,7 +79,10 @@ const KernelSet* find_set(const beam_tile_cfg& c) {
 }
 
 constexpr int kDefaultGroupM = 8;
-constexpr int kMaxK = 1 << 22;
+// Largest K: the buffer descriptor of a 256-row operand tile, (255 * K + K) * 2 bytes, must stay below the
+// out-of-range offset the kernels use for masked chunks (kOobOffset).
+constexpr int kMaxK = (int)((kOobOffset / 512u) & ~7u) - 8;
+static_assert((unsigned long long)kMaxK * 512ull < kOobOffset && kMaxK % 8 == 0, "descriptor range");
 
 // Elements of a side-job array: its byte size must stay below the out-of-range offset the kernels use.
 constexpr long long kMaxSideElems = (long long)(kOobOffset / 16) * 8;
@@ -348,6 +351,7 @@ int beam_matmul_nn(const void* A, const void* B, void* C, int M, int N, int K, i
   if (rc) return rc;
   if (M == 0 || N == 0) return BEAM_OK;
   if (N % 8 != 0) return fail(BEAM_ERR_UNSUPPORTED, "N=%d: rows of B must be multiples of 16 bytes (N %% 8 == 0)", N);
+  if (N > (1 << 24)) return fail(BEAM_ERR_UNSUPPORTED, "N=%d exceeds %d (64 rows of B per buffer descriptor)", N, 1 << 24);
   if ((rc = beam_init())) return rc;
   hipStream_t st = (hipStream_t)stream;
   if (K == 0) {
