@@ -66,13 +66,49 @@ def cpu_baseline(a_bits, b_bits, M, N, K):
     return rec, ref, O
 
 
+def splitk_graph_us(_C, a, b, c, cfg, s, calls=50, replays=10):
+    """Microseconds per split-K call when `calls` of them are captured once and replayed as a HIP graph."""
+    import ctypes
+    L, chk = _C.lib, _C._check
+    M, K = a.shape
+    N = b.shape[0]
+    cc = cfg.to_c()
+    eff = L.beam_splitk_effective(M, N, K, ctypes.byref(cc), s)
+    ws = _C.DeviceArray((max(L.beam_splitk_workspace_bytes(M, N, eff), 256),), _C.F16, 1)
+    stream, graph, e0, e1 = (ctypes.c_void_p() for _ in range(4))
+    chk(L.beam_stream_create(ctypes.byref(stream)))
+    call = lambda st: chk(L.beam_gemmrc_splitk(a.ptr, b.ptr, c.ptr, M, N, K, _C.F16, ctypes.byref(cc), s, ws.ptr, ws.nbytes, st))
+    call(None)
+    _C.sync()
+    chk(L.beam_graph_begin_capture(stream))
+    for _ in range(calls):
+        call(stream)
+    chk(L.beam_graph_end_capture(stream, ctypes.byref(graph)))
+    chk(L.beam_event_create(ctypes.byref(e0)))
+    chk(L.beam_event_create(ctypes.byref(e1)))
+    for _ in range(3):
+        chk(L.beam_graph_launch(graph, stream))
+    chk(L.beam_event_record(e0, stream))
+    for _ in range(replays):
+        chk(L.beam_graph_launch(graph, stream))
+    chk(L.beam_event_record(e1, stream))
+    ms = ctypes.c_float()
+    chk(L.beam_event_elapsed_ms(e0, e1, ctypes.byref(ms)))
+    for e in (e0, e1):
+        L.beam_event_destroy(e)
+    chk(L.beam_graph_destroy(graph))
+    chk(L.beam_stream_destroy(stream))
+    ws.free()
+    return ms.value * 1e3 / (calls * replays)
+
+
 def extra_splitk(_C):
     """split-K at 256x256x32768: best (tile, S) against the best non-split tile."""
     M, N, K = 256, 256, 32768
     a = _C.DeviceArray.from_numpy(_C.host_uniform((M, K), _C.F16, 11, 0))
     b = _C.DeviceArray.from_numpy(_C.host_uniform((N, K), _C.F16, 11, 1))
     c = _C.DeviceArray((M, N))
-    best_plain, best_split = (None, 1e30), (None, 1e30)
+    best_plain, best_split = (None, 1e30), (None, 1e30, None, 0)
     for cfg in _C.list_configs():
         ms = _C.bench(0, a, b, c, config=cfg, warmup=3, iters=20)
         if ms < best_plain[1]:
@@ -84,11 +120,13 @@ def extra_splitk(_C):
             for s in (4, 8, 16, 32, 64):
                 ms = _C.bench(1, a, b, c, config=pc, split_k=s, warmup=3, iters=20)
                 if ms < best_split[1]:
-                    best_split = (f"{pc.name},S={s}", ms)
+                    best_split = (f"{pc.name},S={s}", ms, pc, s)
+    graph_us = splitk_graph_us(_C, a, b, c, best_split[2], best_split[3])
     for x in (a, b, c):
         x.free()
     bytes_alg = 2.0 * (M * K + N * K + M * N)
     return {"shape": [M, N, K], "splitk_us": round(best_split[1] * 1e3, 2), "splitk_config": best_split[0],
+            "splitk_in_graph_us": round(graph_us, 2),
             "best_nonsplit_us": round(best_plain[1] * 1e3, 2), "best_nonsplit_config": best_plain[0],
             "speedup": round(best_plain[1] / best_split[1], 2),
             "hbm_GBs": round(bytes_alg / (best_split[1] * 1e-3) / 1e9, 1),

@@ -92,6 +92,12 @@ def _load() -> ctypes.CDLL:
     L.beam_silu.argtypes = [vp, vp, ctypes.c_longlong, i, vp]
     L.beam_matmul_nn.argtypes = [vp, vp, vp, i, i, i, i, cfgp, vp]
     L.beam_bench.argtypes = [i, ctypes.POINTER(_Problem), cfgp, i, i, vp, ctypes.POINTER(ctypes.c_float)]
+    L.beam_stream_create.argtypes = [ctypes.POINTER(vp)]
+    L.beam_stream_destroy.argtypes = [vp]
+    L.beam_graph_begin_capture.argtypes = [vp]
+    L.beam_graph_end_capture.argtypes = [vp, ctypes.POINTER(vp)]
+    L.beam_graph_launch.argtypes = [vp, vp]
+    L.beam_graph_destroy.argtypes = [vp]
     L.beam_event_create.argtypes = [ctypes.POINTER(vp)]
     L.beam_event_record.argtypes = [vp, vp]
     L.beam_event_elapsed_ms.argtypes = [vp, vp, ctypes.POINTER(ctypes.c_float)]

@@ -20,6 +20,8 @@ hipError_t launch_ln_apply(const float* X, const float* stats, const void* gamma
 // y[i] (16-bit) = silu(x[i]) for i in [0, count); x and y 16-byte aligned.
 hipError_t launch_silu(const void* x, void* y, size_t count, int dtype, hipStream_t stream);
 
+// 16-bit p[0 .. n) = 0: what an operator with K = 0 writes (a kernel, so that the call can be captured in a graph)
+hipError_t launch_zero_u16(void* p, size_t n, hipStream_t stream);
 // ints[0 .. n) = 0 (a fill kernel rather than hipMemsetAsync, so that callers may capture it in a graph).
 hipError_t launch_zero_ints(int* ints, int n, hipStream_t stream);
 // floats[0 .. n) = value

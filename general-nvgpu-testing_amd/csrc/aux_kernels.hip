@@ -125,6 +125,10 @@ __global__ void __launch_bounds__(256) silu_kernel(const T* __restrict__ x, T* _
   if (i < count) y[i] = silu_16<T>(x[i]);
 }
 
+__global__ void zero_u16_kernel(unsigned short* p, size_t n) {
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) p[i] = 0;
+}
+
 __global__ void zero_ints_kernel(int* p, int n) {
   for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x) p[i] = 0;
 }
@@ -150,6 +154,14 @@ hipError_t launch_silu(const void* x, void* y, size_t count, int dtype, hipStrea
 
 hipError_t launch_fill_floats(float* floats, size_t n, float value, hipStream_t stream) {
   hipLaunchKernelGGL(fill_floats_kernel, dim3(256), dim3(256), 0, stream, floats, n, value);
+  return hipGetLastError();
+}
+
+hipError_t launch_zero_u16(void* p, size_t n, hipStream_t stream) {
+  size_t blocks = (n + 255) / 256;
+  if (blocks < 1) blocks = 1;
+  if (blocks > 4096) blocks = 4096;
+  hipLaunchKernelGGL(zero_u16_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, (unsigned short*)p, n);
   return hipGetLastError();
 }
 

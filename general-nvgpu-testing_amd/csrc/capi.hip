@@ -333,7 +333,7 @@ int beam_gemmrc(const void* A, const void* B, void* C, int M, int N, int K, int 
   if ((rc = beam_init())) return rc;
   hipStream_t st = (hipStream_t)stream;
   if (K == 0) {
-    BEAM_HIP(hipMemsetAsync(C, 0, (size_t)M * N * 2, st));
+    BEAM_HIP(launch_zero_u16(C, (size_t)M * N, st));
     return BEAM_OK;
   }
   beam_tile_cfg c;
@@ -355,7 +355,7 @@ int beam_matmul_nn(const void* A, const void* B, void* C, int M, int N, int K, i
   if ((rc = beam_init())) return rc;
   hipStream_t st = (hipStream_t)stream;
   if (K == 0) {
-    BEAM_HIP(hipMemsetAsync(C, 0, (size_t)M * N * 2, st));
+    BEAM_HIP(launch_zero_u16(C, (size_t)M * N, st));
     return BEAM_OK;
   }
   beam_tile_cfg c;
@@ -466,7 +466,7 @@ int beam_gemmrc_splitk(const void* A, const void* B, void* C, int M, int N, int 
   if ((rc = beam_init())) return rc;
   hipStream_t st = (hipStream_t)stream;
   if (K == 0) {
-    BEAM_HIP(hipMemsetAsync(C, 0, (size_t)M * N * 2, st));
+    BEAM_HIP(launch_zero_u16(C, (size_t)M * N, st));
     return BEAM_OK;
   }
   beam_tile_cfg c;
@@ -548,6 +548,16 @@ int beam_gemmrc_ln_ex(const void* A, const void* B, const void* gamma, const voi
   if (c.pipeline == 2) c.pipeline = 0;  // the deep pipeline exists for the store / split-K kernels only
   if (mode == BEAM_LN_FUSED && !ln_fused_applies(c, *ks, N))
     return fail(BEAM_ERR_UNSUPPORTED, "fused LayerNorm: too many column tiles for this tile shape (N=%d, block_n=%d)", N, c.block_n);
+  // A fused launch depends on how many launches its workspace has seen (the two statistics sets
+  // alternate), which a captured graph would freeze: under stream capture AUTO takes the two-pass
+  // path and an explicit FUSED is refused.
+  hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+  if (st != nullptr) (void)hipStreamIsCapturing(st, &capturing);
+  if (capturing != hipStreamCaptureStatusNone) {
+    if (mode == BEAM_LN_FUSED)
+      return fail(BEAM_ERR_UNSUPPORTED, "fused GEMM+LayerNorm cannot be captured in a graph (use BEAM_LN_TWOPASS or BEAM_LN_AUTO)");
+    mode = BEAM_LN_TWOPASS;
+  }
   mode = ln_resolve_mode(mode, c, *ks, N);
   const size_t need = beam_gemmrc_ln_workspace_bytes_ex(M, N, &c, mode);
   if (!ws || ws_bytes < need)
@@ -679,6 +689,49 @@ int beam_bench(int op, const beam_problem* q, const beam_tile_cfg* cfg, int warm
   if (rc) return rc;
   if (he != hipSuccess) return hip_fail(he, "event timing");
   *avg_ms = ms / (float)iters;
+  return BEAM_OK;
+}
+
+int beam_stream_create(void** stream) {
+  if (!stream) return fail(BEAM_ERR_INVALID, "null stream pointer");
+  int rc = beam_init();
+  if (rc) return rc;
+  hipStream_t s;
+  BEAM_HIP(hipStreamCreate(&s));  // default priority
+  *stream = s;
+  return BEAM_OK;
+}
+
+int beam_stream_destroy(void* stream) {
+  BEAM_HIP(hipStreamDestroy((hipStream_t)stream));
+  return BEAM_OK;
+}
+
+int beam_graph_begin_capture(void* stream) {
+  if (!stream) return fail(BEAM_ERR_INVALID, "the default stream cannot be captured");
+  BEAM_HIP(hipStreamBeginCapture((hipStream_t)stream, hipStreamCaptureModeThreadLocal));
+  return BEAM_OK;
+}
+
+int beam_graph_end_capture(void* stream, void** graph_exec) {
+  if (!graph_exec) return fail(BEAM_ERR_INVALID, "null graph pointer");
+  hipGraph_t g = nullptr;
+  BEAM_HIP(hipStreamEndCapture((hipStream_t)stream, &g));
+  hipGraphExec_t e = nullptr;
+  hipError_t err = hipGraphInstantiate(&e, g, nullptr, nullptr, 0);
+  (void)hipGraphDestroy(g);
+  if (err != hipSuccess) return hip_fail(err, "hipGraphInstantiate");
+  *graph_exec = e;
+  return BEAM_OK;
+}
+
+int beam_graph_launch(void* graph_exec, void* stream) {
+  BEAM_HIP(hipGraphLaunch((hipGraphExec_t)graph_exec, (hipStream_t)stream));
+  return BEAM_OK;
+}
+
+int beam_graph_destroy(void* graph_exec) {
+  BEAM_HIP(hipGraphExecDestroy((hipGraphExec_t)graph_exec));
   return BEAM_OK;
 }
 

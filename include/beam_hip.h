@@ -211,6 +211,23 @@ int beam_event_record(void* event, void* stream);
 int beam_event_elapsed_ms(void* start, void* stop, float* ms);
 int beam_event_destroy(void* event);
 
+/* ---- streams and graphs (so that hosts need no other GPU runtime) -------------------------- */
+
+/* Every operator above is one or two kernel launches on the caller's stream and neither allocates nor
+ * synchronises, so a sequence of them can be captured once and replayed as a HIP graph: the usual cure
+ * for launch-bound loops of small GEMMs (a split-K call is two kernels of 13 and 5 us).  The reference
+ * has no counterpart (it launches on the legacy default stream, cuda/cute_kernels/cute_gemm_128x128.cu:
+ * 203).  Rules: call every operator once eagerly before capturing it (the first launch of a kernel
+ * configures its LDS size); the fused GEMM+LayerNorm keeps launch-to-launch state in its workspace and is
+ * refused under capture (BEAM_LN_AUTO takes the two-pass path there); K = 0 clears C with a kernel, not
+ * a memset node.  Streams are created at the default priority. */
+int beam_stream_create(void** stream);
+int beam_stream_destroy(void* stream);
+int beam_graph_begin_capture(void* stream);               /* not the default stream */
+int beam_graph_end_capture(void* stream, void** graph_exec);
+int beam_graph_launch(void* graph_exec, void* stream);
+int beam_graph_destroy(void* graph_exec);
+
 /* ---- device memory (so that hosts need no other GPU runtime) ------------------------------ */
 
 int beam_malloc(void** dptr, size_t bytes);
