@@ -2,6 +2,8 @@
 // normalisation pass.  Both stream fp32 from the workspace once and write 16-bit once.
 #include "aux_kernels.h"
 
+#include <type_traits>
+
 #include "elementwise.h"
 
 namespace beam {
@@ -28,17 +30,28 @@ __global__ void __launch_bounds__(64) splitk_reduce_kernel(const float* __restri
   const size_t stride = (size_t)gridDim.x * blockDim.x;
   for (size_t q = (size_t)blockIdx.x * blockDim.x + threadIdx.x; q < quads; q += stride) {
     const float* src = ws + q * 4;
-    f32x4 s = *(const f32x4*)src;
-    int z = 1;
-    // eight independent loads in flight, added in slice order
-    for (; z + 8 <= splits; z += 8) {
-      f32x4 v[8];
+    f32x4 s = {0.0f, 0.0f, 0.0f, 0.0f};
+    int z = 0;
+    // Batches of 16, 8, 4, 2, 1 slices: all loads of a batch in flight before the first add, the
+    // adds in slice order (slice 0 starts the sum, so that the sign of an all-zero sum is kept).
+    auto batch = [&](auto n_tag) {
+      constexpr int NB = decltype(n_tag)::value;
+      while (z + NB <= splits) {
+        f32x4 v[NB];
 #pragma unroll
-      for (int u = 0; u < 8; ++u) v[u] = *(const f32x4*)(src + (size_t)(z + u) * mn);
+        for (int u = 0; u < NB; ++u) v[u] = *(const f32x4*)(src + (size_t)(z + u) * mn);
+        if (z == 0) s = v[0];
+        else s += v[0];
 #pragma unroll
-      for (int u = 0; u < 8; ++u) s += v[u];
-    }
-    for (; z < splits; ++z) s += *(const f32x4*)(src + (size_t)z * mn);
+        for (int u = 1; u < NB; ++u) s += v[u];
+        z += NB;
+      }
+    };
+    batch(std::integral_constant<int, 16>{});
+    batch(std::integral_constant<int, 8>{});
+    batch(std::integral_constant<int, 4>{});
+    batch(std::integral_constant<int, 2>{});
+    batch(std::integral_constant<int, 1>{});
     vec4 o;
 #pragma unroll
     for (int e = 0; e < 4; ++e) o[e] = (T)s[e];
