@@ -121,7 +121,7 @@ class OperatorTuner:
     def _get_gemm_specs(self) -> List[Operator]:
         ret = []
         for cfg in _C.list_configs():
-            for group_m in (4, 8, 16):
+            for group_m in (2, 4, 8, 16):
                 full = _C.TileConfig(cfg.block_m, cfg.block_n, cfg.wave_m, cfg.wave_n, 0, group_m)
                 ret.append(Operator(
                     partial(_C.gemmrc_spec, shape_threadblock=[cfg.block_m, cfg.block_n],
