@@ -437,11 +437,13 @@ struct GemmTile {
           }
         }
         if constexpr (B_KMAJOR) {
-          // Row 0: everything the previous step read must have arrived; only the LDS reads issued
-          // just above (two per B fragment, one per A fragment) may still be in flight.
+          // Row 0: everything the previous step read must have arrived; only the transposing reads
+          // issued just above (two per B fragment of this row) may still be in flight.  The row's A
+          // fragment reads are not counted: the scheduler may place them on either side of this wait,
+          // and counting one that ends up behind it would let a read of the previous step slip through.
           if (i == 0) {
             constexpr int B_NOW = PER_READ_ROW < FN ? PER_READ_ROW : FN;
-            constexpr int NOW = (PER_READ_ROW < READS ? PER_READ_ROW : READS) + B_NOW;
+            constexpr int NOW = 2 * B_NOW;
             wait_lds<(NOW < 15 ? NOW : 15)>();
             // ... and the MFMAs must not be moved above that wait: tie their B operands to it.
 #pragma unroll
@@ -470,6 +472,21 @@ struct GemmTile {
           const int l = (ROW0 + i) * PER_ROW + u;  // B first: it is needed one tile sooner
           if (l < LB) load_b(l, h + BST - 1);
           else if (l < LOADS) load_a(l - LB, h + AST - 1);
+        }
+        // Inside the row: MFMA, LDS read, MFMA, LDS read, MFMA, the rest of the reads, buffer load, the
+        // remaining MFMAs.  A read or load issued between two MFMAs costs no matrix-core time (an MFMA
+        // occupies its issue port for a quarter of its 16 cycles), whereas in front of the row it delays
+        // the row's first MFMA: +1 to 3% on most tiles.  The 128x128 wavefront tile (a lone wavefront per
+        // SIMD, 8 MFMAs a row) loses 13% with it and keeps reads-first.
+        if constexpr (FN >= 4 && FM * FN < 64) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+          __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x008, FN - 3, 0);
         }
         __builtin_amdgcn_sched_barrier(0);
       }
