@@ -157,6 +157,13 @@ struct GemmTile {
 
   static constexpr int NW = WAVES_M * WAVES_N;
   static constexpr int NT = NW * 64;
+  // Wavefronts that issue the global->LDS loads.  With two wavefronts per SIMD the hardware favours the
+  // older one of each pair (wavefronts 0 .. NW/2-1) when both have an MFMA ready, so those finish a K tile
+  // early and idle at the barrier while the younger ones are the critical path: the older half therefore
+  // issues every load, two wavefronts' worth each, and the younger half none (8192^3: +3.7%; on all-zero
+  // data, where the power cap does not hide it, +21%).
+  static constexpr int LDW = NW >= 8 ? NW / 2 : NW;
+  static constexpr int NTL = LDW * 64;  // threads that issue loads
   static constexpr int TM = BM / WAVES_M;  // wavefront tile
   static constexpr int TN = BN / WAVES_N;
   static constexpr int FM = TM / 16;       // MFMA blocks per wavefront tile
@@ -166,8 +173,8 @@ struct GemmTile {
   static constexpr int B_BYTES = BN * kRowBytes;
   static constexpr int B_REGION = AST * A_BYTES;  // A slots first, then B slots
   static constexpr int LDS_BYTES = AST * A_BYTES + BST * B_BYTES;
-  static constexpr int LA = (BM * kChunksPerRow) / NT;  // buffer loads per wavefront per A tile
-  static constexpr int LB = (BN * kChunksPerRow) / NT;
+  static constexpr int LA = (BM * kChunksPerRow) / NTL;  // buffer loads per wavefront per A tile
+  static constexpr int LB = (BN * kChunksPerRow) / NTL;
   static constexpr int LOADS = LA + LB;
   static constexpr int ROWS = KSTEPS * FM;                 // rows of MFMAs per K tile
   static constexpr int PER_ROW = (LOADS + ROWS - 1) / ROWS;  // buffer loads issued after each row
@@ -180,14 +187,14 @@ struct GemmTile {
 
   static_assert(KSTEPS == 2, "the step pipeline below is written for two 32-wide steps per tile");
   static_assert(TM % 16 == 0 && TN % 16 == 0, "wavefront tile must be made of 16x16 blocks");
-  static_assert((BM * kChunksPerRow) % NT == 0 && (BN * kChunksPerRow) % NT == 0,
+  static_assert((BM * kChunksPerRow) % NTL == 0 && (BN * kChunksPerRow) % NTL == 0,
                 "every wavefront must move a whole number of 1 KiB chunks per tile");
   static_assert(AST >= 2 && BST >= 2 && (AST == BST || AST == BST + 1), "slot counts");
   static_assert(LDS_BYTES <= 160 * 1024, "LDS budget of one CU");
   static_assert(WAIT_STEADY < 64, "vmcnt range");
   static_assert(BM * 8 * (4 * WAVES_N + 2) <= LDS_BYTES, "row statistics scratch of the LayerNorm epilogues");
 
-  // Chunk q = i * NT + tid of an operand tile lives at LDS byte q * 16 of its slot, which is
+  // Chunk q = i * NTL + tid of an operand tile lives at LDS byte q * 16 of its slot, which is
   // row q / 8, position q % 8; the position holds logical chunk position ^ swizzle_of_row(row).
   static __device__ __forceinline__ unsigned chunk_voffset(int q, int K) {
     const int row = q >> 3;
@@ -247,18 +254,18 @@ struct GemmTile {
 
     unsigned voff_a[LA], voff_b[LB];
 #pragma unroll
-    for (int i = 0; i < LA; ++i) voff_a[i] = chunk_voffset(i * NT + tid, K);
+    for (int i = 0; i < LA; ++i) voff_a[i] = chunk_voffset(i * NTL + tid, K);
 #pragma unroll
     for (int i = 0; i < LB; ++i) {
       if (B_KMAJOR) {
         // LDS position q of the stage: row k = q / CPR, and the chunk that lives there is position ^ swizzle
         constexpr int CPR = BN / 8;
-        const int q = i * NT + tid;
+        const int q = i * NTL + tid;
         const int k = q / CPR;
         const int chunk = (q % CPR) ^ kmajor_swizzle(k, BN);
         voff_b[i] = ((unsigned)k * (unsigned)N + (unsigned)chunk * 8u) * 2u;
       } else {
-        voff_b[i] = chunk_voffset(i * NT + tid, K);
+        voff_b[i] = chunk_voffset(i * NTL + tid, K);
       }
     }
 
@@ -270,13 +277,13 @@ struct GemmTile {
     // of the K range get an empty descriptor: the load is still issued and counted (the pipeline below
     // has no special cases for its last iterations) but touches no memory.
     auto load_a = [&](int i, int t) {
-      char* dst = smem + (t % AST) * A_BYTES + wave * 1024 + i * (NT * 16);
+      char* dst = smem + (t % AST) * A_BYTES + wave * 1024 + i * (NTL * 16);
       const __amdgpu_buffer_rsrc_t r = make_rsrc(a_base, t < n_tiles ? bytes_a : 0u);
       __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (__attribute__((address_space(3))) void*)dst, 16,
                                                (int)voff_a[i], tile_koff(t) * 2, 0, 0);
     };
     auto load_b = [&](int i, int t) {
-      char* dst = smem + B_REGION + (t % BST) * B_BYTES + wave * 1024 + i * (NT * 16);
+      char* dst = smem + B_REGION + (t % BST) * B_BYTES + wave * 1024 + i * (NTL * 16);
       if (B_KMAJOR) {
         // Rows koff .. koff + kBK of the slice, as many as exist: rows past the end of K and the
         // columns past the last row's end are out of range and read as zeros.  (Columns past N in
@@ -296,12 +303,14 @@ struct GemmTile {
     };
     // The short tile goes through registers so that chunks at or past `kvalid` are zero-filled.
     // (A K-major B needs none of this: its rows past the end of K are out of range by themselves.)
+    const bool loader = LDW == NW || wave < LDW;
     auto fill_short_tile = [&](int kvalid) {
+      if (!loader) return;
       const int koff = tile_koff(0);
       i32x4 ra[LA], rb[LB];
 #pragma unroll
       for (int i = 0; i < LA; ++i) {
-        const int q = i * NT + tid;
+        const int q = i * NTL + tid;
         const int chunk = (q & 7) ^ swizzle_of_row(q >> 3);
         const unsigned off = (chunk * 8 < kvalid) ? voff_a[i] + (unsigned)koff * 2u : kOobOffset;
         ra[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_a, (int)off, 0, 0);
@@ -309,7 +318,7 @@ struct GemmTile {
       if (!B_KMAJOR) {
 #pragma unroll
         for (int i = 0; i < LB; ++i) {
-          const int q = i * NT + tid;
+          const int q = i * NTL + tid;
           const int chunk = (q & 7) ^ swizzle_of_row(q >> 3);
           const unsigned off = (chunk * 8 < kvalid) ? voff_b[i] + (unsigned)koff * 2u : kOobOffset;
           rb[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, (int)off, 0, 0);
@@ -318,10 +327,10 @@ struct GemmTile {
       char* sa = smem + tid * 16;
       char* sb = smem + B_REGION + tid * 16;
 #pragma unroll
-      for (int i = 0; i < LA; ++i) *(i32x4*)(sa + i * (NT * 16)) = ra[i];
+      for (int i = 0; i < LA; ++i) *(i32x4*)(sa + i * (NTL * 16)) = ra[i];
       if (!B_KMAJOR) {
 #pragma unroll
-        for (int i = 0; i < LB; ++i) *(i32x4*)(sb + i * (NT * 16)) = rb[i];
+        for (int i = 0; i < LB; ++i) *(i32x4*)(sb + i * (NTL * 16)) = rb[i];
       }
     };
 
@@ -421,8 +430,9 @@ struct GemmTile {
     // registers across the two sets, and the step then starts by waiting for its own reads.
     //   ROW0: index of the step's first row inside the tile (the loads are dealt out row by row).
     auto step = [&](const char* sa, const char* sb, vec8(&fa_cur)[FM], vec8(&fa_nxt)[FM], vec8(&fb_cur)[FN],
-                    vec8(&fb_nxt)[FN], int h, auto row0_tag) {
+                    vec8(&fb_nxt)[FN], int h, auto row0_tag, auto ld_tag) {
       constexpr int ROW0 = decltype(row0_tag)::value;
+      constexpr bool LD = decltype(ld_tag)::value;
       constexpr int READS = FM + FN;
       constexpr int READ_ROWS = FM * FN >= 64 ? FM / 2 : (FM > 1 ? FM - 1 : 1);
       constexpr int PER_READ_ROW = (READS + READ_ROWS - 1) / READ_ROWS;
@@ -470,8 +480,10 @@ struct GemmTile {
 #pragma unroll
         for (int u = 0; u < PER_ROW; ++u) {
           const int l = (ROW0 + i) * PER_ROW + u;  // B first: it is needed one tile sooner
-          if (l < LB) load_b(l, h + BST - 1);
-          else if (l < LOADS) load_a(l - LB, h + AST - 1);
+          if constexpr (LD) {
+            if (l < LB) load_b(l, h + BST - 1);
+            else if (l < LOADS) load_a(l - LB, h + AST - 1);
+          }
         }
         // Inside the row: MFMA, LDS read, MFMA, LDS read, MFMA, the rest of the reads, buffer load, the
         // remaining MFMAs.  A read or load issued between two MFMAs costs no matrix-core time (an MFMA
@@ -485,7 +497,7 @@ struct GemmTile {
           __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
           __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
           __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-          __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x020, PER_ROW, 0);
           __builtin_amdgcn_sched_group_barrier(0x008, FN - 3, 0);
         }
         __builtin_amdgcn_sched_barrier(0);
@@ -495,7 +507,7 @@ struct GemmTile {
     // One K tile h: make it visible to every wavefront, then two steps.  Step 0 multiplies the
     // second half of tile h-1 (set 1) while reading the first half of tile h into set 0; step 1
     // multiplies set 0 while reading the second half of tile h into set 1.
-    auto tile_body = [&](int h) {
+    auto tile_body = [&](int h, auto ld_tag) {
       wait_vm_and_lds<WAIT_STEADY>();  // my fills of tile h have landed; my reads of tile h-1 are done
       bare_barrier();                  // ... and so have everyone else's: the slots of tile h-1 are free
       const char* sa = smem + (h % AST) * A_BYTES + a_wave_off;
@@ -503,8 +515,8 @@ struct GemmTile {
       // per-step offset of the B fragments: a swizzled chunk of the row, or 32 rows of k
       const int sb0 = B_KMAJOR ? 0 : frag_off[0];
       const int sb1 = B_KMAJOR ? 32 * BN * 2 : frag_off[1];
-      step(sa + frag_off[0], sb + sb0, fa1, fa0, fb1, fb0, h, std::integral_constant<int, 0>{});
-      step(sa + frag_off[1], sb + sb1, fa0, fa1, fb0, fb1, h, std::integral_constant<int, FM>{});
+      step(sa + frag_off[0], sb + sb0, fa1, fa0, fb1, fb0, h, std::integral_constant<int, 0>{}, ld_tag);
+      step(sa + frag_off[1], sb + sb1, fa0, fa1, fb0, fb1, h, std::integral_constant<int, FM>{}, ld_tag);
       if constexpr (SIDE) {
         side_store(h);
         side_load(h + 1);
@@ -516,7 +528,7 @@ struct GemmTile {
       // wait below is about).  A short tile 0 goes through registers instead.
       if (k_tail) fill_short_tile(k_tail);
 #pragma unroll
-      for (int s = 0; s < AST - 1; ++s) {
+      for (int s = 0; s < (loader ? AST - 1 : 0); ++s) {
         if (!(s == 0 && k_tail)) {
 #pragma unroll
           for (int i = 0; i < LA; ++i) load_a(i, s);
@@ -530,7 +542,15 @@ struct GemmTile {
         side_store(-1);  // dropped; keeps the number of side operations per tile uniform
         side_load(0);
       }
-      for (int h = 0; h < n_tiles; ++h) tile_body(h);
+      // two straight-line versions of the loop, with and without the loads: a branch around every load
+      // would cut each row of MFMAs into several scheduling regions
+      if constexpr (LDW == NW) {
+        for (int h = 0; h < n_tiles; ++h) tile_body(h, std::true_type{});
+      } else if (loader) {
+        for (int h = 0; h < n_tiles; ++h) tile_body(h, std::true_type{});
+      } else {
+        for (int h = 0; h < n_tiles; ++h) tile_body(h, std::false_type{});
+      }
       wait_vm_and_lds<0>();  // the empty fills of the last iterations must be gone before LDS is reused
       // Drain: the second half of the last tile is in set 1.
       if constexpr (B_KMAJOR) {
