@@ -24,11 +24,16 @@
 //     never sees a burst; one s_barrier per K tile;
 //   * fragments are software pipelined one 32-wide step ahead, both operands double buffered
 //     in registers; the reads of the next step are issued in the first rows of the current
-//     one and every row of MFMAs is closed by a scheduling fence, so the order written here
-//     is the order executed;
+//     one, between that row's MFMAs, and every row is closed by a scheduling fence, so the
+//     order written here is the order executed;
+//   * with two wavefronts per SIMD only the older wavefront of each pair issues loads (the
+//     hardware lets it win the matrix pipe, so it has time to spare; the younger one is the
+//     critical path of every K tile);
+//   * B may also be stored [K][N] (B_KMAJOR): its tiles are staged as they lie in memory and
+//     transposed on the way into registers by ds_read_b64_tr_b16;
 //   * the MFMA is issued with B as the first operand, so every lane ends up with 4
 //     consecutive columns of one output row per block: stores are 8 bytes (16-bit C) or 16
-//     bytes (fp32), and a row's statistics reduce over registers plus two lane swaps.
+//     bytes (fp32), and a row's statistics reduce over the lane's own registers first.
 #pragma once
 
 #include <hip/hip_runtime.h>
