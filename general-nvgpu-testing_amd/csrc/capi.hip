@@ -281,22 +281,22 @@ int beam_default_config(int M, int N, int K, beam_tile_cfg* cfg, int* split_k) {
   // them at a time (what LDS allows); a workgroup costs a fixed start-up / epilogue time plus its flops
   // at the per-CU rate of its tile shape, which is higher when several workgroups share the CU.  The
   // rates (TFLOP/s per CU, alone / with a full CU) and fixed costs (us) are fits to timings of all
-  // compiled tiles on 22 shapes from 512^3 to 6144^3 on an MI355X: the pick is within 1.4% of the
-  // best tile on average, 20% at worst (the thresholds this replaces: 4.3% and 57%).
+  // compiled tiles on 22 shapes from 512^3 to 6144^3 on an MI355X: the pick is within 2% of the
+  // best tile on average, 19% at worst (tile-count thresholds: 5.8% and 69%).
   struct Candidate {
     beam_tile_cfg cfg;
     int occ;
     double alone, full, fixed;
   };
   static const Candidate kCandidates[] = {
-      {{256, 256, 128, 64, 0, default_group_m(256, 256)}, 1, 6.16, 6.16, 8.0},
-      {{256, 128, 64, 64, 0, default_group_m(256, 128)}, 1, 4.8, 4.8, 6.0},
+      {{256, 256, 128, 64, 0, default_group_m(256, 256)}, 1, 6.78, 6.78, 8.0},
+      {{256, 128, 64, 64, 0, default_group_m(256, 128)}, 1, 5.54, 5.54, 6.0},
       {{128, 256, 64, 64, 0, default_group_m(128, 256)}, 1, 4.8, 4.8, 6.0},
       {{128, 128, 64, 64, 0, default_group_m(128, 128)}, 2, 3.8, 4.4, 3.42},
       {{128, 128, 64, 32, 2, default_group_m(128, 128)}, 1, 4.05, 4.05, 4.0},
       {{128, 64, 64, 32, 0, default_group_m(128, 64)}, 2, 2.6, 3.4, 3.5},
       {{128, 64, 64, 32, 2, default_group_m(128, 64)}, 1, 3.2, 3.2, 4.2},
-      {{64, 64, 32, 32, 0, default_group_m(64, 64)}, 4, 1.87, 2.9, 2.43},
+      {{64, 64, 32, 32, 0, default_group_m(64, 64)}, 4, 1.87, 2.9, 2.7},
       {{64, 64, 32, 32, 2, default_group_m(64, 64)}, 1, 2.4, 2.4, 4.0},
   };
   beam_tile_cfg c = kCandidates[0].cfg;
