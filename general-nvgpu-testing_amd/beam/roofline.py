@@ -1,6 +1,6 @@
 """Roofline arithmetic for tiled GEMMs, with an MI355X row.
 
-Counterpart of the reference's python/scripts/gemm_flops.py:1-90 (GPUSpec :4-13, spec list
+Counterpart of the reference's python/scripts/gemm_flops.py:1-90 and python/scripts/attn_flops.py:1-16 (GPUSpec :4-13, spec list
 :26-32, print_gemm_bound :37-76): the time a GEMM needs at the matrix-unit peak, the time its
 tiles need at the memory bandwidth when every tile fetches its operands once, and their ratio.
 Differences: a function that returns the numbers (the reference only prints), bytes counted with
@@ -79,6 +79,22 @@ def print_gemm_bound(spec: GPUSpec, dtype: str, n: int, k: int, m: int, micro_n:
     return r
 
 
+def attn_flops(batch_size: int, num_heads: int, seq_len: int, head_dim: int) -> int:
+    """FLOPs of one attention layer's two batched GEMMs, Q.K^T ([b,h,s,d] x [b,h,d,s]) and P.V
+    ([b,h,s,s] x [b,h,s,d]), 2 per multiply-add: 4*b*h*s*s*d.  Same count as the reference's
+    python/scripts/attn_flops.py:1-7 (its example, :11: b=2, h=24, s=4429, d=64)."""
+    return 4 * batch_size * num_heads * seq_len * seq_len * head_dim
+
+
+def attn_bound_ms(spec: GPUSpec, dtype: str, batch_size: int, num_heads: int, seq_len: int, head_dim: int) -> float:
+    """Time of those two GEMMs at the matrix-unit peak of `spec`."""
+    rate = getattr(spec, "fp16" if dtype == "bf16" else dtype)
+    if rate <= 0:
+        raise ValueError(f"{spec.name} has no {dtype} matrix rate")
+    return attn_flops(batch_size, num_heads, seq_len, head_dim) / (rate * 1e12) * 1e3
+
+
 if __name__ == "__main__":
     print_gemm_bound(GPU_NAME_SPEC_MAP["MI355X"], "fp16", 8192, 8192, 8192, 256, 8192, 256)
     print_gemm_bound(GPU_NAME_SPEC_MAP["MI355X"], "fp16", 256, 32768, 256, 64, 2048, 64)
+    print(f"FLOPS: {attn_flops(2, 24, 4096 + 333, 64)}")

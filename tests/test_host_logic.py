@@ -221,3 +221,7 @@ def test_roofline_calculator():
     assert split["ratio"] < 1 and abs(split["memory_ms"] * 1e3 - 4.21) < 0.01  # the 4.2 us HBM floor
     with pytest.raises(ValueError):
         R.gemm_bound(mi, "tf32", 64, 64, 64, 64, 64, 64)
+    # attention: the reference's example (b=2, h=24, s=4429, d=64), counted term by term as it does
+    b, h, sq, d = 2, 24, 4096 + 333, 64
+    assert R.attn_flops(b, h, sq, d) == 2 * (b * h * sq * d * sq + b * h * sq * sq * d) == 241041911808
+    assert abs(R.attn_bound_ms(mi, "bf16", b, h, sq, d) - 241041911808 / 2516.6e12 * 1e3) < 1e-9
