@@ -411,8 +411,20 @@ int beam_parallel_gemmrc_silu(const void* A, const void* B, void* C, int M, int 
   p.side_y = Y;
   p.side_count = count;
   const long long wgs = (long long)p.tiles_m * p.tiles_n;
-  const long long per_pass = wgs * ks->threads;  // vectors one pass of the whole grid covers
-  p.side_iters = (int)(((count >> 3) + per_pass - 1) / per_pass);
+  const long long per_pass = wgs * ks->threads;  // units one K tile of the whole grid covers
+  // The narrowest unit with which the job still ends inside the K loop: the work is then spread
+  // evenly over the tiles instead of crowding the first ones.  A job longer than the loop keeps
+  // 16-byte units and finishes after the GEMM's epilogue.
+  const long long k_tiles = ((long long)K + kBK - 1) / kBK;
+  p.side_width = 16;
+  for (int w = 4; w < 16; w *= 2) {
+    const long long units = (count >> 3) * (16 / w);
+    if ((units + per_pass - 1) / per_pass <= k_tiles) {
+      p.side_width = w;
+      break;
+    }
+  }
+  p.side_iters = (int)(((count >> 3) * (16 / p.side_width) + per_pass - 1) / per_pass);
   BEAM_HIP(ks->launch[dtype][kEpiStoreSide][c.pipeline](p, dim3((unsigned)wgs, 1, 1), (hipStream_t)stream));
   return BEAM_OK;
 }

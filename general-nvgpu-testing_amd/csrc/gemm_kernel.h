@@ -52,6 +52,7 @@ typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 typedef int i32x4 __attribute__((ext_vector_type(4)));
+typedef int i32x2 __attribute__((ext_vector_type(2)));
 
 template <typename T>
 struct ElemTraits;
@@ -103,13 +104,16 @@ struct GemmParams {
   int splits;    // number of K slices (1 = no split); the grid holds tiles_m * tiles_n * splits workgroups
   int group_m;   // rasterisation group height in tiles (fused LayerNorm: bands per band group)
   int group_n;   // fused LayerNorm: columns of a band group owned by one XCD
-  // Side job (kEpiStoreSide): y[i] = silu(x[i]) over a flat 16-bit array.  Whole 8-element
-  // vectors are dealt out in contiguous runs of side_iters * threads vectors per workgroup, one
-  // vector per thread per K tile; the last side_count % 8 elements are done by workgroup 0.
+  // Side job (kEpiStoreSide): y[i] = silu(x[i]) over a flat 16-bit array.  The whole 8-element
+  // groups of the array are cut into units of side_width bytes (16, 8 or 4), dealt out in
+  // contiguous runs of side_iters * threads units per workgroup, `threads` units per K tile; the
+  // last side_count % 8 elements are done by workgroup 0.  The host picks the narrowest unit with
+  // which the job still fits into the K loop, so that every tile carries an equal, small share.
   const void* side_x;
   void* side_y;
   long long side_count;  // elements
-  int side_iters;        // vectors per thread of one workgroup
+  int side_iters;        // K tiles' worth of units per workgroup
+  int side_width;        // bytes per unit
 };
 
 // Buffer descriptor word 3 for gfx9-family raw buffers: 32-bit data format, no swizzle.
@@ -184,11 +188,12 @@ struct GemmTile {
   static constexpr int ROWS = KSTEPS * FM;                 // rows of MFMAs per K tile
   static constexpr int PER_ROW = (LOADS + ROWS - 1) / ROWS;  // buffer loads issued after each row
   // Loads that may still be in flight when tile h is needed: the A tiles and B tiles beyond h.
-  // The side job adds one buffer store and one buffer load at the end of every K tile; the
-  // fills a tile waits for were issued min(AST, BST) - 1 tiles earlier.
+  // The side job adds SV buffer stores and SV buffer loads at the end of every K tile of a loader
+  // wavefront; the fills a tile waits for were issued min(AST, BST) - 1 tiles earlier.
   static constexpr bool SIDE = (EPI == kEpiStoreSide);
+  static constexpr int SV = NW / LDW;  // side vectors per loader thread per K tile
   static constexpr int WAIT_STEADY =
-      (AST - 2) * LA + (BST - 2) * LB + (SIDE ? 2 * ((AST < BST ? AST : BST) - 1) : 0);
+      (AST - 2) * LA + (BST - 2) * LB + (SIDE ? 2 * SV * ((AST < BST ? AST : BST) - 1) : 0);
 
   static_assert(KSTEPS == 2, "the step pipeline below is written for two 32-wide steps per tile");
   static_assert(TM % 16 == 0 && TN % 16 == 0, "wavefront tile must be made of 16x16 blocks");
@@ -400,30 +405,72 @@ struct GemmTile {
       }
 
     // ---- side job: state and pieces ------------------------------------------------------
-    // side_in holds the vector loaded during the previous K tile; one element per MFMA row of
-    // step 1 is pushed through silu into side_out, which is stored at the end of the tile, right
-    // before the load of the next vector.  Vectors outside this workgroup's run get an offset
-    // outside the descriptor: the load returns zeros and the store is dropped.
+    // side_buf holds the units loaded during the previous K tile; step 1 pushes them through silu
+    // in place, a pair of elements at a time on evenly spaced MFMA rows, and they are stored at the
+    // end of the tile, right before the load of the next units.  Units outside this workgroup's
+    // run get an offset outside the descriptor: the load returns zeros and the store is dropped.
+    // Only the loader wavefronts do this work, SV units each.  They are the older wavefront of
+    // their SIMD, win the arbitration for the matrix core and reach the barrier of every tile with
+    // some hundred cycles to spare, while the younger ones set the pace of the loop: arithmetic
+    // given to the older wavefront fills that slack, the same arithmetic in the younger one
+    // lengthens the tile.
     const unsigned side_bytes = SIDE ? (unsigned)((p.side_count >> 3) << 4) : 0u;
     const __amdgpu_buffer_rsrc_t rsrc_sx = make_rsrc(p.side_x, side_bytes);
     const __amdgpu_buffer_rsrc_t rsrc_sy = make_rsrc(p.side_y, side_bytes);
     const unsigned side_v0 = SIDE ? ((unsigned)blockIdx.x * (unsigned)p.side_iters * NT + tid) : 0u;
-    i32x4 side_in = {0, 0, 0, 0};
-    vec8 side_out;
+    int side_buf[SV][4];  // pairs of elements: x when loaded, overwritten pair by pair with silu(x)
 #pragma unroll
-    for (int e = 0; e < 8; ++e) side_out[e] = 0;
-    auto side_offset = [&](int it) {
-      return (it >= 0 && it < p.side_iters) ? (side_v0 + (unsigned)it * NT) * 16u : kOobOffset;
+    for (int s = 0; s < SV; ++s) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) side_buf[s][e] = 0;
+    }
+    // W: bytes per unit (compile time inside each version of the loop).  The host picks wide units
+    // only for an array that is large beside the GEMM; its traffic is then marked non-temporal
+    // (auxiliary bit 1), so that lines written once do not push the GEMM's operands out of the L2:
+    // 900 -> 866 us for 8192^3 carrying 256 Mi elements.  A small array (4-byte units) is better
+    // left in the cache, for whoever reads y next.
+    auto side_offset = [&](int it, int s, int W) {  // thread tid of the loaders owns units tid + s * NTL of a tile
+      return (it >= 0 && it < p.side_iters) ? (side_v0 + (unsigned)it * NT + (unsigned)s * NTL) * (unsigned)W : kOobOffset;
     };
-    auto side_load = [&](int it) {
-      side_in = __builtin_amdgcn_raw_buffer_load_b128(rsrc_sx, (int)side_offset(it), 0, 0);
+    auto side_load = [&](int it, auto w_tag) {
+      constexpr int W = decltype(w_tag)::value;
+      constexpr int AUX = W >= 8 ? 2 : 0;
+#pragma unroll
+      for (int s = 0; s < SV; ++s) {
+        const int off = (int)side_offset(it, s, W);
+        if constexpr (W == 16) {
+          const i32x4 v = __builtin_amdgcn_raw_buffer_load_b128(rsrc_sx, off, 0, AUX);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) side_buf[s][e] = v[e];
+        } else if constexpr (W == 8) {
+          const i32x2 v = __builtin_amdgcn_raw_buffer_load_b64(rsrc_sx, off, 0, AUX);
+          side_buf[s][0] = v[0];
+          side_buf[s][1] = v[1];
+        } else {
+          side_buf[s][0] = __builtin_amdgcn_raw_buffer_load_b32(rsrc_sx, off, 0, AUX);
+        }
+      }
     };
-    auto side_store = [&](int it) {
-      __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(i32x4, side_out), rsrc_sy, (int)side_offset(it), 0, 0);
+    auto side_store = [&](int it, auto w_tag) {
+      constexpr int W = decltype(w_tag)::value;
+      constexpr int AUX = W >= 8 ? 2 : 0;
+#pragma unroll
+      for (int s = 0; s < SV; ++s) {
+        const int off = (int)side_offset(it, s, W);
+        const int* o = side_buf[s];
+        if constexpr (W == 16) __builtin_amdgcn_raw_buffer_store_b128(i32x4{o[0], o[1], o[2], o[3]}, rsrc_sy, off, 0, AUX);
+        else if constexpr (W == 8) __builtin_amdgcn_raw_buffer_store_b64(i32x2{o[0], o[1]}, rsrc_sy, off, 0, AUX);
+        else __builtin_amdgcn_raw_buffer_store_b32(o[0], rsrc_sy, off, 0, AUX);
+      }
     };
-    auto side_element = [&](int e) {
-      const vec8 x = __builtin_bit_cast(vec8, side_in);
-      side_out[e] = silu_16<T>(x[e]);
+    auto side_pair = [&](int e) {  // pair e of every unit this thread holds
+#pragma unroll
+      for (int s = 0; s < SV; ++s) {
+        typedef T pair_t __attribute__((ext_vector_type(2)));
+        const pair_t x = __builtin_bit_cast(pair_t, side_buf[s][e]);
+        const pair_t y = {silu_16<T>(x[0]), silu_16<T>(x[1])};
+        side_buf[s][e] = __builtin_bit_cast(int, y);
+      }
     };
 
     // One pipeline step = FM rows of FN MFMAs on the fragments in (fa_cur, fb_cur).  The FM + FN
@@ -435,9 +482,10 @@ struct GemmTile {
     // registers across the two sets, and the step then starts by waiting for its own reads.
     //   ROW0: index of the step's first row inside the tile (the loads are dealt out row by row).
     auto step = [&](const char* sa, const char* sb, vec8(&fa_cur)[FM], vec8(&fa_nxt)[FM], vec8(&fb_cur)[FN],
-                    vec8(&fb_nxt)[FN], int h, auto row0_tag, auto ld_tag) {
+                    vec8(&fb_nxt)[FN], int h, auto row0_tag, auto ld_tag, auto w_tag) {
       constexpr int ROW0 = decltype(row0_tag)::value;
       constexpr bool LD = decltype(ld_tag)::value;
+      constexpr int SIDE_PAIRS = decltype(w_tag)::value / 4;  // pairs of elements per side unit
       constexpr int READS = FM + FN;
       constexpr int READ_ROWS = FM * FN >= 64 ? FM / 2 : (FM > 1 ? FM - 1 : 1);
       constexpr int PER_READ_ROW = (READS + READ_ROWS - 1) / READ_ROWS;
@@ -474,12 +522,14 @@ struct GemmTile {
           const int j = (NW >= 8 && (i & 1)) ? FN - 1 - jj : jj;
           acc[i][j] = Traits::mfma(fb_cur[j], fa_cur[i], acc[i][j]);
         }
-        if constexpr (SIDE && ROW0 != 0) {  // step 1: this row's share of the side vector
-          constexpr int PER = (8 + FM - 1) / FM;
-          if (h < p.side_iters) {  // uniform: tiles past the workgroup's run carry nothing
+        if constexpr (SIDE && LD && ROW0 != 0) {  // step 1: this row's share of the side vectors
+          // pairs are dealt to every (FM / SIDE_PAIRS)-th row, or several to a row of a short step
+          constexpr int EVERY = FM >= SIDE_PAIRS ? FM / SIDE_PAIRS : 1;
+          constexpr int PER = FM >= SIDE_PAIRS ? 1 : (SIDE_PAIRS + FM - 1) / FM;
+          if (i % EVERY == 0 && h < p.side_iters) {  // uniform: tiles past the workgroup's run carry nothing
 #pragma unroll
             for (int u = 0; u < PER; ++u)
-              if (i * PER + u < 8) side_element(i * PER + u);
+              if ((i / EVERY) * PER + u < SIDE_PAIRS) side_pair((i / EVERY) * PER + u);
           }
         }
 #pragma unroll
@@ -512,7 +562,7 @@ struct GemmTile {
     // One K tile h: make it visible to every wavefront, then two steps.  Step 0 multiplies the
     // second half of tile h-1 (set 1) while reading the first half of tile h into set 0; step 1
     // multiplies set 0 while reading the second half of tile h into set 1.
-    auto tile_body = [&](int h, auto ld_tag) {
+    auto tile_body = [&](int h, auto ld_tag, auto w_tag) {
       wait_vm_and_lds<WAIT_STEADY>();  // my fills of tile h have landed; my reads of tile h-1 are done
       bare_barrier();                  // ... and so have everyone else's: the slots of tile h-1 are free
       const char* sa = smem + (h % AST) * A_BYTES + a_wave_off;
@@ -520,11 +570,11 @@ struct GemmTile {
       // per-step offset of the B fragments: a swizzled chunk of the row, or 32 rows of k
       const int sb0 = B_KMAJOR ? 0 : frag_off[0];
       const int sb1 = B_KMAJOR ? 32 * BN * 2 : frag_off[1];
-      step(sa + frag_off[0], sb + sb0, fa1, fa0, fb1, fb0, h, std::integral_constant<int, 0>{}, ld_tag);
-      step(sa + frag_off[1], sb + sb1, fa0, fa1, fb0, fb1, h, std::integral_constant<int, FM>{}, ld_tag);
-      if constexpr (SIDE) {
-        side_store(h);
-        side_load(h + 1);
+      step(sa + frag_off[0], sb + sb0, fa1, fa0, fb1, fb0, h, std::integral_constant<int, 0>{}, ld_tag, w_tag);
+      step(sa + frag_off[1], sb + sb1, fa0, fa1, fb0, fb1, h, std::integral_constant<int, FM>{}, ld_tag, w_tag);
+      if constexpr (SIDE && decltype(ld_tag)::value) {
+        side_store(h, w_tag);
+        side_load(h + 1, w_tag);
       }
     };
 
@@ -543,18 +593,34 @@ struct GemmTile {
           for (int i = 0; i < LB; ++i) load_b(i, s);
         }
       }
-      if constexpr (SIDE) {
-        side_store(-1);  // dropped; keeps the number of side operations per tile uniform
-        side_load(0);
+      using W16 = std::integral_constant<int, 16>;
+      using W8 = std::integral_constant<int, 8>;
+      using W4 = std::integral_constant<int, 4>;
+      if (SIDE && loader) {
+        side_store(-1, W4{});  // dropped; keeps the number of side operations per tile uniform
+        if (p.side_width == 16) side_load(0, W16{});
+        else if (p.side_width == 8) side_load(0, W8{});
+        else side_load(0, W4{});
       }
       // two straight-line versions of the loop, with and without the loads: a branch around every load
       // would cut each row of MFMAs into several scheduling regions
-      if constexpr (LDW == NW) {
-        for (int h = 0; h < n_tiles; ++h) tile_body(h, std::true_type{});
+      // (and the side job one version per unit width: the unit's elements are dealt to rows at compile time)
+      if constexpr (SIDE) {
+        if (!loader) {
+          for (int h = 0; h < n_tiles; ++h) tile_body(h, std::false_type{}, W16{});
+        } else if (p.side_width == 16) {
+          for (int h = 0; h < n_tiles; ++h) tile_body(h, std::true_type{}, W16{});
+        } else if (p.side_width == 8) {
+          for (int h = 0; h < n_tiles; ++h) tile_body(h, std::true_type{}, W8{});
+        } else {
+          for (int h = 0; h < n_tiles; ++h) tile_body(h, std::true_type{}, W4{});
+        }
+      } else if constexpr (LDW == NW) {
+        for (int h = 0; h < n_tiles; ++h) tile_body(h, std::true_type{}, W16{});
       } else if (loader) {
-        for (int h = 0; h < n_tiles; ++h) tile_body(h, std::true_type{});
+        for (int h = 0; h < n_tiles; ++h) tile_body(h, std::true_type{}, W16{});
       } else {
-        for (int h = 0; h < n_tiles; ++h) tile_body(h, std::false_type{});
+        for (int h = 0; h < n_tiles; ++h) tile_body(h, std::false_type{}, W16{});
       }
       wait_vm_and_lds<0>();  // the empty fills of the last iterations must be gone before LDS is reused
       // Drain: the second half of the last tile is in set 1.
@@ -707,11 +773,12 @@ struct GemmTile {
       if constexpr (SIDE) {
         // Side vectors beyond the K tiles of this workgroup (a short K loop or a long array), then
         // the elements after the last whole vector.
-        for (int it = n_tiles; it < p.side_iters; ++it) {
+        // (the host narrows the units only when the job then still fits into the loop: 16-byte units here)
+        for (int it = n_tiles; loader && it < p.side_iters; ++it) {
 #pragma unroll
-          for (int e = 0; e < 8; ++e) side_element(e);
-          side_store(it);
-          side_load(it + 1);
+          for (int e = 0; e < 4; ++e) side_pair(e);
+          side_store(it, std::integral_constant<int, 16>{});
+          side_load(it + 1, std::integral_constant<int, 16>{});
         }
         const long long done = (p.side_count >> 3) << 3;
         if (blockIdx.x == 0 && done + tid < p.side_count) {

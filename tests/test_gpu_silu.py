@@ -138,6 +138,21 @@ def test_pair_every_config(gpu, beamc, oracle):
                     assert_same_bits(ygot, run_silu(beamc, x, F16), x, f"{c.name} n={n}")
 
 
+def test_pair_unit_widths(gpu, beamc, oracle):
+    """The side array is cut into 4-, 8- or 16-byte units depending on how much of the K loop it
+    fills.  512 x 512 x 2048 has 32 K tiles; with 2048 (256x256 tile) or 4096 (128x128 tile) units per
+    tile the sizes below land in each width, at both ends of its range, and beyond the loop."""
+    M, N, K = 512, 512, 2048
+    a = beamc.host_uniform((M, K), F16, 1, 0)
+    b = beamc.host_uniform((N, K), F16, 1, 1)
+    for tile in ((256, 256, 128, 64), (128, 128, 64, 32)):
+        c = beamc.TileConfig(*tile, 0, 0)
+        for n in (8, 65536, 131072 + 8, 200005, 262144, 400001, 524288, 800007, 1048576, 1200003, 2400001):
+            x = beamc.host_normal((n,), F16, 31, n, 0.0, 2.5)
+            _, ygot = run_pair(beamc, a, b, x, F16, c)
+            assert_same_bits(ygot, run_silu(beamc, x, F16), x, f"{c.name} n={n}")
+
+
 @pytest.mark.parametrize("dtype", [F16, BF16])
 def test_pair_1024_cube(gpu, beamc, oracle, dtype):
     M = N = K = 1024
