@@ -32,8 +32,10 @@
 //   * B may also be stored [K][N] (B_KMAJOR): its tiles are staged as they lie in memory and
 //     transposed on the way into registers by ds_read_b64_tr_b16;
 //   * the MFMA is issued with B as the first operand, so every lane ends up with 4
-//     consecutive columns of one output row per block: stores are 8 bytes (16-bit C) or 16
-//     bytes (fp32), and a row's statistics reduce over the lane's own registers first.
+//     consecutive columns of one output row per block: a row's statistics reduce over the
+//     lane's own registers first, fp32 output is stored 16 bytes at a time, and 16-bit output
+//     takes one trip through the (by then idle) LDS so that it leaves as whole rows of the
+//     wavefront's sub-tile, 16 bytes per lane.
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -748,28 +750,77 @@ struct GemmTile {
     const int n_base = col0 + wn * TN + 4 * (lane >> 4);
     const bool vec_ok = (N % 4) == 0;
 
-    if (EPI == kEpiStore || EPI == kEpiStoreSide) {
-      T* C = (T*)p.C;
+    // 16-bit output through LDS, so that a store instruction writes whole rows of the wavefront's
+    // sub-tile (TN columns = TN / 8 lanes of 16 bytes each) instead of 16 rows x 32 bytes: the
+    // direct stores cost 3% at 4096^3 and 5% at 16384 x 16384 x 2048.  Each wavefront uses a
+    // private region of (TM / HALVES) rows of TN * 2 bytes behind the first RESERVED bytes of LDS;
+    // the caller has made sure that LDS is free (a barrier).
+    // Layout of a region (measured with the bank-conflict counter): an 8-byte write is served 16
+    // lanes (= the 16 rows of a block, one column group) at a time out of 32 banks, so the 16 rows
+    // must land in 16 different 8-byte slots of a 128-byte window.  A row's 16-byte chunks are
+    // XORed with the row number (3 bits; 2 bits and the row's parity where two rows share a
+    // window) and rows 8..15 of a block have the two halves of every chunk swapped.  The 16-byte
+    // reads run over whole rows (any padding of the rows makes them conflict) and undo both.
+    //   row_ctx(i): per-row values of block row i, passed on to value(i, j, ctx) -> 4 outputs.
+    auto staged_store = [&](T* C, auto reserved_tag, auto row_ctx, auto value) {
+      constexpr int RESERVED = decltype(reserved_tag)::value;
+      constexpr int AVAIL = LDS_BYTES - RESERVED;
+      constexpr int RB = TN * 2;  // bytes per row
+      constexpr int HALVES = NW * TM * RB <= AVAIL ? 1 : (NW * TM * RB <= 2 * AVAIL ? 2 : 4);
+      static_assert(NW * (TM / HALVES) * RB <= AVAIL && FM % HALVES == 0 && RESERVED % 128 == 0, "staging area");
+      static_assert(RB == 64 || RB == 128 || RB == 256, "row of a wavefront's sub-tile");
+      constexpr int FMH = FM / HALVES;  // blocks of 16 rows per pass
+      constexpr int LPR = TN / 8;       // lanes per row
+      constexpr int RPI = 64 / LPR;     // rows per store instruction
+      auto chunk_xor = [](int r) { return RB == 64 ? (r >> 1) & 3 : r & 7; };
+      char* stage = smem + RESERVED + wave * (FMH * 16 * RB);
+      const bool wide_ok = (N % 8) == 0 && ((size_t)C & 15) == 0;
+      const int srow = lane / LPR, schunk = lane % LPR;
+      const int wr = lane & 15, wg = lane >> 4;  // writer: row of the block, column group
+      const int w_off = wr * RB + (((wg & 1) ^ (wr >> 3)) << 3);
 #pragma unroll
-      for (int i = 0; i < FM; ++i) {
-        const int m = m_base + i * 16;
-        if (m >= M) continue;
-        T* crow = C + (size_t)m * N;
+      for (int hf = 0; hf < HALVES; ++hf) {
 #pragma unroll
-        for (int j = 0; j < FN; ++j) {
-          const int n = n_base + j * 16;
-          vec4 v;
+        for (int i = 0; i < FMH; ++i) {
+          const auto ctx = row_ctx(hf * FMH + i);
 #pragma unroll
-          for (int e = 0; e < 4; ++e) v[e] = (T)acc[i][j][e];
-          if (vec_ok && n + 3 < N) {
-            *(vec4*)(crow + n) = v;
-          } else {
+          for (int j = 0; j < FN; ++j)
+            *(vec4*)(stage + i * 16 * RB + w_off + (((2 * j + (wg >> 1)) ^ chunk_xor(wr)) << 4)) = value(hf * FMH + i, j, ctx);
+        }
 #pragma unroll
-            for (int e = 0; e < 4; ++e)
-              if (n + e < N) crow[n + e] = v[e];
+        for (int it = 0; it < FMH * 16 / RPI; ++it) {
+          const int r = it * RPI + srow;
+          vec8 v = *(const vec8*)(stage + r * RB + schunk * 16);
+          if ((r >> 3) & 1) v = vec8{v[4], v[5], v[6], v[7], v[0], v[1], v[2], v[3]};
+          const int n_st = col0 + wn * TN + (schunk ^ chunk_xor(r)) * 8;
+          const int m = row0 + wm * TM + hf * FMH * 16 + r;
+          if (m < M) {
+            T* dst = C + (size_t)m * N + n_st;
+            if (wide_ok && n_st + 7 < N) {
+              *(vec8*)dst = v;
+            } else if (vec_ok && n_st + 7 < N) {  // C only 8-byte aligned, or N % 8 == 4
+              *(vec4*)dst = vec4{v[0], v[1], v[2], v[3]};
+              *(vec4*)(dst + 4) = vec4{v[4], v[5], v[6], v[7]};
+            } else {
+#pragma unroll
+              for (int e = 0; e < 8; ++e)
+                if (n_st + e < N) dst[e] = v[e];
+            }
           }
         }
       }
+    };
+
+    if (EPI == kEpiStore || EPI == kEpiStoreSide) {
+      T* C = (T*)p.C;
+      __syncthreads();  // every wavefront is done with the last tile, and no fill is still landing
+      staged_store(C, std::integral_constant<int, 0>{}, [](int) { return 0; },
+                   [&](int i, int j, int) {
+                     vec4 v;
+#pragma unroll
+                     for (int e = 0; e < 4; ++e) v[e] = (T)acc[i][j][e];
+                     return v;
+                   });
       if constexpr (SIDE) {
         // Side vectors beyond the K tiles of this workgroup (a short K loop or a long array), then
         // the elements after the last whole vector.
@@ -892,31 +943,21 @@ struct GemmTile {
         red[rl * 2 + 1] = 1.0f / sqrtf(m2 / (float)N + p.eps);
       }
       __syncthreads();
-      // 5. normalise the accumulators and store Y
+      // 5. normalise the accumulators and store Y (through LDS, behind the row statistics)
       T* Y = (T*)p.C;
+      struct RowStat { float mean, rstd; };
+      staged_store(Y, std::integral_constant<int, BM * 2 * 4>{},
+                   [&](int i) {
+                     const int rl = wm * TM + i * 16 + (lane & 15);
+                     return RowStat{red[rl * 2 + 0], red[rl * 2 + 1]};
+                   },
+                   [&](int i, int j, RowStat st) {
+                     vec4 v;
 #pragma unroll
-      for (int i = 0; i < FM; ++i) {
-        const int m = m_base + i * 16;
-        if (m >= M) continue;
-        const int rl = wm * TM + i * 16 + (lane & 15);
-        const float mean = red[rl * 2 + 0];
-        const float rstd = red[rl * 2 + 1];
-        T* yrow = Y + (size_t)m * N;
-#pragma unroll
-        for (int j = 0; j < FN; ++j) {
-          const int n = n_base + j * 16;
-          vec4 v;
-#pragma unroll
-          for (int e = 0; e < 4; ++e) v[e] = (T)((acc[i][j][e] - mean) * rstd * (float)gv[j][e] + (float)bv[j][e]);
-          if (vec_ok && n + 3 < N) {
-            *(vec4*)(yrow + n) = v;
-          } else {
-#pragma unroll
-            for (int e = 0; e < 4; ++e)
-              if (n + e < N) yrow[n + e] = v[e];
-          }
-        }
-      }
+                     for (int e = 0; e < 4; ++e)
+                       v[e] = (T)((acc[i][j][e] - st.mean) * st.rstd * (float)gv[j][e] + (float)bv[j][e]);
+                     return v;
+                   });
     } else {
       if (EPI == kEpiLnStats) {
         // Per-row statistics over the columns this workgroup owns, from the fp32 accumulators.

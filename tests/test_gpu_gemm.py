@@ -75,6 +75,37 @@ def test_ragged_small_every_config(gpu, beamc, oracle, shape):
         assert_close(oracle, got, ref, K, F16, f"{shape} {cfg.name}")
 
 
+@pytest.mark.parametrize("shape", [(300, 264, 136), (257, 132, 72), (130, 70, 48)])
+def test_output_8_byte_aligned(gpu, beamc, shape):
+    """C needs 8-byte alignment only.  The epilogue writes 16-byte pieces of rows where it can
+    (C 16-byte aligned and N % 8 == 0) and falls back to 8-byte or single-element stores otherwise:
+    all three must give the same bits, and none may write outside C."""
+    M, N, K = shape
+    a_bits = beamc.host_uniform((M, K), F16, 5, 0)
+    b_bits = beamc.host_uniform((N, K), F16, 5, 1)
+    a = beamc.DeviceArray.from_numpy(a_bits, F16)
+    b = beamc.DeviceArray.from_numpy(b_bits, F16)
+    full = beamc.DeviceArray((M * N + 64,), F16)
+    c = beamc.DeviceArray.__new__(beamc.DeviceArray)
+    c.shape, c.dtype, c.itemsize, c.nbytes = (M, N), F16, 2, M * N * 2
+    try:
+        for cfg in all_configs(beamc):
+            outs = []
+            for shift in (0, 4, 8, 12):  # elements: 0, 8, 16 and 24 bytes past a 256-byte boundary
+                full.fill_bytes(0xEE)
+                c.ptr = full.ptr + 2 * shift
+                beamc.gemmrc(a, b, c, config=cfg)
+                out = full.to_numpy()
+                assert (out[:shift] == 0xEEEE).all() and (out[shift + M * N:] == 0xEEEE).all(), (cfg.name, shift)
+                outs.append(out[shift:shift + M * N])
+            for o in outs[1:]:
+                assert (o == outs[0]).all(), cfg.name
+    finally:
+        c.ptr = 0
+        for x in (a, b, full):
+            x.free()
+
+
 def test_ragged_3000x5000x2000(gpu, beamc, oracle):
     """Edge tiles in M and N and a short last K tile (K = 31*64 + 16), fp16 and bf16."""
     M, N, K = 3000, 5000, 2000
