@@ -122,11 +122,15 @@ def extra_splitk(_C):
                 if ms < best_split[1]:
                     best_split = (f"{pc.name},S={s}", ms, pc, s)
     graph_us = splitk_graph_us(_C, a, b, c, best_split[2], best_split[3])
+    # what a call that names neither tile nor slice count gets
+    auto_cfg, auto_s = _C.default_config(M, N, K)
+    auto_ms = min(_C.bench(1, a, b, c, config=None, split_k=0, warmup=20, iters=100) for _ in range(2))
     for x in (a, b, c):
         x.free()
     bytes_alg = 2.0 * (M * K + N * K + M * N)
     return {"shape": [M, N, K], "splitk_us": round(best_split[1] * 1e3, 2), "splitk_config": best_split[0],
             "splitk_in_graph_us": round(graph_us, 2),
+            "library_choice_us": round(auto_ms * 1e3, 2), "library_choice": f"{auto_cfg.name},S={auto_s}",
             "best_nonsplit_us": round(best_plain[1] * 1e3, 2), "best_nonsplit_config": best_plain[0],
             "speedup": round(best_plain[1] / best_split[1], 2),
             "hbm_GBs": round(bytes_alg / (best_split[1] * 1e-3) / 1e9, 1),
@@ -206,7 +210,7 @@ def main():
     a, b = _C.DeviceArray.from_numpy(a_bits), _C.DeviceArray.from_numpy(b_bits)
     c = _C.DeviceArray((M, N))
     c.fill_bytes(0xEE)
-    cfg, _ = _C.default_config(M, N, K)
+    cfg, _ = _C.default_config(M, N, K, split=False)
 
     def step():
         _C.gemmrc(a, b, c)

@@ -163,10 +163,12 @@ def list_configs() -> List[TileConfig]:
     return out
 
 
-def default_config(M: int, N: int, K: int):
+def default_config(M: int, N: int, K: int, split: bool = True):
+    """(tile, K slices) the library would use.  split=True: the best tile together with its slice
+    count (for callers with a workspace); split=False: the best tile without a split, slices = 1."""
     c = _TileCfg()
     s = ctypes.c_int(1)
-    _check(lib.beam_default_config(M, N, K, ctypes.byref(c), ctypes.byref(s)))
+    _check(lib.beam_default_config(M, N, K, ctypes.byref(c), ctypes.byref(s) if split else None))
     return TileConfig(c.block_m, c.block_n, c.wave_m, c.wave_n, c.pipeline, c.group_m), s.value
 
 

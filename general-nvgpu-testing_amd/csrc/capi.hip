@@ -104,12 +104,30 @@ int check_problem(const void* A, const void* B, const void* C, int M, int N, int
   return BEAM_OK;
 }
 
-int resolve_cfg(const beam_tile_cfg* in, int M, int N, int K, beam_tile_cfg* out, const KernelSet** ks) {
+// Slices for `tiles` output tiles when the caller leaves the choice to the library: as many as make
+// one full round of workgroups (tiles * slices = CUs), at least 4 K tiles each.  Measured at
+// 256 x 256 x 32768: 16 tiles x 16 slices 15.1 us, x 24 (one and a half rounds, what the reference's
+// rule gives: beam_slice_heuristic) 19.8 us, x 32 17.6 us; 8 tiles x 32 slices 14.2 us, x 16 17.0 us.
+int auto_slices(long tiles, int K, int cus) {
+  if (tiles * 2 > cus) return 1;
+  const int ktiles = (K + kBK - 1) / kBK;
+  long s = cus / (tiles < 1 ? 1 : tiles);
+  if (s > ktiles / 4) s = ktiles / 4;
+  if (s > 64) s = 64;  // the reduction reads every slice: 64 x 64 x 32768 takes 9.1 us with 64 slices, 11.4 with 128
+  return s < 1 ? 1 : (int)s;
+}
+
+int choose_default(int M, int N, int K, bool may_split, beam_tile_cfg* cfg, int* split_k);
+
+// may_split: the caller can run K slices (it has a workspace); the default tile is then chosen together
+// with its slice count.
+int resolve_cfg(const beam_tile_cfg* in, int M, int N, int K, beam_tile_cfg* out, const KernelSet** ks,
+                bool may_split = false) {
   if (in) {
     *out = *in;
   } else {
     int s;
-    int rc = beam_default_config(M, N, K, out, &s);
+    int rc = choose_default(M, N, K, may_split, out, &s);
     if (rc) return rc;
   }
   if (out->pipeline < 0 || out->pipeline > 2) return fail(BEAM_ERR_UNSUPPORTED, "pipeline %d: 0 (3 A + 2 B LDS slots), 1 (2 + 2) or 2 (deep)", out->pipeline);
@@ -274,6 +292,14 @@ int beam_slice_heuristic(int tiles, int compute_units) {
 }
 
 int beam_default_config(int M, int N, int K, beam_tile_cfg* cfg, int* split_k) {
+  return choose_default(M, N, K, split_k != nullptr, cfg, split_k);
+}
+
+}  // extern "C"
+
+namespace {
+
+int choose_default(int M, int N, int K, bool may_split, beam_tile_cfg* cfg, int* split_k) {
   if (!cfg) return fail(BEAM_ERR_INVALID, "null cfg");
   const int cus = g_dev.cus > 0 ? g_dev.cus : 256;
   auto tiles = [&](int bm, int bn) { return (long)((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
@@ -281,15 +307,16 @@ int beam_default_config(int M, int N, int K, beam_tile_cfg* cfg, int* split_k) {
   // them at a time (what LDS allows); a workgroup costs a fixed start-up / epilogue time plus its flops
   // at the per-CU rate of its tile shape, which is higher when several workgroups share the CU.  The
   // rates (TFLOP/s per CU, alone / with a full CU) and fixed costs (us) are fits to timings of all
-  // compiled tiles on 22 shapes from 512^3 to 6144^3 on an MI355X: the pick is within 2% of the
-  // best tile on average, 19% at worst (tile-count thresholds: 5.8% and 69%).
+  // compiled tiles on 29 shapes from 512^3 to 8192^3 (square, skinny and short-K) on an MI355X:
+  // the pick is within 0.5% of the best tile on average, 3.7% at worst (tile-count thresholds:
+  // 5.5% and 75%).
   struct Candidate {
     beam_tile_cfg cfg;
     int occ;
     double alone, full, fixed;
   };
   static const Candidate kCandidates[] = {
-      {{256, 256, 128, 64, 0, default_group_m(256, 256)}, 1, 6.78, 6.78, 8.0},
+      {{256, 256, 128, 64, 0, default_group_m(256, 256)}, 1, 6.1, 6.1, 8.0},
       {{256, 128, 64, 64, 0, default_group_m(256, 128)}, 1, 5.54, 5.54, 6.0},
       {{128, 256, 64, 64, 0, default_group_m(128, 256)}, 1, 4.8, 4.8, 6.0},
       {{128, 128, 64, 64, 0, default_group_m(128, 128)}, 2, 3.8, 4.4, 3.42},
@@ -298,35 +325,39 @@ int beam_default_config(int M, int N, int K, beam_tile_cfg* cfg, int* split_k) {
       {{128, 64, 64, 32, 2, default_group_m(128, 64)}, 1, 3.2, 3.2, 4.2},
       {{64, 64, 32, 32, 0, default_group_m(64, 64)}, 4, 1.87, 2.9, 2.7},
       {{64, 64, 32, 32, 2, default_group_m(64, 64)}, 1, 2.4, 2.4, 4.0},
+      {{64, 128, 32, 64, 0, default_group_m(64, 128)}, 2, 3.15, 3.4, 3.5},
+      {{64, 128, 32, 64, 2, default_group_m(64, 128)}, 1, 3.3, 3.3, 4.0},
   };
+  // With a workspace at hand the deep-pipeline candidates are priced with their K slices: the
+  // slices' workgroups fill the CUs, and the reduction costs a launch plus reading the partial sums.
   beam_tile_cfg c = kCandidates[0].cfg;
+  int c_split = 1;
   double best_us = 1e300;
   for (const Candidate& k : kCandidates) {
-    const long load = (tiles(k.cfg.block_m, k.cfg.block_n) + cus - 1) / cus;  // workgroups per CU
+    const long t = tiles(k.cfg.block_m, k.cfg.block_n);
+    const int s = (may_split && k.cfg.pipeline == 2) ? auto_slices(t, K, cus) : 1;
+    const long load = (t * s + cus - 1) / cus;  // workgroups per CU
     const long conc = load < k.occ ? load : k.occ;
     const double rate = k.occ == 1 ? k.alone : k.alone + (k.full - k.alone) * (double)(conc - 1) / (k.occ - 1);
-    const double mflop = 2.0e-6 * k.cfg.block_m * k.cfg.block_n * (double)K;
-    const double us = (double)((load + k.occ - 1) / k.occ) * k.fixed + (double)load * mflop / rate;
+    const double mflop = 2.0e-6 * k.cfg.block_m * k.cfg.block_n * (double)K / s;
+    double us = (double)((load + k.occ - 1) / k.occ) * k.fixed + (double)load * mflop / rate;
+    if (s > 1) us += 3.0 + (double)s * M * N * 4.0 / 3.0e6;
     if (us < best_us) {
       best_us = us;
       c = k.cfg;
+      c_split = s;
     }
   }
   *cfg = c;
-  if (split_k) {
-    const long t = tiles(c.block_m, c.block_n);
-    int s = 1;
-    if (t < cus / 2 && K >= 2048) {
-      s = beam_slice_heuristic((int)t, cus);
-      const int ktiles = (K + kBK - 1) / kBK;
-      if (s > ktiles / 4) s = ktiles / 4;  // keep at least 4 K tiles per slice
-      if (s < 1) s = 1;
-    }
-    if (s > 1) cfg->pipeline = 2;  // few workgroups per CU: a long prefetch queue keeps HBM busy
-    *split_k = s;
-  }
+  if (!may_split && tiles(c.block_m, c.block_n) < cus / 2 && K >= 2048)
+    cfg->pipeline = 2;  // few workgroups per CU: a long prefetch queue keeps HBM busy
+  if (split_k) *split_k = c_split;
   return BEAM_OK;
 }
+
+}  // namespace
+
+extern "C" {
 
 int beam_gemmrc(const void* A, const void* B, void* C, int M, int N, int K, int dtype,
                 const beam_tile_cfg* cfg, void* stream) {
@@ -457,7 +488,7 @@ static int effective_split(int M, int N, int K, const beam_tile_cfg& c, int spli
   if (s <= 0) {
     const int cus = g_dev.cus > 0 ? g_dev.cus : 256;
     const long t = (long)((M + c.block_m - 1) / c.block_m) * ((N + c.block_n - 1) / c.block_n);
-    s = beam_slice_heuristic((int)(t > 1 << 20 ? 1 << 20 : t), cus);
+    s = auto_slices(t, K, cus);
   }
   if (s > ktiles) s = ktiles;
   if (s < 1) s = 1;
@@ -469,7 +500,7 @@ int beam_splitk_effective(int M, int N, int K, const beam_tile_cfg* cfg, int spl
   beam_tile_cfg c;
   const KernelSet* ks;
   if (M <= 0 || N <= 0 || K < 0) return 1;
-  if (resolve_cfg(cfg, M, N, K, &c, &ks)) return -1;
+  if (resolve_cfg(cfg, M, N, K, &c, &ks, true)) return -1;
   return effective_split(M, N, K, c, split_k);
 }
 
@@ -486,7 +517,7 @@ int beam_gemmrc_splitk(const void* A, const void* B, void* C, int M, int N, int 
   }
   beam_tile_cfg c;
   const KernelSet* ks;
-  if ((rc = resolve_cfg(cfg, M, N, K, &c, &ks))) return rc;
+  if ((rc = resolve_cfg(cfg, M, N, K, &c, &ks, true))) return rc;
   const int s = effective_split(M, N, K, c, split_k);
   if (s == 1) {  // nothing to reduce: the plain kernel writes C directly
     GemmParams p = base_params(A, B, M, N, K, c);

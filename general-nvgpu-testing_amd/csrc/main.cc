@@ -498,7 +498,7 @@ int cli_bench(const Args& a) {
                                     : BEAM_OP_GEMM;
   beam_tile_cfg cfg;
   int split = 1;
-  if (beam_default_config(M, N, K, &cfg, &split) != BEAM_OK) return 2;
+  if (beam_default_config(M, N, K, &cfg, op == BEAM_OP_SPLITK ? &split : nullptr) != BEAM_OK) return 2;
   if (a.has("tile") && !parse_pair(a.str("tile", ""), &cfg.block_m, &cfg.block_n)) return 2;
   if (a.has("wave") && !parse_pair(a.str("wave", ""), &cfg.wave_m, &cfg.wave_n)) return 2;
   cfg.pipeline = a.num("pipeline", cfg.pipeline);

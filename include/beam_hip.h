@@ -58,8 +58,10 @@ int beam_device_info(char* name, int len, int* compute_units, int* clock_khz, si
  * Replaces the hard-coded search spaces of python/beam/tuner.py:52-95. */
 int beam_num_configs(void);
 int beam_get_config(int index, beam_tile_cfg* out);
-/* Library default for a problem: writes the configuration and the split factor (1 = no
- * split).  Replaces CUTLASS's default shapes, cuda/cutlass_kernels/cutlass_gemmrc.cu:22-24. */
+/* Library default for a problem: writes the configuration and, if split_k is not NULL, the
+ * number of K slices that goes with it (1 = no split; the tile is then the one that is best
+ * *with* that many slices and a workspace).  split_k == NULL: the best tile without a split.
+ * Replaces CUTLASS's default shapes, cuda/cutlass_kernels/cutlass_gemmrc.cu:22-24. */
 int beam_default_config(int M, int N, int K, beam_tile_cfg* cfg, int* split_k);
 
 /* ---- tiled GEMM ------------------------------------------------------------------------ */
@@ -80,14 +82,19 @@ int beam_custom_gemmrc_256x128(const void* A, const void* B, void* C, int M, int
 
 /* ---- split-K ---------------------------------------------------------------------------- */
 
-/* Slices the library would choose for `tiles` output tiles on `compute_units` CUs: the rule of
+/* The reference's slice count for `tiles` output tiles on `compute_units` CUs: the rule of
  * get_slice_heuristic (cuda/cutlass_kernels/cutlass_gemmrc_splitk.cu:44-57) with the device's
- * CU count in place of the hard-coded 108. */
+ * CU count in place of the hard-coded 108.  Kept for callers that want that rule; it aims at a
+ * last round of workgroups that is at least half full, which on this machine (one workgroup
+ * of a split-K tile per CU, launch-latency bound) is slower than exactly one full round, so
+ * beam_gemmrc_splitk with split_k <= 0 uses floor(CUs / tiles) instead (at most 64, at least
+ * 4 K tiles of 64 per slice; 1 when the tiles already fill half the CUs). */
 int beam_slice_heuristic(int tiles, int compute_units);
 /* Bytes of fp32 workspace for `split_k` partial results (replaces the hidden grow-only
  * buffer get_the_buffer, cutlass_gemmrc_splitk.cu:31-42: the caller owns the workspace). */
 size_t beam_splitk_workspace_bytes(int M, int N, int split_k);
-/* split_k <= 0: heuristic.  The effective factor is clamped to [1, ceil(K/64)].
+/* split_k <= 0: the library chooses (see above; with cfg == NULL the tile is chosen together
+ * with its slice count).  The effective factor is clamped to [1, ceil(K/64)].
  * Slice s covers K elements [s*len, (s+1)*len), len = ceil(ceil(K/64)/split_k)*64; partial
  * sums are fp32 in ws[split][M][N]; a second kernel adds them in slice order 0,1,2,... and
  * rounds once, so results are bit-identical from run to run.

@@ -56,6 +56,20 @@ def test_ln_small(gpu, beamc, oracle, shape):
                 check_ln(oracle, got, ref, dtype, f"{shape} dtype {dtype} {cfg.name if cfg else 'default'} mode {mode}")
 
 
+def test_ln_every_config(gpu, beamc, oracle):
+    """Ragged 300 x 1000 x 200, every compiled tile with every LDS slot count, both modes.  With two
+    slots per operand the 256-row tiles stage their output through LDS in two passes."""
+    M, N, K = 300, 1000, 200
+    a, b, g, bt = make_ln_inputs(beamc, M, N, K, F16, 23)
+    ref = oracle.gemmrc_ln(a, b, g, bt, 1e-5, F16)
+    for cfg in beamc.list_configs():
+        for pipe in (0, 1, 2):
+            c = beamc.TileConfig(cfg.block_m, cfg.block_n, cfg.wave_m, cfg.wave_n, pipe, 0)
+            for mode in (beamc.LN_TWOPASS, beamc.LN_FUSED):
+                got = run_ln(beamc, a, b, g, bt, F16, config=c, mode=mode)
+                check_ln(oracle, got, ref, F16, f"{c.name} mode {mode}")
+
+
 def test_ln_4096_cube(gpu, beamc, oracle):
     """X[4096x4096] . W[4096x4096]^T, LayerNorm over N = 4096, eps = 1e-5."""
     M = N = K = 4096
