@@ -331,25 +331,29 @@ def gemmrc_spec(a, b, c, shape_threadblock=(128, 128), shape_warp=(64, 64), pipe
     _check(lib.beam_gemmrc(pa, pb, pc, M, N, K, d, ctypes.byref(cfg), st))
 
 
+def _splitk(a, b, c, cfgp, split_k_slices: int) -> None:
+    pa, pb, pc, M, N, K, d, st = _problem(a, b, c)
+    s = lib.beam_splitk_effective(M, N, K, cfgp, split_k_slices)
+    if s < 0:
+        raise BeamError(2, lib.beam_last_error().decode())
+    need = lib.beam_splitk_workspace_bytes(M, N, s) if s > 1 else 0
+    ws = _get_workspace(need) if need else None
+    _check(lib.beam_gemmrc_splitk(pa, pb, pc, M, N, K, d, cfgp, split_k_slices,
+                                  ws.ptr if ws else None, ws.nbytes if ws else 0, st))
+
+
 def gemmrc_splitk(a, b, c, split_k_slices: int = 0) -> None:
-    """Split-K with the library's default small tile; split_k_slices <= 0 = heuristic
+    """Split-K with the library's default tile for the problem; split_k_slices <= 0: the library
+    picks the slice count as well (one full round of workgroups)
     (reference: cutlass_gemmrc_splitk, python/beam/_C/beam_C.pyi:18)."""
-    gemmrc_splitk_spec(a, b, c, shape_threadblock=(128, 128), shape_warp=(64, 64),
-                       split_k_slices=split_k_slices)
+    _splitk(a, b, c, None, split_k_slices)
 
 
 def gemmrc_splitk_spec(a, b, c, shape_threadblock=(128, 128), shape_warp=(64, 64), split_k_slices: int = 0,
                        pipeline: int = 0, group_m: int = 0) -> None:
     """Split-K with explicit tiles (reference: cutlass_gemmrc_splitk_spec, beam_C.pyi:20)."""
-    pa, pb, pc, M, N, K, d, st = _problem(a, b, c)
     cfg = _cfg_from_shapes(shape_threadblock, shape_warp, pipeline, group_m)
-    s = lib.beam_splitk_effective(M, N, K, ctypes.byref(cfg), split_k_slices)
-    if s < 0:
-        raise BeamError(2, lib.beam_last_error().decode())
-    need = lib.beam_splitk_workspace_bytes(M, N, s) if s > 1 else 0
-    ws = _get_workspace(need) if need else None
-    _check(lib.beam_gemmrc_splitk(pa, pb, pc, M, N, K, d, ctypes.byref(cfg), split_k_slices,
-                                  ws.ptr if ws else None, ws.nbytes if ws else 0, st))
+    _splitk(a, b, c, ctypes.byref(cfg), split_k_slices)
 
 
 LN_AUTO, LN_TWOPASS, LN_FUSED = 0, 1, 2
