@@ -148,6 +148,10 @@ def test_bf16_sweep(gpu, beamc, oracle):
         for cfg in [None, beamc.TileConfig(128, 128, 64, 64), beamc.TileConfig(64, 64, 32, 32)]:
             got = run_gemm(beamc, a, b, BF16, cfg)
             assert_close(oracle, got, ref, K, BF16, f"{(M, N, K)}")
+    for (M, N, K) in [(4096, 4096, 4096), (4096, 11008, 4096), (4096, 4096, 11008)]:
+        a = beamc.host_uniform((M, K), BF16, 5, 0)
+        b = beamc.host_uniform((N, K), BF16, 5, 1)
+        assert_close(oracle, run_gemm(beamc, a, b, BF16), oracle.gemmrc(a, b, BF16), K, BF16, f"{(M, N, K)}")
 
 
 @pytest.mark.parametrize("shape", [(512, 512, 512), (2048, 2048, 2048), (4096, 4096, 4096),
@@ -159,6 +163,33 @@ def test_fp16_sweep(gpu, beamc, oracle, shape):
     ref = oracle.gemmrc(a, b, F16)
     got = run_gemm(beamc, a, b, F16)
     assert_close(oracle, got, ref, K, F16, f"{shape}")
+
+
+def _decode(bits, dtype):
+    if dtype == F16:
+        return bits.view(np.float16).astype(np.float64)
+    return (bits.astype(np.uint32) << 16).view(np.float32).astype(np.float64)
+
+
+@pytest.mark.parametrize("dtype", [F16, BF16])
+def test_16384_cube_sampled_rows_and_column_sums(gpu, beamc, oracle, dtype):
+    """The largest square of the sweep, 4096 tiles of 256 x 256.  The oracle computes one row out of every
+    256-row band (every tile contributes columns to the comparison), and every element enters the
+    column sums 1^T C, which must equal (1^T A) B^T (float64) up to the rounding of the 16-bit outputs."""
+    M = N = K = 16384
+    a = beamc.host_uniform((M, K), dtype, 8, 0)
+    b = beamc.host_uniform((N, K), dtype, 8, 1)
+    got = run_gemm(beamc, a, b, dtype)
+    rows = np.array([t * 256 + (37 * t) % 256 for t in range(M // 256)])
+    ref = oracle.gemmrc(np.ascontiguousarray(a[rows]), b, dtype)
+    r = assert_close(oracle, np.ascontiguousarray(got[rows]), ref, K, dtype, "sampled rows")
+    assert abs(r["rms_ref"] / (K ** 0.5 / 3) - 1) < 0.05      # RMS(C) = sqrt(K)/3 for uniform inputs
+    bf = _decode(b, dtype)
+    want = bf @ _decode(a, dtype).sum(axis=0)                  # [N]
+    have = _decode(got, dtype).sum(axis=0)
+    half_ulp = 2.0 ** -11 if dtype == F16 else 2.0 ** -8
+    bound = 8 * np.sqrt(M) * half_ulp * 4 * r["rms_ref"]       # 8 sigma of M roundings of values up to ~4 RMS
+    assert np.abs(have - want).max() <= bound, (np.abs(have - want).max(), bound)
 
 
 def test_headline_8192_cube(gpu, beamc, oracle):
