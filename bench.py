@@ -200,6 +200,18 @@ def extra_nn(_C):
     return {"shape": [M, N, K], "us": round(ms * 1e3, 1), "TFLOPs": round(2.0 * M * N * K / (ms * 1e-3) / 1e12, 1)}
 
 
+def extra_bf16(_C):
+    """The headline shape in bf16 (same kernel template, v_mfma_f32_16x16x32_bf16)."""
+    M = N = K = 8192
+    a = _C.DeviceArray.from_numpy(_C.host_normal((M, K), _C.BF16, 7, 0, 0.0, K ** -0.5), _C.BF16)
+    b = _C.DeviceArray.from_numpy(_C.host_normal((N, K), _C.BF16, 7, 1, 0.0, K ** -0.5), _C.BF16)
+    c = _C.DeviceArray((M, N), _C.BF16)
+    ms = _C.bench(_C.OP_GEMM, a, b, c, warmup=100, iters=200)
+    for t in (a, b, c):
+        t.free()
+    return {"shape": [M, N, K], "us": round(ms * 1e3, 1), "TFLOPs": round(2.0 * M * N * K / (ms * 1e-3) / 1e12, 1)}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -259,7 +271,7 @@ def main():
         x.free()
     if not args.no_extra:
         out["extra"] = {"splitk": extra_splitk(_C), "gemm_ln": extra_ln(_C), "gemm_silu": extra_silu(_C),
-                        "matmul_nn": extra_nn(_C)}
+                        "matmul_nn": extra_nn(_C), "gemm_bf16": extra_bf16(_C)}
     print(json.dumps(out))
     if "check" in out and not out["check"]["ok"]:
         sys.exit("bench.py: GPU result outside the tolerance of the CPU oracle")
