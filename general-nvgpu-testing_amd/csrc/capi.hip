@@ -117,17 +117,17 @@ int auto_slices(long tiles, int K, int cus) {
   return s < 1 ? 1 : (int)s;
 }
 
-int choose_default(int M, int N, int K, bool may_split, beam_tile_cfg* cfg, int* split_k);
+int choose_default(int M, int N, int K, int split_req, beam_tile_cfg* cfg, int* split_k);
 
-// may_split: the caller can run K slices (it has a workspace); the default tile is then chosen together
-// with its slice count.
+// split_req: -1 the caller cannot run K slices (no workspace); 0 it can, and leaves the number to
+// the library; > 0 it asks for that many.  The default tile is chosen for that situation.
 int resolve_cfg(const beam_tile_cfg* in, int M, int N, int K, beam_tile_cfg* out, const KernelSet** ks,
-                bool may_split = false) {
+                int split_req = -1) {
   if (in) {
     *out = *in;
   } else {
     int s;
-    int rc = choose_default(M, N, K, may_split, out, &s);
+    int rc = choose_default(M, N, K, split_req, out, &s);
     if (rc) return rc;
   }
   if (out->pipeline < 0 || out->pipeline > 2) return fail(BEAM_ERR_UNSUPPORTED, "pipeline %d: 0 (3 A + 2 B LDS slots), 1 (2 + 2) or 2 (deep)", out->pipeline);
@@ -292,14 +292,14 @@ int beam_slice_heuristic(int tiles, int compute_units) {
 }
 
 int beam_default_config(int M, int N, int K, beam_tile_cfg* cfg, int* split_k) {
-  return choose_default(M, N, K, split_k != nullptr, cfg, split_k);
+  return choose_default(M, N, K, split_k ? 0 : -1, cfg, split_k);
 }
 
 }  // extern "C"
 
 namespace {
 
-int choose_default(int M, int N, int K, bool may_split, beam_tile_cfg* cfg, int* split_k) {
+int choose_default(int M, int N, int K, int split_req, beam_tile_cfg* cfg, int* split_k) {
   if (!cfg) return fail(BEAM_ERR_INVALID, "null cfg");
   const int cus = g_dev.cus > 0 ? g_dev.cus : 256;
   auto tiles = [&](int bm, int bn) { return (long)((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
@@ -335,7 +335,11 @@ int choose_default(int M, int N, int K, bool may_split, beam_tile_cfg* cfg, int*
   double best_us = 1e300;
   for (const Candidate& k : kCandidates) {
     const long t = tiles(k.cfg.block_m, k.cfg.block_n);
-    const int s = (may_split && k.cfg.pipeline == 2) ? auto_slices(t, K, cus) : 1;
+    int s = 1;
+    if (k.cfg.pipeline == 2 && split_req >= 0) {
+      const int ktiles = (K + kBK - 1) / kBK;
+      s = split_req == 0 ? auto_slices(t, K, cus) : (split_req < ktiles ? split_req : (ktiles > 0 ? ktiles : 1));
+    }
     const long load = (t * s + cus - 1) / cus;  // workgroups per CU
     const long conc = load < k.occ ? load : k.occ;
     const double rate = k.occ == 1 ? k.alone : k.alone + (k.full - k.alone) * (double)(conc - 1) / (k.occ - 1);
@@ -349,7 +353,7 @@ int choose_default(int M, int N, int K, bool may_split, beam_tile_cfg* cfg, int*
     }
   }
   *cfg = c;
-  if (!may_split && tiles(c.block_m, c.block_n) < cus / 2 && K >= 2048)
+  if (split_req < 0 && tiles(c.block_m, c.block_n) < cus / 2 && K >= 2048)
     cfg->pipeline = 2;  // few workgroups per CU: a long prefetch queue keeps HBM busy
   if (split_k) *split_k = c_split;
   return BEAM_OK;
@@ -500,7 +504,7 @@ int beam_splitk_effective(int M, int N, int K, const beam_tile_cfg* cfg, int spl
   beam_tile_cfg c;
   const KernelSet* ks;
   if (M <= 0 || N <= 0 || K < 0) return 1;
-  if (resolve_cfg(cfg, M, N, K, &c, &ks, true)) return -1;
+  if (resolve_cfg(cfg, M, N, K, &c, &ks, split_k > 0 ? split_k : 0)) return -1;
   return effective_split(M, N, K, c, split_k);
 }
 
@@ -517,7 +521,7 @@ int beam_gemmrc_splitk(const void* A, const void* B, void* C, int M, int N, int 
   }
   beam_tile_cfg c;
   const KernelSet* ks;
-  if ((rc = resolve_cfg(cfg, M, N, K, &c, &ks, true))) return rc;
+  if ((rc = resolve_cfg(cfg, M, N, K, &c, &ks, split_k > 0 ? split_k : 0))) return rc;
   const int s = effective_split(M, N, K, c, split_k);
   if (s == 1) {  // nothing to reduce: the plain kernel writes C directly
     GemmParams p = base_params(A, B, M, N, K, c);
