@@ -110,6 +110,28 @@ def test_slice_heuristic_matches_reference_rule(beamc, oracle):
     assert beamc.lib.beam_slice_heuristic(4, 108) == 41
 
 
+def test_automatic_slice_count(beamc):
+    """split_k <= 0: one full round of workgroups on the 256 CUs, at most 64 slices, at least 4 K tiles
+    of 64 per slice, and no split once the tiles fill half the machine.  With no tile given either,
+    the library picks both (a deep-pipeline tile with more than one slice for a split-K shaped problem,
+    no split for a big square)."""
+    eff = beamc.lib.beam_splitk_effective
+    t64 = beamc.TileConfig(64, 64, 32, 32, 2, 0).to_c()
+    t64x128 = beamc.TileConfig(64, 128, 32, 64, 2, 0).to_c()
+    assert eff(256, 256, 32768, ctypes.byref(t64), 0) == 16        # 16 tiles x 16 slices = 256
+    assert eff(256, 256, 32768, ctypes.byref(t64x128), 0) == 32    # 8 tiles x 32
+    assert eff(64, 64, 32768, ctypes.byref(t64), 0) == 64          # one tile: capped
+    assert eff(256, 256, 1024, ctypes.byref(t64), 0) == 4          # 16 K tiles: 4 per slice
+    assert eff(1024, 1024, 8192, ctypes.byref(t64), 0) == 1        # 256 tiles already
+    assert eff(640, 640, 16384, ctypes.byref(t64), 0) == 2         # 100 tiles
+    cfg, s = beamc.default_config(256, 256, 32768)
+    assert s > 1 and cfg.pipeline == 2 and eff(256, 256, 32768, None, 0) == s
+    cfg, s = beamc.default_config(8192, 8192, 8192)
+    assert s == 1 and eff(8192, 8192, 8192, None, 0) == 1
+    cfg, s = beamc.default_config(256, 256, 32768, split=False)
+    assert s == 1
+
+
 def test_split_partition(beamc, oracle):
     cfg = beamc.TileConfig(64, 64, 32, 32).to_c()
     for K in (64, 200, 1000, 4104, 32768):
