@@ -116,6 +116,8 @@ def _load() -> ctypes.CDLL:
     L.beam_dbg_kmajor_lds_offset.argtypes = [i, i, i]
     L.beam_dbg_band_block_tile.argtypes = [i, i, i, i, i, ctypes.POINTER(i), ctypes.POINTER(i)]
     L.beam_dbg_band_block_grid.argtypes = [i, i, i]
+    L.beam_dbg_band_xcd_tile.argtypes = [i, i, i, i, ctypes.POINTER(i), ctypes.POINTER(i)]
+    L.beam_dbg_band_xcd_grid.argtypes = [i, i, i]
     return L
 
 

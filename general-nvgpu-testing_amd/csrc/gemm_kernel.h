@@ -105,7 +105,7 @@ struct GemmParams {
   int k_slice;   // K elements per split-K slice, a multiple of kBK
   int splits;    // number of K slices (1 = no split); the grid holds tiles_m * tiles_n * splits workgroups
   int group_m;   // rasterisation group height in tiles (fused LayerNorm: bands per band group)
-  int group_n;   // fused LayerNorm: columns of a band group owned by one XCD
+  int group_n;   // fused LayerNorm: columns of a band group owned by one XCD; 0: whole bands, group_m of them, per XCD
   // Side job (kEpiStoreSide): y[i] = silu(x[i]) over a flat 16-bit array.  The whole 8-element
   // groups of the array are cut into units of side_width bytes (16, 8 or 4), dealt out in
   // contiguous runs of side_iters * threads units per workgroup, `threads` units per K tile; the
@@ -228,7 +228,8 @@ struct GemmTile {
     TileCoord tc;
     int slice = 0;
     if (EPI == kEpiLnFused) {
-      tc = band_block_tile(blockIdx.x, p.tiles_m, p.tiles_n, p.group_m, p.group_n);
+      tc = p.group_n > 0 ? band_block_tile(blockIdx.x, p.tiles_m, p.tiles_n, p.group_m, p.group_n)
+                         : band_xcd_tile(blockIdx.x, p.tiles_m, p.tiles_n, p.group_m);
       if (tc.tm < 0) return;
     } else if (p.splits > 1) {
       const int tiles = p.tiles_m * p.tiles_n;

@@ -110,6 +110,30 @@ BEAM_HD int band_block_grid(int tiles_m, int gb, int gc) {
   return kNumXcd * ((tiles_m + gb - 1) / gb) * gb * gc;
 }
 
+// The same contract with whole bands on one XCD, for bands short enough (tiles_n * bx <= CUs per
+// XCD): XCD x holds bands (g * 8 + x) * bx .. + bx - 1 in round g, M fastest.  The XCDs of one part
+// run at clocks that differ by several percent under a matrix-core load (measured: the same tiles
+// take 5% longer on some XCDs than on others), so a band spread over all XCDs waits for the slowest
+// of them; a band inside one XCD finishes together.  L2 traffic is the same as for band_block_tile
+// (bx A panels + tiles_n B panels per XCD and round, against gb + gc).
+BEAM_HD TileCoord band_xcd_tile(int wg, int tiles_m, int tiles_n, int bx) {
+  const int xcd = wg % kNumXcd;
+  const int local = wg / kNumXcd;
+  const int per_group = bx * tiles_n;
+  const int g = local / per_group;
+  const int within = local - g * per_group;
+  TileCoord t;
+  t.tm = (g * kNumXcd + xcd) * bx + within % bx;
+  t.tn = within / bx;
+  if (t.tm >= tiles_m) t.tm = -1;
+  return t;
+}
+
+BEAM_HD int band_xcd_grid(int tiles_m, int tiles_n, int bx) {
+  const int bands_per_round = kNumXcd * bx;
+  return ((tiles_m + bands_per_round - 1) / bands_per_round) * bands_per_round * tiles_n;
+}
+
 BEAM_HD TileCoord tile_of_workgroup(int wg, int tiles_m, int tiles_n, int group_m) {
   return grouped_tile(xcd_remap(wg, tiles_m * tiles_n), tiles_m, tiles_n, group_m);
 }

@@ -269,6 +269,10 @@ int beam_dbg_kmajor_lds_offset(int k, int n, int block_n);
  * the id is padding), and the size of that grid. */
 int beam_dbg_band_block_tile(int wg, int tiles_m, int tiles_n, int gb, int gc, int* tm, int* tn);
 int beam_dbg_band_block_grid(int tiles_m, int gb, int gc);
+/* The same for the order that keeps whole bands (bx at a time) on one XCD, used when a band is
+ * short enough for it. */
+int beam_dbg_band_xcd_tile(int wg, int tiles_m, int tiles_n, int bx, int* tm, int* tn);
+int beam_dbg_band_xcd_grid(int tiles_m, int tiles_n, int bx);
 
 #ifdef __cplusplus
 }

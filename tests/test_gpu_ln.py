@@ -43,7 +43,7 @@ def check_ln(oracle, got_bits, ref32, dtype, what):
 
 
 @pytest.mark.parametrize("shape", [(256, 512, 256), (1024, 1024, 512), (300, 1000, 200), (64, 4096, 128),
-                                   (17, 40, 64)])
+                                   (17, 40, 64), (16384, 2048, 128), (4200, 1000, 72)])
 def test_ln_small(gpu, beamc, oracle, shape):
     M, N, K = shape
     for dtype in (F16, BF16):

@@ -34,6 +34,30 @@ def test_rasterisation_is_xcd_local(beamc):
         assert len(ms) == 8 and len(ns) == 4, (xcd, sorted(block))
 
 
+@pytest.mark.parametrize("tiles_m,tiles_n,bx", [(16, 16, 2), (64, 8, 4), (40, 9, 3), (8, 32, 1), (33, 4, 8), (9, 16, 1)])
+def test_band_xcd_order(beamc, tiles_m, tiles_n, bx):
+    """The fused GEMM+LayerNorm's order for short bands: every tile exactly once, padding flagged, all
+    column tiles of a band on one XCD (ids congruent modulo 8) and inside one group of at most 32
+    consecutive workgroups of that XCD (resident together)."""
+    L = beamc.lib
+    assert bx * tiles_n <= 32
+    grid = L.beam_dbg_band_xcd_grid(tiles_m, tiles_n, bx)
+    assert grid % 8 == 0
+    seen = {}
+    for wg in range(grid):
+        a, b = ctypes.c_int(), ctypes.c_int()
+        assert L.beam_dbg_band_xcd_tile(wg, tiles_m, tiles_n, bx, ctypes.byref(a), ctypes.byref(b)) == 0
+        if a.value < 0:
+            continue
+        assert 0 <= a.value < tiles_m and 0 <= b.value < tiles_n and (a.value, b.value) not in seen
+        seen[(a.value, b.value)] = wg
+    assert len(seen) == tiles_m * tiles_n
+    for band in range(tiles_m):
+        ids = [seen[(band, tn)] for tn in range(tiles_n)]
+        assert len({w % 8 for w in ids}) == 1
+        assert len({(w // 8) // (bx * tiles_n) for w in ids}) == 1
+
+
 @pytest.mark.parametrize("tiles_m,tiles_n", [(16, 16), (32, 32), (2, 43), (5, 7), (1, 1), (3, 64), (40, 9)])
 def test_band_block_order(beamc, tiles_m, tiles_n):
     """Padded band-block grid of the fused GEMM+LayerNorm: every tile exactly once, padding ids are
