@@ -136,7 +136,7 @@ def extra_splitk(_C):
     graph_us = splitk_graph_us(_C, a, b, c, best_split[2], best_split[3])
     cold_us = splitk_graph_us(_C, a, b, c, best_split[2], best_split[3], calls=48, operand_sets=12)
     # what a call that names neither tile nor slice count gets
-    auto_cfg, auto_s = _C.default_config(M, N, K)
+    auto_cfg, auto_s = _C.default_config(M, N, K, split=True)
     auto_ms = min(_C.bench(1, a, b, c, config=None, split_k=0, warmup=20, iters=100) for _ in range(2))
     for x in (a, b, c):
         x.free()

@@ -165,9 +165,10 @@ def list_configs() -> List[TileConfig]:
     return out
 
 
-def default_config(M: int, N: int, K: int, split: bool = True):
-    """(tile, K slices) the library would use.  split=True: the best tile together with its slice
-    count (for callers with a workspace); split=False: the best tile without a split, slices = 1."""
+def default_config(M: int, N: int, K: int, split: bool = False):
+    """(tile, K slices) the library would use.  split=False: the best tile for a call without a
+    workspace (gemmrc), slices = 1; split=True: the best tile together with its slice count
+    (gemmrc_splitk)."""
     c = _TileCfg()
     s = ctypes.c_int(1)
     _check(lib.beam_default_config(M, N, K, ctypes.byref(c), ctypes.byref(s) if split else None))

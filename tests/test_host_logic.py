@@ -148,7 +148,7 @@ def test_automatic_slice_count(beamc):
     assert eff(256, 256, 1024, ctypes.byref(t64), 0) == 4          # 16 K tiles: 4 per slice
     assert eff(1024, 1024, 8192, ctypes.byref(t64), 0) == 1        # 256 tiles already
     assert eff(640, 640, 16384, ctypes.byref(t64), 0) == 2         # 100 tiles
-    cfg, s = beamc.default_config(256, 256, 32768)
+    cfg, s = beamc.default_config(256, 256, 32768, split=True)
     assert s > 1 and cfg.pipeline == 2 and eff(256, 256, 32768, None, 0) == s
     cfg, s = beamc.default_config(8192, 8192, 8192)
     assert s == 1 and eff(8192, 8192, 8192, None, 0) == 1
@@ -246,7 +246,7 @@ def test_config_table(beamc):
         assert (3 * c.block_m + 2 * c.block_n) * 128 <= 160 * 1024
     cfg, split = beamc.default_config(8192, 8192, 8192)
     assert (cfg.block_m, cfg.block_n) == (256, 256) and split == 1
-    cfg, split = beamc.default_config(256, 256, 32768)
+    cfg, split = beamc.default_config(256, 256, 32768, split=True)
     assert split > 1
 
 
