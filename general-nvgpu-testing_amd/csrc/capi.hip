@@ -307,10 +307,11 @@ int choose_default(int M, int N, int K, int split_req, beam_tile_cfg* cfg, int* 
   // them at a time (what LDS allows); a workgroup costs a fixed start-up / epilogue time plus its flops
   // at the per-CU rate of its tile shape, which is higher when several workgroups share the CU.  The
   // rates (TFLOP/s per CU, alone / with a full CU) and fixed costs (us) are fits to timings of all
-  // compiled tiles on 35 shapes from 512^3 to 8192^3 (square, skinny and short-K) on an MI355X:
-  // the pick is within 0.7% of the best tile on average, 5.4% at worst (tile-count thresholds:
-  // 6% and 76%).  The 192-row tile is there for what 256 rows divide badly: 3072^3 is 0.75 of a
-  // round of its tiles against 0.56 of a round of 256 x 256 ones, 50.5 against 58.6 us.
+  // compiled tiles on 39 shapes from 512^3 to 8192^3 (square, skinny and short-K) on an MI355X:
+  // the pick is within 0.8% of the best tile on average, 6.7% at worst (tile-count thresholds:
+  // 6% and 76%).  The 224- and 192-row tiles are there for what 256 rows divide badly: 3072^3 is
+  // 0.75 of a round of 192 x 256 tiles against 0.56 of a round of 256 x 256 ones (49.5 against
+  // 58.6 us), 7168^3 is 3.5 rounds of 224 x 256 tiles against 3.06 (546 against 613 us).
   struct Candidate {
     beam_tile_cfg cfg;
     int occ;
@@ -318,7 +319,8 @@ int choose_default(int M, int N, int K, int split_req, beam_tile_cfg* cfg, int* 
   };
   static const Candidate kCandidates[] = {
       {{256, 256, 128, 64, 0, default_group_m(256, 256)}, 1, 6.04, 6.04, 8.0},
-      {{192, 256, 96, 64, 0, default_group_m(192, 256)}, 1, 5.8, 5.8, 8.0},
+      {{224, 256, 112, 64, 0, default_group_m(224, 256)}, 1, 5.95, 5.95, 8.0},
+      {{192, 256, 96, 64, 0, default_group_m(192, 256)}, 1, 5.22, 5.22, 8.0},
       {{256, 128, 64, 64, 0, default_group_m(256, 128)}, 1, 4.99, 4.99, 6.0},
       {{128, 256, 64, 64, 0, default_group_m(128, 256)}, 1, 4.8, 4.8, 6.0},
       {{128, 128, 64, 64, 0, default_group_m(128, 128)}, 2, 3.8, 4.4, 3.42},

@@ -85,6 +85,7 @@ KernelSet make_kernel_set() {
   X(256, 256, 128, 64)       \
   X(256, 256, 64, 128)       \
   X(256, 256, 128, 128)      \
+  X(224, 256, 112, 64)       \
   X(192, 256, 96, 64)        \
   X(256, 128, 64, 64)        \
   X(256, 128, 128, 32)       \
