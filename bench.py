@@ -200,6 +200,23 @@ def extra_nn(_C):
     return {"shape": [M, N, K], "us": round(ms * 1e3, 1), "TFLOPs": round(2.0 * M * N * K / (ms * 1e-3) / 1e12, 1)}
 
 
+def extra_shapes(_C):
+    """A few shapes of the sweep with the tile the library picks for them."""
+    out = []
+    for (M, N, K) in [(2048, 2048, 2048), (3072, 3072, 3072), (4096, 4096, 4096), (6144, 6144, 6144), (7168, 7168, 7168),
+                      (4096, 11008, 4096), (4096, 4096, 11008), (16384, 16384, 2048)]:
+        a = _C.DeviceArray.from_numpy(_C.host_normal((M, K), _C.F16, 5, 0, 0.0, K ** -0.5))
+        b = _C.DeviceArray.from_numpy(_C.host_normal((N, K), _C.F16, 5, 1, 0.0, K ** -0.5))
+        c = _C.DeviceArray((M, N))
+        cfg, _ = _C.default_config(M, N, K, split=False)
+        ms = min(_C.bench(_C.OP_GEMM, a, b, c, warmup=50, iters=100) for _ in range(2))
+        for t in (a, b, c):
+            t.free()
+        out.append({"shape": [M, N, K], "tile": cfg.name, "us": round(ms * 1e3, 1),
+                    "TFLOPs": round(2.0 * M * N * K / (ms * 1e-3) / 1e12, 1)})
+    return out
+
+
 def extra_bf16(_C):
     """The headline shape in bf16 (same kernel template, v_mfma_f32_16x16x32_bf16)."""
     M = N = K = 8192
@@ -271,7 +288,7 @@ def main():
         x.free()
     if not args.no_extra:
         out["extra"] = {"splitk": extra_splitk(_C), "gemm_ln": extra_ln(_C), "gemm_silu": extra_silu(_C),
-                        "matmul_nn": extra_nn(_C), "gemm_bf16": extra_bf16(_C)}
+                        "matmul_nn": extra_nn(_C), "gemm_bf16": extra_bf16(_C), "fp16_shapes": extra_shapes(_C)}
     print(json.dumps(out))
     if "check" in out and not out["check"]["ok"]:
         sys.exit("bench.py: GPU result outside the tolerance of the CPU oracle")
