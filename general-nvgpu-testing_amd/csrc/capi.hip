@@ -383,7 +383,19 @@ int beam_gemmrc(const void* A, const void* B, void* C, int M, int N, int K, int 
   if ((rc = resolve_cfg(cfg, M, N, K, &c, &ks))) return rc;
   GemmParams p = base_params(A, B, M, N, K, c);
   p.C = C;
-  BEAM_HIP(ks->launch[dtype][kEpiStore][c.pipeline](p, dim3((unsigned)(p.tiles_m * p.tiles_n), 1, 1), st));
+  // More than one round of workgroups of a large tile: one workgroup per CU walks the tiles and
+  // loads the next one's first operand tiles while it stores the current one (kEpiStoreLoop).
+  // That kernel stores 16 bytes per lane through a buffer descriptor and has no short K tile.
+  // Against one workgroup per tile, same machine: 16384 x 16384 x 2048 822 against 841 us,
+  // 8192 x 8192 x 512 71 against 74.5 us, 8192 x 8192 x 2048 205 against 207 us, 8192^3 no difference.
+  const long tiles = (long)p.tiles_m * p.tiles_n;
+  const int cus = g_dev.cus > 0 ? g_dev.cus : 256;
+  GemmLauncher loop = c.pipeline == 0 ? ks->launch[dtype][kEpiStoreLoop][0] : nullptr;
+  if (loop && tiles > cus && K % kBK == 0 && N % 8 == 0 && ((uintptr_t)C & 15) == 0 && N <= (1 << 21)) {
+    BEAM_HIP(loop(p, dim3((unsigned)cus, 1, 1), st));
+    return BEAM_OK;
+  }
+  BEAM_HIP(ks->launch[dtype][kEpiStore][c.pipeline](p, dim3((unsigned)tiles, 1, 1), st));
   return BEAM_OK;
 }
 

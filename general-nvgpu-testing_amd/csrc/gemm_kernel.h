@@ -84,8 +84,11 @@ enum Epilogue : int {
   kEpiLnStats = 2,  // store fp32 X and per-(row, column-tile) mean / M2 for LayerNorm
   kEpiLnFused = 3,  // LayerNorm in the epilogue: tiles of a row band exchange statistics only
   kEpiStoreSide = 4,  // kEpiStore plus an independent elementwise job (SiLU) streamed through the K loop
+  // kEpiStore for a grid smaller than the tile count: a workgroup walks the tiles id, id + grid, ...
+  // and has the first operand tiles of the next one in flight while it stores the current one
+  kEpiStoreLoop = 5,
 };
-constexpr int kNumEpilogues = 5;
+constexpr int kNumEpilogues = 6;
 
 struct GemmParams {
   const void* A;
@@ -193,6 +196,9 @@ struct GemmTile {
   // The side job adds SV buffer stores and SV buffer loads at the end of every K tile of a loader
   // wavefront; the fills a tile waits for were issued min(AST, BST) - 1 tiles earlier.
   static constexpr bool SIDE = (EPI == kEpiStoreSide);
+  static constexpr bool LOOP = (EPI == kEpiStoreLoop);
+  // global stores of one wavefront per tile when its output leaves as whole rows, 16 bytes per lane
+  static constexpr int NST = TM * (TN / 8) / 64;
   static constexpr int SV = NW / LDW;  // side vectors per loader thread per K tile
   static constexpr int WAIT_STEADY =
       (AST - 2) * LA + (BST - 2) * LB + (SIDE ? 2 * SV * ((AST < BST ? AST : BST) - 1) : 0);
@@ -239,8 +245,8 @@ struct GemmTile {
     } else {
       tc = tile_of_workgroup(blockIdx.x, p.tiles_m, p.tiles_n, p.group_m);
     }
-    const int row0 = tc.tm * BM;
-    const int col0 = tc.tn * BN;
+    int row0 = tc.tm * BM;
+    int col0 = tc.tn * BN;
     const int M = p.M, N = p.N, K = p.K;
 
     // K range of this slice.
@@ -254,16 +260,29 @@ struct GemmTile {
 
     // Buffer descriptors cover exactly the rows of this tile that exist and the K range of
     // this slice; anything else is out of range: reads return zero and touch no memory.
-    const int rows_a = (M - row0) < BM ? (M - row0) : BM;
-    const int rows_b = (N - col0) < BN ? (N - col0) : BN;
+    int rows_a = (M - row0) < BM ? (M - row0) : BM;
+    int rows_b = (N - col0) < BN ? (N - col0) : BN;
     const T* a_base = (const T*)p.A + ((size_t)row0 * K + kb);
     // B as [N][K] (rows of K): like A.  B as [K][N] (B_KMAJOR): the tile's columns start at col0 of
     // row kb; a descriptor is made per K tile (load_b) so that it ends with the tile's last row.
     const T* b_base = B_KMAJOR ? (const T*)p.B + ((size_t)kb * N + col0) : (const T*)p.B + ((size_t)col0 * K + kb);
-    const unsigned bytes_a = klen > 0 ? ((unsigned)(rows_a - 1) * K + klen) * 2u : 0u;
-    const unsigned bytes_b = klen > 0 ? ((unsigned)(rows_b - 1) * K + klen) * 2u : 0u;
+    unsigned bytes_a = klen > 0 ? ((unsigned)(rows_a - 1) * K + klen) * 2u : 0u;
+    unsigned bytes_b = klen > 0 ? ((unsigned)(rows_b - 1) * K + klen) * 2u : 0u;
     const __amdgpu_buffer_rsrc_t rsrc_a = make_rsrc(a_base, bytes_a);
     const __amdgpu_buffer_rsrc_t rsrc_b = make_rsrc(b_base, bytes_b);
+    // kEpiStoreLoop: the same for the next tile of this workgroup (neither split-K nor the [K][N]
+    // layout nor a short K tile exist in that mode: the host sees to it)
+    auto set_tile = [&](int id) {
+      tc = tile_of_workgroup(id, p.tiles_m, p.tiles_n, p.group_m);
+      row0 = tc.tm * BM;
+      col0 = tc.tn * BN;
+      rows_a = (M - row0) < BM ? (M - row0) : BM;
+      rows_b = (N - col0) < BN ? (N - col0) : BN;
+      a_base = (const T*)p.A + (size_t)row0 * K;
+      b_base = (const T*)p.B + (size_t)col0 * K;
+      bytes_a = ((unsigned)(rows_a - 1) * K + klen) * 2u;
+      bytes_b = ((unsigned)(rows_b - 1) * K + klen) * 2u;
+    };
 
     unsigned voff_a[LA], voff_b[LB];
 #pragma unroll
@@ -381,31 +400,37 @@ struct GemmTile {
     };
 
     f32x4 acc[FM][FN];
+    auto zero_acc = [&]() {
 #pragma unroll
-    for (int i = 0; i < FM; ++i)
+      for (int i = 0; i < FM; ++i)
 #pragma unroll
-      for (int j = 0; j < FN; ++j)
+        for (int j = 0; j < FN; ++j)
 #pragma unroll
-        for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.0f;
+          for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.0f;
+    };
+    zero_acc();
 
     // Fragments: both operands are double-buffered in registers (set 0 / set 1).  While the MFMAs
     // of one step consume one set, the LDS reads of the next step fill the other.  They start as
     // zeros so that the very first step of the pipeline multiplies nothing.
     vec8 fa0[FM], fa1[FM], fb0[FN], fb1[FN];
+    auto zero_fragments = [&]() {
 #pragma unroll
-    for (int i = 0; i < FM; ++i)
+      for (int i = 0; i < FM; ++i)
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        fa0[i][e] = 0;
-        fa1[i][e] = 0;
-      }
+        for (int e = 0; e < 8; ++e) {
+          fa0[i][e] = 0;
+          fa1[i][e] = 0;
+        }
 #pragma unroll
-    for (int j = 0; j < FN; ++j)
+      for (int j = 0; j < FN; ++j)
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        fb0[j][e] = 0;
-        fb1[j][e] = 0;
-      }
+        for (int e = 0; e < 8; ++e) {
+          fb0[j][e] = 0;
+          fb1[j][e] = 0;
+        }
+    };
+    zero_fragments();
 
     // ---- side job: state and pieces ------------------------------------------------------
     // side_buf holds the units loaded during the previous K tile; step 1 pushes them through silu
@@ -565,9 +590,19 @@ struct GemmTile {
     // One K tile h: make it visible to every wavefront, then two steps.  Step 0 multiplies the
     // second half of tile h-1 (set 1) while reading the first half of tile h into set 0; step 1
     // multiplies set 0 while reading the second half of tile h into set 1.
+    bool stores_pending = false;  // kEpiStoreLoop: a store epilogue precedes the tile being started
     auto tile_body = [&](int h, auto ld_tag, auto w_tag) {
-      wait_vm_and_lds<WAIT_STEADY>();  // my fills of tile h have landed; my reads of tile h-1 are done
-      bare_barrier();                  // ... and so have everyone else's: the slots of tile h-1 are free
+      // my fills of tile h have landed; my reads of tile h-1 are done
+      if constexpr (!decltype(ld_tag)::value) {
+        wait_lds<0>();  // a wavefront that loads nothing has no fills to wait for
+      } else if constexpr (LOOP) {
+        // the first tile after a store epilogue: that epilogue's NST stores are younger than the fills
+        if (h == 0 && stores_pending) wait_vm_and_lds<WAIT_STEADY + NST>();
+        else wait_vm_and_lds<WAIT_STEADY>();
+      } else {
+        wait_vm_and_lds<WAIT_STEADY>();
+      }
+      bare_barrier();  // ... and so have everyone else's: the slots of tile h-1 are free
       const char* sa = smem + (h % AST) * A_BYTES + a_wave_off;
       const char* sb = smem + B_REGION + (h % BST) * B_BYTES + b_wave_off;
       // per-step offset of the B fragments: a swizzled chunk of the row, or 32 rows of k
@@ -581,9 +616,9 @@ struct GemmTile {
       }
     };
 
-    if (n_tiles > 0) {
-      // Prologue: A tiles 0 .. AST-2 and B tiles 0 .. BST-2, oldest first (tile 0 is what the first
-      // wait below is about).  A short tile 0 goes through registers instead.
+    // Prologue: A tiles 0 .. AST-2 and B tiles 0 .. BST-2, oldest first (tile 0 is what the first
+    // wait of the loop is about).  A short tile 0 goes through registers instead.
+    auto issue_prologue = [&]() {
       if (k_tail) fill_short_tile(k_tail);
 #pragma unroll
       for (int s = 0; s < (loader ? AST - 1 : 0); ++s) {
@@ -596,6 +631,8 @@ struct GemmTile {
           for (int i = 0; i < LB; ++i) load_b(i, s);
         }
       }
+    };
+    auto k_loop_and_drain = [&]() {
       using W16 = std::integral_constant<int, 16>;
       using W8 = std::integral_constant<int, 8>;
       using W4 = std::integral_constant<int, 4>;
@@ -608,22 +645,20 @@ struct GemmTile {
       // two straight-line versions of the loop, with and without the loads: a branch around every load
       // would cut each row of MFMAs into several scheduling regions
       // (and the side job one version per unit width: the unit's elements are dealt to rows at compile time)
+      auto tiles = [&](auto ld_tag, auto w_tag) {
+        for (int h = 0; h < n_tiles; ++h) tile_body(h, ld_tag, w_tag);
+      };
       if constexpr (SIDE) {
-        if (!loader) {
-          for (int h = 0; h < n_tiles; ++h) tile_body(h, std::false_type{}, W16{});
-        } else if (p.side_width == 16) {
-          for (int h = 0; h < n_tiles; ++h) tile_body(h, std::true_type{}, W16{});
-        } else if (p.side_width == 8) {
-          for (int h = 0; h < n_tiles; ++h) tile_body(h, std::true_type{}, W8{});
-        } else {
-          for (int h = 0; h < n_tiles; ++h) tile_body(h, std::true_type{}, W4{});
-        }
+        if (!loader) tiles(std::false_type{}, W16{});
+        else if (p.side_width == 16) tiles(std::true_type{}, W16{});
+        else if (p.side_width == 8) tiles(std::true_type{}, W8{});
+        else tiles(std::true_type{}, W4{});
       } else if constexpr (LDW == NW) {
-        for (int h = 0; h < n_tiles; ++h) tile_body(h, std::true_type{}, W16{});
+        tiles(std::true_type{}, W16{});
       } else if (loader) {
-        for (int h = 0; h < n_tiles; ++h) tile_body(h, std::true_type{}, W16{});
+        tiles(std::true_type{}, W16{});
       } else {
-        for (int h = 0; h < n_tiles; ++h) tile_body(h, std::false_type{}, W16{});
+        tiles(std::false_type{}, W16{});
       }
       wait_vm_and_lds<0>();  // the empty fills of the last iterations must be gone before LDS is reused
       // Drain: the second half of the last tile is in set 1.
@@ -635,6 +670,10 @@ struct GemmTile {
       for (int i = 0; i < FM; ++i)
 #pragma unroll
         for (int j = 0; j < FN; ++j) acc[i][j] = Traits::mfma(fb1[j], fa1[i], acc[i][j]);
+    };
+    if (n_tiles > 0) {
+      issue_prologue();
+      if constexpr (!LOOP) k_loop_and_drain();
     }
 
     // ---- per-row statistics of the tile (LayerNorm epilogues) -------------------------------
@@ -838,6 +877,77 @@ struct GemmTile {
           T* y = (T*)p.side_y;
           y[done + tid] = silu_16<T>(x[done + tid]);
         }
+      }
+    } else if constexpr (LOOP) {
+      // Walk the tiles id, id + grid, ...  After the K loop of one tile every LDS slot is dead: the
+      // first operand tiles of the next one go into the slots they belong to (A 0 .. AST-2, B 0 ..
+      // BST-2) right away, and the output is staged in the two slots that stay free, in as many
+      // passes as that takes.  The stores leave through a buffer descriptor (rows and columns that
+      // do not exist get an offset outside it and are dropped), so every wavefront issues exactly
+      // NST of them per tile and the first wait of the next K loop can count them.
+      static_assert(!B_KMAJOR && AST >= 3 && BST >= 2 && NW % 2 == 0, "looping store kernel");
+      constexpr int RB = TN * 2;
+      constexpr int FREE = A_BYTES < B_BYTES ? A_BYTES : B_BYTES;  // bytes of a free slot half the wavefronts share
+      constexpr int PASSES = (NW / 2) * TM * RB <= FREE ? 1
+                           : (FM % 2 == 0 && (NW / 2) * (TM / 2) * RB <= FREE) ? 2
+                           : (FM % 4 == 0 && (NW / 2) * (TM / 4) * RB <= FREE) ? 4 : FM;
+      constexpr int FMH = FM / PASSES;
+      static_assert(FM % PASSES == 0 && (NW / 2) * FMH * 16 * RB <= FREE, "staging area");
+      static_assert(RB == 64 || RB == 128 || RB == 256, "row of a wavefront's sub-tile");
+      constexpr int LPR = TN / 8, RPI = 64 / LPR;
+      auto chunk_xor = [](int r) { return RB == 64 ? (r >> 1) & 3 : r & 7; };
+      T* C = (T*)p.C;
+      const int total = p.tiles_m * p.tiles_n;
+      int id = blockIdx.x;
+      for (;;) {
+        k_loop_and_drain();
+        __syncthreads();  // every wavefront is done with the last K tile, and no fill is still landing
+        // The epilogue's lane constants are recomputed per tile from a value the compiler cannot see
+        // through: hoisted out of this loop they would stay live across the K loop, which has no
+        // register to spare.
+        int ol = lane;
+        asm volatile("" : "+v"(ol));
+        char* stage = (wave < NW / 2 ? smem + (AST - 1) * A_BYTES + wave * (FMH * 16 * RB)
+                                     : smem + B_REGION + (BST - 1) * B_BYTES + (wave - NW / 2) * (FMH * 16 * RB));
+        const int srow = ol / LPR, schunk = ol % LPR;
+        const int wr = ol & 15, wg = ol >> 4;
+        const int w_off = wr * RB + (((wg & 1) ^ (wr >> 3)) << 3);
+        const int s_row0 = row0, s_col0 = col0, s_rows = rows_a, s_cols = rows_b;
+        id += gridDim.x;
+        const bool more = id < total;  // uniform
+        if (more) {
+          set_tile(id);
+          issue_prologue();
+        }
+        const __amdgpu_buffer_rsrc_t rsrc_c =
+            make_rsrc(C + ((size_t)s_row0 * N + s_col0), ((unsigned)(s_rows - 1) * N + s_cols) * 2u);
+#pragma unroll
+        for (int ps = 0; ps < PASSES; ++ps) {
+#pragma unroll
+          for (int i = 0; i < FMH; ++i) {
+#pragma unroll
+            for (int j = 0; j < FN; ++j) {
+              vec4 v;
+#pragma unroll
+              for (int e = 0; e < 4; ++e) v[e] = (T)acc[ps * FMH + i][j][e];
+              *(vec4*)(stage + i * 16 * RB + w_off + (((2 * j + (wg >> 1)) ^ chunk_xor(wr)) << 4)) = v;
+            }
+          }
+#pragma unroll
+          for (int it = 0; it < FMH * 16 / RPI; ++it) {
+            const int r = it * RPI + srow;
+            vec8 v = *(const vec8*)(stage + r * RB + schunk * 16);
+            if ((r >> 3) & 1) v = vec8{v[4], v[5], v[6], v[7], v[0], v[1], v[2], v[3]};
+            const int tr = wm * TM + ps * FMH * 16 + r;                    // row inside the tile
+            const int tcn = wn * TN + (schunk ^ chunk_xor(r)) * 8;          // column inside the tile
+            const unsigned off = (tr < s_rows && tcn < s_cols) ? ((unsigned)tr * (unsigned)N + (unsigned)tcn) * 2u : kOobOffset;
+            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(i32x4, v), rsrc_c, (int)off, 0, 0);
+          }
+        }
+        if (!more) break;
+        stores_pending = true;
+        zero_acc();
+        zero_fragments();
       }
     } else if (EPI == kEpiLnFused) {
       // gamma / beta for this lane's columns: issued now, consumed in step 5

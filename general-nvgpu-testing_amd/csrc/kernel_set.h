@@ -38,6 +38,16 @@ hipError_t launch_gemm(const GemmParams& p, dim3 grid, hipStream_t stream) {
   return hipGetLastError();
 }
 
+// The looping store kernel exists for the large 8-wavefront tiles, the ones problems of several
+// rounds of workgroups run with (3 A + 2 B slots only).
+template <typename T, int BM, int BN, int WVM, int WVN>
+GemmLauncher loop_launcher() {
+  if constexpr (WVM * WVN == 8 && BM >= 192 && BN == 256 && BN / WVN == 64)
+    return launch_gemm<T, BM, BN, WVM, WVN, kEpiStoreLoop, 3, 2>;
+  else
+    return nullptr;
+}
+
 template <int BM, int BN, int TM, int TN>
 KernelSet make_kernel_set() {
   constexpr int WVM = BM / TM, WVN = BN / TN;
@@ -68,7 +78,10 @@ KernelSet make_kernel_set() {
   k.launch[D][kEpiStoreSide][1] = launch_gemm<T, BM, BN, WVM, WVN, kEpiStoreSide, 2, 2>; \
   k.launch[D][kEpiStoreSide][2] = nullptr; \
   k.launch_kmajor[D][0] = launch_gemm<T, BM, BN, WVM, WVN, kEpiStore, 3, 2, true>; \
-  k.launch_kmajor[D][1] = launch_gemm<T, BM, BN, WVM, WVN, kEpiStore, 2, 2, true>;
+  k.launch_kmajor[D][1] = launch_gemm<T, BM, BN, WVM, WVN, kEpiStore, 2, 2, true>; \
+  k.launch[D][kEpiStoreLoop][0] = loop_launcher<T, BM, BN, WVM, WVN>();              \
+  k.launch[D][kEpiStoreLoop][1] = nullptr;                                            \
+  k.launch[D][kEpiStoreLoop][2] = nullptr;
   BEAM_FILL(0, _Float16)
   BEAM_FILL(1, __bf16)
 #undef BEAM_FILL

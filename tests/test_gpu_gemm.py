@@ -165,6 +165,24 @@ def test_fp16_sweep(gpu, beamc, oracle, shape):
     assert_close(oracle, got, ref, K, F16, f"{shape}")
 
 
+@pytest.mark.parametrize("shape", [(4200, 4296, 128), (8192, 8200, 64), (2600, 9000, 192), (4096, 4104, 256)])
+def test_more_tiles_than_compute_units(gpu, beamc, oracle, shape):
+    """More tiles than CUs: with 3 A + 2 B slots the large tiles run as one workgroup per CU that walks
+    its tiles and prefetches the next one's operands during the store.  Ragged M and N (rows and
+    columns dropped by the store's buffer descriptor), against the oracle and, bit for bit, against the
+    same tile with 2 + 2 slots, which runs one workgroup per tile."""
+    M, N, K = shape
+    for dtype in (F16, BF16):
+        a = beamc.host_uniform((M, K), dtype, 12, 0)
+        b = beamc.host_uniform((N, K), dtype, 12, 1)
+        ref = oracle.gemmrc(a, b, dtype)
+        for tile in ((256, 256, 128, 64), (224, 256, 112, 64), (192, 256, 96, 64)):
+            walk = run_gemm(beamc, a, b, dtype, beamc.TileConfig(*tile, 0, 0))
+            once = run_gemm(beamc, a, b, dtype, beamc.TileConfig(*tile, 1, 0))
+            assert_close(oracle, walk, ref, K, dtype, f"{shape} {tile}")
+            assert (walk == once).all(), (shape, tile)
+
+
 def _decode(bits, dtype):
     if dtype == F16:
         return bits.view(np.float16).astype(np.float64)
