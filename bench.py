@@ -28,7 +28,7 @@ HBM_PEAK_GBS = 8000.0
 # HBM/fabric bytes per launch of the headline kernel, from the counter runs summarised in
 # profiles/gemmrc_256x256_fp16_8192cube.txt (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000, the factors of
 # profiles/copy_256MiB_counter_calibration.txt).  Counters cannot be read from inside this script.
-PROFILED_TRAFFIC_BYTES = 1.745e9
+PROFILED_TRAFFIC_BYTES = 1.749e9
 
 
 def time_region(_C, fn, steps):
