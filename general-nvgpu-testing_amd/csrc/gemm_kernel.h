@@ -119,6 +119,7 @@ struct GemmParams {
   long long side_count;  // elements
   int side_iters;        // K tiles' worth of units per workgroup
   int side_width;        // bytes per unit
+  int c_streaming;       // kEpiStoreLoop: store C non-temporal
 };
 
 // Buffer descriptor word 3 for gfx9-family raw buffers: 32-bit data format, no swizzle.
@@ -921,6 +922,11 @@ struct GemmTile {
         }
         const __amdgpu_buffer_rsrc_t rsrc_c =
             make_rsrc(C + ((size_t)s_row0 * N + s_col0), ((unsigned)(s_rows - 1) * N + s_cols) * 2u);
+        // Non-temporal stores when the host asks for them (an output larger than the last-level cache:
+        // its lines then do not push operand panels out of the L2).  Two copies of the loop, not a
+        // branch per store: the reads of a pass stay batched ahead of its stores.
+        auto store_tile = [&](auto aux_tag) {
+        constexpr int AUX = decltype(aux_tag)::value;
 #pragma unroll
         for (int ps = 0; ps < PASSES; ++ps) {
 #pragma unroll
@@ -941,9 +947,12 @@ struct GemmTile {
             const int tr = wm * TM + ps * FMH * 16 + r;                    // row inside the tile
             const int tcn = wn * TN + (schunk ^ chunk_xor(r)) * 8;          // column inside the tile
             const unsigned off = (tr < s_rows && tcn < s_cols) ? ((unsigned)tr * (unsigned)N + (unsigned)tcn) * 2u : kOobOffset;
-            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(i32x4, v), rsrc_c, (int)off, 0, 0);
+            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(i32x4, v), rsrc_c, (int)off, 0, AUX);
           }
         }
+        };
+        if (p.c_streaming) store_tile(std::integral_constant<int, 2>{});
+        else store_tile(std::integral_constant<int, 0>{});
         if (!more) break;
         stores_pending = true;
         zero_acc();
