@@ -273,7 +273,7 @@ struct GemmTile {
     const __amdgpu_buffer_rsrc_t rsrc_b = make_rsrc(b_base, bytes_b);
     // kEpiStoreLoop: the same for the next tile of this workgroup (neither split-K nor the [K][N]
     // layout nor a short K tile exist in that mode: the host sees to it)
-    auto set_tile = [&](int id) {
+    auto set_tile = [&](int id) __attribute__((always_inline)) {
       tc = tile_of_workgroup(id, p.tiles_m, p.tiles_n, p.group_m);
       row0 = tc.tm * BM;
       col0 = tc.tn * BN;
@@ -309,13 +309,13 @@ struct GemmTile {
     // One buffer load (1 KiB per wavefront) of A tile t / B tile t into its slot.  Tiles past the end
     // of the K range get an empty descriptor: the load is still issued and counted (the pipeline below
     // has no special cases for its last iterations) but touches no memory.
-    auto load_a = [&](int i, int t) {
+    auto load_a = [&](int i, int t) __attribute__((always_inline)) {
       char* dst = smem + (t % AST) * A_BYTES + wave * 1024 + i * (NTL * 16);
       const __amdgpu_buffer_rsrc_t r = make_rsrc(a_base, t < n_tiles ? bytes_a : 0u);
       __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (__attribute__((address_space(3))) void*)dst, 16,
                                                (int)voff_a[i], tile_koff(t) * 2, 0, 0);
     };
-    auto load_b = [&](int i, int t) {
+    auto load_b = [&](int i, int t) __attribute__((always_inline)) {
       char* dst = smem + B_REGION + (t % BST) * B_BYTES + wave * 1024 + i * (NTL * 16);
       if (B_KMAJOR) {
         // Rows koff .. koff + kBK of the slice, as many as exist: rows past the end of K and the
@@ -337,7 +337,7 @@ struct GemmTile {
     // The short tile goes through registers so that chunks at or past `kvalid` are zero-filled.
     // (A K-major B needs none of this: its rows past the end of K are out of range by themselves.)
     const bool loader = LDW == NW || wave < LDW;
-    auto fill_short_tile = [&](int kvalid) {
+    auto fill_short_tile = [&](int kvalid) __attribute__((always_inline)) {
       if (!loader) return;
       const int koff = tile_koff(0);
       i32x4 ra[LA], rb[LB];
@@ -388,7 +388,7 @@ struct GemmTile {
     // LDS read it can see behind all outstanding global->LDS fills (vmcnt(0)), which would
     // serialise the pipeline.  Results of inline assembly are not tracked by the compiler's
     // wait-count insertion, so the step below waits for them explicitly.
-    auto read_b_fragment = [&](const char* sb, int j) -> vec8 {
+    auto read_b_fragment = [&](const char* sb, int j) __attribute__((always_inline)) -> vec8 {
       if constexpr (B_KMAJOR) {
         const unsigned addr = (unsigned)(size_t)(__attribute__((address_space(3))) const char*)(sb + bfrag_off[j]);
         vec4 lo, hi;
@@ -401,7 +401,7 @@ struct GemmTile {
     };
 
     f32x4 acc[FM][FN];
-    auto zero_acc = [&]() {
+    auto zero_acc = [&]() __attribute__((always_inline)) {
 #pragma unroll
       for (int i = 0; i < FM; ++i)
 #pragma unroll
@@ -415,7 +415,7 @@ struct GemmTile {
     // of one step consume one set, the LDS reads of the next step fill the other.  They start as
     // zeros so that the very first step of the pipeline multiplies nothing.
     vec8 fa0[FM], fa1[FM], fb0[FN], fb1[FN];
-    auto zero_fragments = [&]() {
+    auto zero_fragments = [&]() __attribute__((always_inline)) {
 #pragma unroll
       for (int i = 0; i < FM; ++i)
 #pragma unroll
@@ -458,10 +458,10 @@ struct GemmTile {
     // (auxiliary bit 1), so that lines written once do not push the GEMM's operands out of the L2:
     // 900 -> 866 us for 8192^3 carrying 256 Mi elements.  A small array (4-byte units) is better
     // left in the cache, for whoever reads y next.
-    auto side_offset = [&](int it, int s, int W) {  // thread tid of the loaders owns units tid + s * NTL of a tile
+    auto side_offset = [&](int it, int s, int W) __attribute__((always_inline)) {  // thread tid of the loaders owns units tid + s * NTL of a tile
       return (it >= 0 && it < p.side_iters) ? (side_v0 + (unsigned)it * NT + (unsigned)s * NTL) * (unsigned)W : kOobOffset;
     };
-    auto side_load = [&](int it, auto w_tag) {
+    auto side_load = [&](int it, auto w_tag) __attribute__((always_inline)) {
       constexpr int W = decltype(w_tag)::value;
       constexpr int AUX = W >= 8 ? 2 : 0;
 #pragma unroll
@@ -480,7 +480,7 @@ struct GemmTile {
         }
       }
     };
-    auto side_store = [&](int it, auto w_tag) {
+    auto side_store = [&](int it, auto w_tag) __attribute__((always_inline)) {
       constexpr int W = decltype(w_tag)::value;
       constexpr int AUX = W >= 8 ? 2 : 0;
 #pragma unroll
@@ -492,7 +492,7 @@ struct GemmTile {
         else __builtin_amdgcn_raw_buffer_store_b32(o[0], rsrc_sy, off, 0, AUX);
       }
     };
-    auto side_pair = [&](int e) {  // pair e of every unit this thread holds
+    auto side_pair = [&](int e) __attribute__((always_inline)) {  // pair e of every unit this thread holds
 #pragma unroll
       for (int s = 0; s < SV; ++s) {
         typedef T pair_t __attribute__((ext_vector_type(2)));
@@ -511,7 +511,7 @@ struct GemmTile {
     // registers across the two sets, and the step then starts by waiting for its own reads.
     //   ROW0: index of the step's first row inside the tile (the loads are dealt out row by row).
     auto step = [&](const char* sa, const char* sb, vec8(&fa_cur)[FM], vec8(&fa_nxt)[FM], vec8(&fb_cur)[FN],
-                    vec8(&fb_nxt)[FN], int h, auto row0_tag, auto ld_tag, auto w_tag) {
+                    vec8(&fb_nxt)[FN], int h, auto row0_tag, auto ld_tag, auto w_tag) __attribute__((always_inline)) {
       constexpr int ROW0 = decltype(row0_tag)::value;
       constexpr bool LD = decltype(ld_tag)::value;
       constexpr int SIDE_PAIRS = decltype(w_tag)::value / 4;  // pairs of elements per side unit
@@ -592,7 +592,7 @@ struct GemmTile {
     // second half of tile h-1 (set 1) while reading the first half of tile h into set 0; step 1
     // multiplies set 0 while reading the second half of tile h into set 1.
     bool stores_pending = false;  // kEpiStoreLoop: a store epilogue precedes the tile being started
-    auto tile_body = [&](int h, auto ld_tag, auto w_tag) {
+    auto tile_body = [&](int h, auto ld_tag, auto w_tag) __attribute__((always_inline)) {
       // my fills of tile h have landed; my reads of tile h-1 are done
       if constexpr (!decltype(ld_tag)::value) {
         wait_lds<0>();  // a wavefront that loads nothing has no fills to wait for
@@ -619,7 +619,7 @@ struct GemmTile {
 
     // Prologue: A tiles 0 .. AST-2 and B tiles 0 .. BST-2, oldest first (tile 0 is what the first
     // wait of the loop is about).  A short tile 0 goes through registers instead.
-    auto issue_prologue = [&]() {
+    auto issue_prologue = [&]() __attribute__((always_inline)) {
       if (k_tail) fill_short_tile(k_tail);
 #pragma unroll
       for (int s = 0; s < (loader ? AST - 1 : 0); ++s) {
@@ -633,33 +633,29 @@ struct GemmTile {
         }
       }
     };
-    auto k_loop_and_drain = [&]() {
-      using W16 = std::integral_constant<int, 16>;
-      using W8 = std::integral_constant<int, 8>;
-      using W4 = std::integral_constant<int, 4>;
-      if (SIDE && loader) {
-        side_store(-1, W4{});  // dropped; keeps the number of side operations per tile uniform
-        if (p.side_width == 16) side_load(0, W16{});
-        else if (p.side_width == 8) side_load(0, W8{});
-        else side_load(0, W4{});
-      }
+    using W16 = std::integral_constant<int, 16>;
+    using W8 = std::integral_constant<int, 8>;
+    using W4 = std::integral_constant<int, 4>;
+    auto k_loop_and_drain = [&]() __attribute__((always_inline)) {
       // two straight-line versions of the loop, with and without the loads: a branch around every load
       // would cut each row of MFMAs into several scheduling regions
       // (and the side job one version per unit width: the unit's elements are dealt to rows at compile time)
-      auto tiles = [&](auto ld_tag, auto w_tag) {
-        for (int h = 0; h < n_tiles; ++h) tile_body(h, ld_tag, w_tag);
-      };
       if constexpr (SIDE) {
-        if (!loader) tiles(std::false_type{}, W16{});
-        else if (p.side_width == 16) tiles(std::true_type{}, W16{});
-        else if (p.side_width == 8) tiles(std::true_type{}, W8{});
-        else tiles(std::true_type{}, W4{});
+        if (!loader) {
+          for (int h = 0; h < n_tiles; ++h) tile_body(h, std::false_type{}, W16{});
+        } else if (p.side_width == 16) {
+          for (int h = 0; h < n_tiles; ++h) tile_body(h, std::true_type{}, W16{});
+        } else if (p.side_width == 8) {
+          for (int h = 0; h < n_tiles; ++h) tile_body(h, std::true_type{}, W8{});
+        } else {
+          for (int h = 0; h < n_tiles; ++h) tile_body(h, std::true_type{}, W4{});
+        }
       } else if constexpr (LDW == NW) {
-        tiles(std::true_type{}, W16{});
+        for (int h = 0; h < n_tiles; ++h) tile_body(h, std::true_type{}, W16{});
       } else if (loader) {
-        tiles(std::true_type{}, W16{});
+        for (int h = 0; h < n_tiles; ++h) tile_body(h, std::true_type{}, W16{});
       } else {
-        tiles(std::false_type{}, W16{});
+        for (int h = 0; h < n_tiles; ++h) tile_body(h, std::false_type{}, W16{});
       }
       wait_vm_and_lds<0>();  // the empty fills of the last iterations must be gone before LDS is reused
       // Drain: the second half of the last tile is in set 1.
@@ -674,6 +670,12 @@ struct GemmTile {
     };
     if (n_tiles > 0) {
       issue_prologue();
+      if (SIDE && loader) {
+        side_store(-1, W4{});  // dropped; keeps the number of side operations per tile uniform
+        if (p.side_width == 16) side_load(0, W16{});
+        else if (p.side_width == 8) side_load(0, W8{});
+        else side_load(0, W4{});
+      }
       if constexpr (!LOOP) k_loop_and_drain();
     }
 
@@ -925,7 +927,7 @@ struct GemmTile {
         // Non-temporal stores when the host asks for them (an output larger than the last-level cache:
         // its lines then do not push operand panels out of the L2).  Two copies of the loop, not a
         // branch per store: the reads of a pass stay batched ahead of its stores.
-        auto store_tile = [&](auto aux_tag) {
+        auto store_tile = [&](auto aux_tag) __attribute__((always_inline)) {
         constexpr int AUX = decltype(aux_tag)::value;
 #pragma unroll
         for (int ps = 0; ps < PASSES; ++ps) {
