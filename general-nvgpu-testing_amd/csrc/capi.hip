@@ -383,13 +383,25 @@ int beam_gemmrc(const void* A, const void* B, void* C, int M, int N, int K, int 
   if ((rc = resolve_cfg(cfg, M, N, K, &c, &ks))) return rc;
   GemmParams p = base_params(A, B, M, N, K, c);
   p.C = C;
-  // More than one round of workgroups of a large tile: one workgroup per CU walks the tiles and
+  const long tiles = (long)p.tiles_m * p.tiles_n;
+  const int cus = g_dev.cus > 0 ? g_dev.cus : 256;
+  // The 256 x 256 tile of four 128 x 128 wavefronts has a kernel of its own (gemm_w4.h), built for problems
+  // of a round of workgroups or more: one workgroup per CU walks its tiles with the operand ring running
+  // through the tile boundaries.  It is what the tile {256, 256, 128, 128} means wherever its preconditions
+  // hold, and what a call without a tile gets in place of the 8-wavefront 256 x 256 tile from one full
+  // round of workgroups on (8192^3 fp16, same machine, in turn: 1490-1515 against 1455-1465 TFLOP/s).
+  const bool w4_fits = c.pipeline == 0 && K % kBK == 0 && K >= kW4MinK && N % 8 == 0 && ((uintptr_t)C & 15) == 0 && N <= (1 << 21);
+  const bool w4_named = c.block_m == 256 && c.block_n == 256 && c.wave_m == 128 && c.wave_n == 128;
+  const bool w4_default = !cfg && c.block_m == 256 && c.block_n == 256 && tiles >= cus;
+  if (w4_fits && (w4_named || w4_default)) {
+    BEAM_HIP(launch_gemm_w4(p, dtype, dim3((unsigned)(tiles < cus ? tiles : cus), 1, 1), st));
+    return BEAM_OK;
+  }
+  // More than one round of workgroups of another large tile: one workgroup per CU walks the tiles and
   // loads the next one's first operand tiles while it stores the current one (kEpiStoreLoop).
   // That kernel stores 16 bytes per lane through a buffer descriptor and has no short K tile.
   // Against one workgroup per tile, same machine: 16384 x 16384 x 2048 822 against 841 us,
   // 8192 x 8192 x 512 71 against 74.5 us, 8192 x 8192 x 2048 205 against 207 us, 8192^3 no difference.
-  const long tiles = (long)p.tiles_m * p.tiles_n;
-  const int cus = g_dev.cus > 0 ? g_dev.cus : 256;
   GemmLauncher loop = c.pipeline == 0 ? ks->launch[dtype][kEpiStoreLoop][0] : nullptr;
   if (loop && tiles > cus && K % kBK == 0 && N % 8 == 0 && ((uintptr_t)C & 15) == 0 && N <= (1 << 21)) {
     // Non-temporal stores of C pay when C is larger than the 256 MB last-level cache (and the K loops

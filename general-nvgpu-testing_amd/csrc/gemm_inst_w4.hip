@@ -1,0 +1,25 @@
+// The 256x256 tile of four 128x128 wavefronts (gemm_w4.h), fp16 and bf16.
+#include "gemm_w4.h"
+#include "kernel_set.h"
+
+namespace beam {
+
+template <typename T>
+static hipError_t launch_w4_t(const GemmParams& p, dim3 grid, hipStream_t stream) {
+  auto kern = gemmrc_w4_kernel<T>;
+  static bool configured = false;  // benign race: the attribute call is idempotent
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       GemmW4<T>::LDS_BYTES);
+    if (e != hipSuccess) return e;
+    configured = true;
+  }
+  hipLaunchKernelGGL(kern, grid, dim3(GemmW4<T>::NT), GemmW4<T>::LDS_BYTES, stream, p);
+  return hipGetLastError();
+}
+
+hipError_t launch_gemm_w4(const GemmParams& p, int dtype, dim3 grid, hipStream_t stream) {
+  return dtype == BEAM_BF16 ? launch_w4_t<__bf16>(p, grid, stream) : launch_w4_t<_Float16>(p, grid, stream);
+}
+
+}  // namespace beam

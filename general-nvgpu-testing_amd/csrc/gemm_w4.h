@@ -1,0 +1,434 @@
+// Large-problem gemmrc kernel for gfx950: 256 x 256 workgroup tile, four wavefronts of 128 x 128,
+// one wavefront per SIMD, accumulators in the 256 accumulation registers, one workgroup per CU
+// walking its output tiles with the operand ring running straight through the tile boundaries.
+//
+// Same operation and layouts as gemm_kernel.h (C = A . B^T, fp32 accumulation, 16-bit output;
+// reference: cuda/cute_kernels/cute_gemm_128x256.cu:17-194, its software-pipelined K loop
+// :141-167).  What differs from the 8-wavefront tiles and why:
+//
+//   * a 128 x 128 wavefront tile needs 16 LDS fragment reads per 64 MFMAs instead of 12 per 32: a
+//     third fewer LDS bytes per flop, and this part is power limited on real data;
+//   * a wavefront alone on its SIMD issues in order, so what it issues between two MFMAs decides
+//     whether the matrix core idles.  Measured on this machine with a lone wavefront per SIMD
+//     (64 independent v_mfma_f32_16x16x32_f16 per loop pass = 1024 matrix-core cycles): nothing
+//     else 1045 cycles per pass; one ds_read_b128 after every 4th MFMA 1057; the same 16 reads
+//     in groups of four 1120, all at the head 1129; 8 LDS-direct buffer loads, one after every 8th
+//     MFMA, +4; a workgroup barrier per pass +16.  Hence the rule of the loop below: at most ONE
+//     memory instruction between two MFMAs, never two in a row;
+//   * the MFMAs are inline assembly with the accumulator tied to an accumulation register.  Left to
+//     the compiler, 64 live accumulator blocks (all 256 registers) make it rotate blocks through
+//     spare registers with v_accvgpr_mov/read/write and wait states inside the loop;
+//   * the ring of LDS operand slots (3 for A, 2 for B) never drains: while the last K tiles of one
+//     output tile are multiplied, the first K tiles of the workgroup's next output tile are already
+//     being fetched, and the finished accumulators are converted and stored row block by row block
+//     in the gaps of the next tile's first K tile (whose first MFMAs start from a zero addend
+//     instead of from cleared registers).  No LDS staging, no extra barrier, no pipeline refill;
+//   * the B fragment of MFMA block b takes rows 32*(b/2) + 8*(r/4) + 4*(b%2) + r%4 (r = lane % 16)
+//     of the wavefront's B rows instead of 16*b + r: a lane then holds 8 consecutive output
+//     columns per pair of blocks and stores them as one 16-byte access (64 contiguous bytes per
+//     output row and instruction).  The B slots use a swizzle made for that row pattern.
+//
+// Preconditions (the host checks them; anything else takes the kernels of gemm_kernel.h):
+// K a multiple of 64 and at least 192, N a multiple of 8, C 16-byte aligned, grid <= number of tiles.
+#pragma once
+
+#include "gemm_kernel.h"
+
+namespace beam {
+
+// The 64 accumulator blocks of a wavefront live in the accumulation registers a0 .. a255 (block n in
+// a[4n : 4n+3]) and are named only inside inline assembly: the compiler never allocates, copies or
+// spills them.  (Handed 64 live four-register values that fill the whole file, its allocator starts
+// rotating blocks through spare registers and scratch memory.)  The compiler is told once, by a clobber
+// list, that these registers are in use; it has no reason to touch them itself as long as the rest of
+// the kernel fits the 256 ordinary registers.
+template <typename T>
+struct W4Mfma;
+
+template <>
+struct W4Mfma<_Float16> {
+  // block BLK += b x a (b supplies the output columns, a the output rows)
+  template <int BLK>
+  static __device__ __forceinline__ void fma(f16x8 b, f16x8 a) {
+    asm volatile("v_mfma_f32_16x16x32_f16 a[%2:%3], %0, %1, a[%2:%3]" ::"v"(b), "v"(a), "n"(4 * BLK), "n"(4 * BLK + 3));
+  }
+  // block BLK = b x a: the first K step of an output tile
+  template <int BLK>
+  static __device__ __forceinline__ void first(f16x8 b, f16x8 a) {
+    asm volatile("v_mfma_f32_16x16x32_f16 a[%2:%3], %0, %1, 0" ::"v"(b), "v"(a), "n"(4 * BLK), "n"(4 * BLK + 3));
+  }
+};
+
+template <>
+struct W4Mfma<__bf16> {
+  template <int BLK>
+  static __device__ __forceinline__ void fma(bf16x8 b, bf16x8 a) {
+    asm volatile("v_mfma_f32_16x16x32_bf16 a[%2:%3], %0, %1, a[%2:%3]" ::"v"(b), "v"(a), "n"(4 * BLK), "n"(4 * BLK + 3));
+  }
+  template <int BLK>
+  static __device__ __forceinline__ void first(bf16x8 b, bf16x8 a) {
+    asm volatile("v_mfma_f32_16x16x32_bf16 a[%2:%3], %0, %1, 0" ::"v"(b), "v"(a), "n"(4 * BLK), "n"(4 * BLK + 3));
+  }
+};
+
+// Element REG of the accumulation registers.  The caller keeps matrix-core results at least three MFMAs
+// (48 cycles) old before reading them: the compiler cannot insert the wait states it does not know about.
+template <int REG>
+__device__ __forceinline__ float w4_acc_read() {
+  float x;
+  asm volatile("v_accvgpr_read_b32 %0, a[%1:%1]" : "=v"(x) : "n"(REG));
+  return x;
+}
+
+__device__ __forceinline__ void w4_claim_acc_registers() {
+  asm volatile("" ::: "a0", "a1", "a2", "a3", "a4", "a5", "a6", "a7", "a8", "a9", "a10", "a11", "a12", "a13", "a14", "a15",
+               "a16", "a17", "a18", "a19", "a20", "a21", "a22", "a23", "a24", "a25", "a26", "a27", "a28", "a29", "a30", "a31",
+               "a32", "a33", "a34", "a35", "a36", "a37", "a38", "a39", "a40", "a41", "a42", "a43", "a44", "a45", "a46", "a47",
+               "a48", "a49", "a50", "a51", "a52", "a53", "a54", "a55", "a56", "a57", "a58", "a59", "a60", "a61", "a62", "a63",
+               "a64", "a65", "a66", "a67", "a68", "a69", "a70", "a71", "a72", "a73", "a74", "a75", "a76", "a77", "a78", "a79",
+               "a80", "a81", "a82", "a83", "a84", "a85", "a86", "a87", "a88", "a89", "a90", "a91", "a92", "a93", "a94", "a95",
+               "a96", "a97", "a98", "a99", "a100", "a101", "a102", "a103", "a104", "a105", "a106", "a107", "a108", "a109",
+               "a110", "a111", "a112", "a113", "a114", "a115", "a116", "a117", "a118", "a119", "a120", "a121", "a122", "a123",
+               "a124", "a125", "a126", "a127", "a128", "a129", "a130", "a131", "a132", "a133", "a134", "a135", "a136", "a137",
+               "a138", "a139", "a140", "a141", "a142", "a143", "a144", "a145", "a146", "a147", "a148", "a149", "a150", "a151",
+               "a152", "a153", "a154", "a155", "a156", "a157", "a158", "a159", "a160", "a161", "a162", "a163", "a164", "a165",
+               "a166", "a167", "a168", "a169", "a170", "a171", "a172", "a173", "a174", "a175", "a176", "a177", "a178", "a179",
+               "a180", "a181", "a182", "a183", "a184", "a185", "a186", "a187", "a188", "a189", "a190", "a191", "a192", "a193",
+               "a194", "a195", "a196", "a197", "a198", "a199", "a200", "a201", "a202", "a203", "a204", "a205", "a206", "a207",
+               "a208", "a209", "a210", "a211", "a212", "a213", "a214", "a215", "a216", "a217", "a218", "a219", "a220", "a221",
+               "a222", "a223", "a224", "a225", "a226", "a227", "a228", "a229", "a230", "a231", "a232", "a233", "a234", "a235",
+               "a236", "a237", "a238", "a239", "a240", "a241", "a242", "a243", "a244", "a245", "a246", "a247", "a248", "a249",
+               "a250", "a251", "a252", "a253", "a254", "a255");
+}
+
+// f(std::integral_constant<int, 0>{}), ..., f(std::integral_constant<int, N - 1>{}): a loop whose index is a
+// constant expression in the body (register numbers inside assembly text have to be).
+template <int I, int N, typename F>
+__device__ __forceinline__ void w4_static_for(F&& f) {
+  if constexpr (I < N) {
+    f(std::integral_constant<int, I>{});
+    w4_static_for<I + 1, N>(f);
+  }
+}
+
+// XOR pattern of the 16-byte chunks of a B row in LDS.  A fragment read touches, per 16 lanes, rows
+// base + 8*(r/4) + r%4 (+4 for odd blocks), r = 0..15: bits 1, 3 and 4 of the row number take all
+// 8 combinations and bit 0 selects the half of the 256-byte bank sweep, so 16 distinct 16-byte slots.
+__host__ __device__ inline int w4_swizzle_b(int row) { return (((row >> 3) & 3) << 1) | ((row >> 1) & 1); }
+// First B row (inside the wavefront's 128) of MFMA block b, and the row of lane-row r in it.
+__host__ __device__ inline int w4_b_row(int b, int r) { return 32 * (b >> 1) + 4 * (b & 1) + 8 * (r >> 2) + (r & 3); }
+
+// SB, SA: a wavefront issues its 8 loads of the next B tile in gaps 0, SB, 2 SB, ... of step A and its 8
+// loads of the A tile after next in gaps 0, SA, ... of step B.  The path from the vector-memory unit into
+// LDS moves 64 bytes per cycle and CU, i.e. one 1 KiB load per 64 cycles (4 MFMAs) and wavefront when all
+// four issue: loads issued faster than that stall the wavefront, and with it its MFMAs, at issue.
+template <typename T, int SB = 4, int SA = 8>
+struct GemmW4 {
+  using Traits = ElemTraits<T>;
+  using vec8 = typename Traits::vec8;
+  using Mfma = W4Mfma<T>;
+
+  static constexpr int BM = 256, BN = 256;
+  static constexpr int NW = 4, NT = 256;
+  static constexpr int FM = 8, FN = 8;          // 16 x 16 blocks of a wavefront tile
+  static constexpr int SLOT = 256 * kRowBytes;  // one operand tile of 64 K elements: 32 KiB
+  static constexpr int AST = 3, BST = 2;
+  static constexpr int B_REGION = AST * SLOT;
+  static constexpr int LDS_BYTES = (AST + BST) * SLOT;
+  static constexpr int LPT = SLOT / (NW * 1024);  // buffer loads per wavefront per operand tile (8)
+  static_assert(LDS_BYTES == 160 * 1024 && LPT == 8, "LDS budget");
+  // What goes into gap m (after MFMA m) of a step: load number k, or fragment read number n (B 0..7, then
+  // A 0..7; they take the gaps the loads leave free, in order), or nothing (-1).
+  static constexpr int G0 = 2;  // gaps 0 and 1 of step A: nothing, then the wait and the barrier
+  static constexpr int load_at(int half, int m) {
+    const int s = half == 0 ? SB : SA;
+    return (m >= G0 && (m - G0) % s == 0 && (m - G0) / s < LPT) ? (m - G0) / s : -1;
+  }
+  static constexpr int read_at(int half, int m) {
+    if (m < G0 || load_at(half, m) >= 0) return -1;
+    int n = 0;
+    for (int x = G0; x < m; ++x) n += load_at(half, x) < 0;
+    return n < FN + FM ? n : -1;
+  }
+  static constexpr int LAST_B = G0 + (LPT - 1) * SB, LAST_A = G0 + (LPT - 1) * SA;  // gaps of a step's last load
+  static constexpr int last_read(int half) {
+    int m = 63;
+    while (read_at(half, m) < 0) --m;
+    return m;
+  }
+  static constexpr int LAST_READ = last_read(0) > last_read(1) ? last_read(0) : last_read(1);
+  static_assert(LAST_B + 3 < 64 && LAST_A + 3 < 64 && LAST_READ + 2 < LAST_A, "room for the scalar bookkeeping");
+  static_assert(load_at(0, LAST_B) == LPT - 1 && load_at(1, LAST_A) == LPT - 1 && LAST_B < 62 && LAST_A < 62, "loads fit a step");
+
+  static __device__ __forceinline__ void run(const GemmParams& p, char* smem) {
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave & 1, wn = wave >> 1;
+    const int r = lane & 15, g = lane >> 4;
+    const int M = p.M, N = p.N, K = p.K;
+    const int n_k = K / kBK;
+    const int total_tiles = p.tiles_m * p.tiles_n;
+    const int first_tile = blockIdx.x, tile_step = gridDim.x;
+    const int my_tiles = (total_tiles - first_tile + tile_step - 1) / tile_step;
+    const int g_total = my_tiles * n_k;  // K tiles this workgroup multiplies
+
+    // ---- global -> LDS -----------------------------------------------------------------------
+    // Load i of wavefront w fills bytes [(4 i + w) KiB, + 1 KiB) of a slot = rows 32 i + 8 w .. + 8;
+    // lane l writes position l % 8 of row 32 i + 8 w + l / 8 and fetches the chunk that belongs there.
+    // (Neither swizzle depends on i.)  The row goes into the per-lane offset, the K tile into the scalar
+    // offset: the hardware checks only the former against the descriptor, and that check is what keeps
+    // rows past the end of a matrix from touching memory.
+    const int fill_row = 8 * wave + (lane >> 3);
+    unsigned voff_a[LPT], voff_b[LPT];
+#pragma unroll
+    for (int i = 0; i < LPT; ++i) {
+      const unsigned row_bytes = (unsigned)(fill_row + 32 * i) * (unsigned)K * 2u;
+      voff_a[i] = row_bytes + (unsigned)(((lane & 7) ^ swizzle_of_row(fill_row)) << 4);
+      voff_b[i] = row_bytes + (unsigned)(((lane & 7) ^ w4_swizzle_b(fill_row)) << 4);
+    }
+
+    // Operand rows of the workgroup's j-th output tile as (address, bytes) of a buffer descriptor; empty
+    // past its last tile: such loads are issued and counted like any other and touch no memory.
+    auto tile_coord = [&](int j) { return tile_of_workgroup(first_tile + j * tile_step, p.tiles_m, p.tiles_n, p.group_m); };
+    auto rows_of_a = [&](int j, TileCoord tc) {
+      if (j >= my_tiles) return make_rsrc(p.A, 0u);
+      const int row0 = tc.tm * BM;
+      const int rows = (M - row0) < BM ? (M - row0) : BM;
+      return make_rsrc((const T*)p.A + (size_t)row0 * K, (unsigned)rows * (unsigned)K * 2u);
+    };
+    auto rows_of_b = [&](int j, TileCoord tc) {
+      if (j >= my_tiles) return make_rsrc(p.B, 0u);
+      const int col0 = tc.tn * BN;
+      const int rows = (N - col0) < BN ? (N - col0) : BN;
+      return make_rsrc((const T*)p.B + (size_t)col0 * K, (unsigned)rows * (unsigned)K * 2u);
+    };
+    // A load stream: the operand rows of the output tile it is at (a finished buffer descriptor), the K
+    // tile inside them (byte offset in a row) and the ring slot (byte offset in LDS, plus this wavefront's
+    // KiB) its next loads go to.  The streams run ahead of the multiplication, across the boundaries of
+    // output tiles.  Advancing one is a handful of scalar selects (no branch), dealt out over a few gaps
+    // between MFMAs like everything else.
+    struct Stream {
+      __amdgpu_buffer_rsrc_t rows;
+      int koff;
+      int lds;
+    };
+    const int k_bytes = K * 2;
+    // The LDS address of an LDS-direct load comes from M0.  The compiler's own sequence for the builtin
+    // is "write M0, one wait state, load" in one place; here M0 is written one gap ahead of the load, so
+    // the MFMA between them is the wait state and no gap holds more than one scalar and one memory
+    // instruction.  The loads are therefore invisible to the compiler's wait-count bookkeeping; every wait
+    // for them in this kernel is an explicit s_waitcnt vmcnt.
+    auto set_load_target = [&](const Stream& st, auto i_tag) __attribute__((always_inline)) {
+      asm volatile("s_add_u32 m0, %0, %1" ::"s"(st.lds), "n"(decltype(i_tag)::value * 4096) : "memory");
+    };
+    auto load_tile_part = [&](const Stream& st, unsigned voff) __attribute__((always_inline)) {
+      asm volatile("buffer_load_dwordx4 %0, %1, %2 offen lds" ::"v"(voff), "s"(st.rows), "s"(st.koff) : "memory");
+    };
+    // (in `part`s of two or three scalar instructions, one part per gap; part < 0: all of them)
+    bool wrap_a = false, wrap_b = false;
+    auto advance = [&](Stream& st, bool& wrap, __amdgpu_buffer_rsrc_t next, int ring_begin, int ring_end, int part) __attribute__((always_inline)) {
+      if (part == 0 || part < 0) {
+        const int lds = st.lds + SLOT;
+        st.lds = lds == ring_end + wave * 1024 ? ring_begin + wave * 1024 : lds;
+      }
+      if (part == 1 || part < 0) {
+        const int k = st.koff + kBK * 2;
+        wrap = k == k_bytes;
+        st.koff = wrap ? 0 : k;
+      }
+      if (part == 2 || part < 0) st.rows = wrap ? next : st.rows;
+    };
+
+    // ---- LDS -> fragments ----------------------------------------------------------------------
+    // 16x16x32 operand: lane supplies row r of the block, K elements 8 g .. 8 g + 7 of the 32-wide step.
+    int a_off[2], b_off[2];
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk) {
+      a_off[kk] = lds_offset(wm * 128 + r, 4 * kk + g);
+      const int brow = wn * 128 + w4_b_row(0, r);
+      b_off[kk] = brow * kRowBytes + (((4 * kk + g) ^ w4_swizzle_b(brow)) << 4);
+    }
+
+    w4_claim_acc_registers();  // block (i, b) of the wavefront tile is accumulator block 8 i + b
+    // Fragments, double buffered: set 0 holds the first 32 K elements of a tile, set 1 the second.
+    vec8 fa0[FM], fa1[FM], fb0[FN], fb1[FN];
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        fa0[i][e] = 0;
+        fa1[i][e] = 0;
+        fb0[i][e] = 0;
+        fb1[i][e] = 0;
+      }
+
+    // ---- output --------------------------------------------------------------------------------
+    // acc[i][b][e]: row 128 wm + 16 i + r, column 128 wn + 32 (b / 2) + 8 g + 4 (b % 2) + e of the tile.
+    // A pair of blocks is one 16-byte store per lane through a descriptor of row blocks i .. 7 of the
+    // tile's part of C (per row block, because only the per-lane offset is range checked): rows that do
+    // not exist fall outside it, columns that do not exist get an offset outside it.
+    struct OutTile {
+      char* base;  // first element of the tile in C
+      int bytes;   // from there to the end of the tile's last valid row
+      unsigned voff[FN / 2];
+    };
+    auto out_tile_of = [&](int j, TileCoord tc) {
+      OutTile o;
+      if (j < 0 || j >= my_tiles) {
+        o.base = (char*)p.C;
+        o.bytes = 0;
+#pragma unroll
+        for (int q = 0; q < FN / 2; ++q) o.voff[q] = kOobOffset;
+        return o;
+      }
+      const int row0 = tc.tm * BM, col0 = tc.tn * BN;
+      const int rows = (M - row0) < BM ? (M - row0) : BM;
+      const int cols = (N - col0) < BN ? (N - col0) : BN;
+      o.base = (char*)((T*)p.C + ((size_t)row0 * N + col0));
+      o.bytes = ((rows - 1) * N + cols) * 2;
+#pragma unroll
+      for (int q = 0; q < FN / 2; ++q) {
+        const int col = wn * 128 + 32 * q + 8 * g;
+        o.voff[q] = col < cols ? ((unsigned)(wm * 128 + r) * (unsigned)N + (unsigned)col) * 2u : kOobOffset;
+      }
+      return o;
+    };
+    OutTile out = out_tile_of(-1, TileCoord{0, 0});  // the tile whose accumulators are being stored
+    auto store_pair = [&](auto i_tag, auto q_tag) __attribute__((always_inline)) {
+      constexpr int i = decltype(i_tag)::value, q = decltype(q_tag)::value;
+      constexpr int R0 = 4 * (8 * i + 2 * q);  // first register of block (i, 2 q); block (i, 2 q + 1) follows
+      vec8 v;
+      v[0] = (T)w4_acc_read<R0 + 0>();
+      v[1] = (T)w4_acc_read<R0 + 1>();
+      v[2] = (T)w4_acc_read<R0 + 2>();
+      v[3] = (T)w4_acc_read<R0 + 3>();
+      v[4] = (T)w4_acc_read<R0 + 4>();
+      v[5] = (T)w4_acc_read<R0 + 5>();
+      v[6] = (T)w4_acc_read<R0 + 6>();
+      v[7] = (T)w4_acc_read<R0 + 7>();
+      const int skip = i * 16 * N * 2;  // bytes of the row blocks above this one
+      const int left = out.bytes - skip;
+      const __amdgpu_buffer_rsrc_t rsrc = make_rsrc(out.base + skip, left > 0 ? (unsigned)left : 0u);
+      __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(i32x4, v), rsrc, (int)out.voff[q], 0, 0);
+    };
+
+    // ---- one K tile ------------------------------------------------------------------------------
+    // Step A multiplies the second half of the previous K tile (set 1) while the first half of this
+    // one is read into set 0 and B of the next K tile is fetched; step B multiplies set 0 while the
+    // second half is read into set 1 and A of the K tile after next is fetched.  Every MFMA is
+    // followed by at most one memory instruction and a scheduling fence.
+    // FIRST: this is the first K tile of an output tile.  Step A then completes the previous output
+    // tile row block by row block; each pair of its blocks is converted and stored a little later
+    // (three MFMAs after the row's last one at the earliest: results of the matrix core must not be
+    // read sooner, and the compiler does not see the inline-assembly MFMAs), always before step B
+    // overwrites it.
+    Stream ld_a, ld_b;         // where the next A / B loads go
+    __amdgpu_buffer_rsrc_t next_a, next_b;  // operand rows of the output tile after the one the streams are at
+    int rd_a = 0, rd_b = B_REGION;  // slots (byte offsets) of the K tile being multiplied
+    auto k_tile = [&](auto first_tag) __attribute__((always_inline)) {
+      constexpr bool FIRST = decltype(first_tag)::value;
+      const char* sa = smem + rd_a;
+      const char* sb = smem + rd_b;
+      w4_static_for<0, 128>([&](auto gap_tag) __attribute__((always_inline)) {
+        constexpr int gap = decltype(gap_tag)::value;
+        constexpr int half = gap >> 6, m = gap & 63;
+        // row blocks in turn, the B fragments forwards and backwards alternately: consecutive MFMAs always
+        // share one operand (fewer input toggles; this part is power limited)
+        constexpr int i = m >> 3, b = (i & 1) ? 7 - (m & 7) : (m & 7);
+        constexpr int blk = 8 * i + b;
+        if constexpr (half == 0) Mfma::template fma<blk>(fb1[b], fa1[i]);
+        else if constexpr (FIRST) Mfma::template first<blk>(fb0[b], fa0[i]);
+        else Mfma::template fma<blk>(fb0[b], fa0[i]);
+        // the gap
+        if constexpr (gap == G0 - 1) {
+          // Two MFMAs of the previous K tile are in the matrix core's queue while the wavefronts meet.
+          wait_vm_and_lds<LPT>();  // my fills of this K tile have landed (the youngest 8 are A of the next one)
+          bare_barrier();          // ... everyone's have, and everyone is done reading the slots refilled below
+        }
+        constexpr int ld = load_at(half, m), rd = read_at(half, m);
+        constexpr int ld_next = m + 1 < 64 ? load_at(half, m + 1) : -1;
+        if constexpr (ld_next >= 0) {
+          if constexpr (half == 0) set_load_target(ld_b, std::integral_constant<int, ld_next>{});
+          else set_load_target(ld_a, std::integral_constant<int, ld_next>{});
+        }
+        if constexpr (ld >= 0) {
+          if constexpr (half == 0) load_tile_part(ld_b, voff_b[ld]);
+          else load_tile_part(ld_a, voff_a[ld]);
+        } else if constexpr (rd >= 0 && rd < FN) {
+          const vec8 v = *(const vec8*)(sb + b_off[half] + (rd >> 1) * 4096 + (rd & 1) * 512);
+          if constexpr (half == 0) fb0[rd] = v;
+          else fb1[rd] = v;
+        } else if constexpr (rd >= FN) {
+          const vec8 v = *(const vec8*)(sa + a_off[half] + (rd - FN) * 2048);
+          if constexpr (half == 0) fa0[rd - FN] = v;
+          else fa1[rd - FN] = v;
+        }
+        // scalar bookkeeping, a few instructions per gap: the B stream moves on after its last load, ...
+        if constexpr (half == 0 && m > LAST_B && m <= LAST_B + 3) advance(ld_b, wrap_b, next_b, B_REGION, LDS_BYTES, m - LAST_B - 1);
+        // ... the read slots once the last fragment read of the K tile is out, the A stream after its last load
+        if constexpr (half == 1 && m == LAST_READ + 1) rd_a = rd_a + SLOT == B_REGION ? 0 : rd_a + SLOT;
+        if constexpr (half == 1 && m == LAST_READ + 2) rd_b = rd_b + SLOT == LDS_BYTES ? B_REGION : rd_b + SLOT;
+        if constexpr (half == 1 && m > LAST_A && m <= LAST_A + 3) advance(ld_a, wrap_a, next_a, 0, B_REGION, m - LAST_A - 1);
+        if constexpr (FIRST && gap >= 10 && gap < 10 + 8 * FM && ((gap - 10) & 1) == 0) {
+          // pair q of row block i goes into gap 10 + 8 i + 2 q
+          store_pair(std::integral_constant<int, (gap - 10) / 8>{}, std::integral_constant<int, ((gap - 10) / 2) % 4>{});
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      });
+    };
+
+    if (g_total > 0) {
+      // Prologue: A and B of K tile 0, A of K tile 1 (oldest first: the first wait is about tile 0).
+      TileCoord tc_cur = tile_coord(0);
+      const __amdgpu_buffer_rsrc_t rows_a0 = rows_of_a(0, tc_cur), rows_b0 = rows_of_b(0, tc_cur);
+      next_a = rows_a0;  // (never used: the host sends K >= 3 tiles, so FIRST(0) sets them before any wrap)
+      next_b = rows_b0;
+      ld_a = Stream{rows_a0, 0, wave * 1024};
+      ld_b = Stream{rows_b0, 0, B_REGION + wave * 1024};
+      auto load_whole_tile = [&](const Stream& st, const unsigned(&voff)[LPT]) __attribute__((always_inline)) {
+        w4_static_for<0, LPT>([&](auto i_tag) __attribute__((always_inline)) {
+          set_load_target(st, i_tag);
+          asm volatile("s_nop 0");  // the wait state between the write of M0 and its use
+          load_tile_part(st, voff[decltype(i_tag)::value]);
+        });
+      };
+      load_whole_tile(ld_a, voff_a);
+      load_whole_tile(ld_b, voff_b);
+      advance(ld_a, wrap_a, next_a, 0, B_REGION, -1);
+      advance(ld_b, wrap_b, next_b, B_REGION, LDS_BYTES, -1);
+      load_whole_tile(ld_a, voff_a);
+      advance(ld_a, wrap_a, next_a, 0, B_REGION, -1);
+
+      for (int j = 0; j < my_tiles; ++j) {
+        k_tile(std::true_type{});
+        // From here on the accumulators belong to tile j, and the streams will move on to tile j + 1
+        // (A in the last but one K tile of tile j, B in the last).
+        out = out_tile_of(j, tc_cur);
+        tc_cur = tile_coord(j + 1 < my_tiles ? j + 1 : j);
+        next_a = rows_of_a(j + 1, tc_cur);
+        next_b = rows_of_b(j + 1, tc_cur);
+        for (int h = 1; h < n_k; ++h) k_tile(std::false_type{});
+      }
+      // Drain: the second half of the last K tile is in set 1; then the last tile's output.
+      wait_vm_and_lds<0>();
+      w4_static_for<0, 64>([&](auto m_tag) __attribute__((always_inline)) {
+        constexpr int m = decltype(m_tag)::value;
+        Mfma::template fma<m>(fb1[m & 7], fa1[m >> 3]);
+      });
+      asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+      w4_static_for<0, FM * FN / 2>([&](auto o_tag) __attribute__((always_inline)) {
+        constexpr int o = decltype(o_tag)::value;
+        store_pair(std::integral_constant<int, o / 4>{}, std::integral_constant<int, o % 4>{});
+      });
+    }
+  }
+};
+
+template <typename T, int SB = 4, int SA = 8>
+__global__ void __launch_bounds__(256) gemmrc_w4_kernel(const GemmParams p) {
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+  GemmW4<T, SB, SA>::run(p, smem);
+}
+
+}  // namespace beam

@@ -114,4 +114,10 @@ KernelSet make_kernel_set() {
 
 BEAM_FOR_EACH_SET(BEAM_DECLARE_SET)
 
+// The large-problem kernel of gemm_w4.h (256 x 256 tile, four wavefronts of 128 x 128, one workgroup per
+// CU walking its tiles).  Needs K % 64 == 0, K >= 192, N % 8 == 0, C 16-byte aligned and
+// grid <= tiles_m * tiles_n; kW4MinK names the K bound.
+constexpr int kW4MinK = 192;
+hipError_t launch_gemm_w4(const GemmParams& p, int dtype, dim3 grid, hipStream_t stream);
+
 }  // namespace beam
