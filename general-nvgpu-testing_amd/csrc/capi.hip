@@ -394,6 +394,9 @@ int beam_gemmrc(const void* A, const void* B, void* C, int M, int N, int K, int 
   const bool w4_named = c.block_m == 256 && c.block_n == 256 && c.wave_m == 128 && c.wave_n == 128;
   const bool w4_default = !cfg && c.block_m == 256 && c.block_n == 256 && tiles >= cus;
   if (w4_fits && (w4_named || w4_default)) {
+    // Non-temporal stores of C pay when C is larger than the 256 MB last-level cache (and the K loops
+    // are not so short that the writes are the bound).
+    p.c_streaming = (size_t)M * N * 2 >= ((size_t)256 << 20) && K >= 1024;
     BEAM_HIP(launch_gemm_w4(p, dtype, dim3((unsigned)(tiles < cus ? tiles : cus), 1, 1), st));
     return BEAM_OK;
   }

@@ -122,7 +122,9 @@ __host__ __device__ inline int w4_b_row(int b, int r) { return 32 * (b >> 1) + 4
 // loads of the A tile after next in gaps 0, SA, ... of step B.  The path from the vector-memory unit into
 // LDS moves 64 bytes per cycle and CU, i.e. one 1 KiB load per 64 cycles (4 MFMAs) and wavefront when all
 // four issue: loads issued faster than that stall the wavefront, and with it its MFMAs, at issue.
-template <typename T, int SB = 4, int SA = 8>
+// C_NT: C is stored non-temporal (an output larger than the last-level cache: its lines then do not push
+// operand panels out of the caches).
+template <typename T, bool C_NT = false, int SB = 4, int SA = 8, int G0 = 2>
 struct GemmW4 {
   using Traits = ElemTraits<T>;
   using vec8 = typename Traits::vec8;
@@ -139,7 +141,7 @@ struct GemmW4 {
   static_assert(LDS_BYTES == 160 * 1024 && LPT == 8, "LDS budget");
   // What goes into gap m (after MFMA m) of a step: load number k, or fragment read number n (B 0..7, then
   // A 0..7; they take the gaps the loads leave free, in order), or nothing (-1).
-  static constexpr int G0 = 2;  // gaps 0 and 1 of step A: nothing, then the wait and the barrier
+  // G0: gaps 0 .. G0 - 1 of step A hold nothing but, in the last of them, the wait and the barrier
   static constexpr int load_at(int half, int m) {
     const int s = half == 0 ? SB : SA;
     return (m >= G0 && (m - G0) % s == 0 && (m - G0) / s < LPT) ? (m - G0) / s : -1;
@@ -310,7 +312,7 @@ struct GemmW4 {
       const int skip = i * 16 * N * 2;  // bytes of the row blocks above this one
       const int left = out.bytes - skip;
       const __amdgpu_buffer_rsrc_t rsrc = make_rsrc(out.base + skip, left > 0 ? (unsigned)left : 0u);
-      __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(i32x4, v), rsrc, (int)out.voff[q], 0, 0);
+      __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(i32x4, v), rsrc, (int)out.voff[q], 0, C_NT ? 2 : 0);
     };
 
     // ---- one K tile ------------------------------------------------------------------------------
@@ -425,10 +427,10 @@ struct GemmW4 {
   }
 };
 
-template <typename T, int SB = 4, int SA = 8>
+template <typename T, bool C_NT = false, int SB = 4, int SA = 8, int G0 = 2>
 __global__ void __launch_bounds__(256) gemmrc_w4_kernel(const GemmParams p) {
   extern __shared__ __attribute__((aligned(1024))) char smem[];
-  GemmW4<T, SB, SA>::run(p, smem);
+  GemmW4<T, C_NT, SB, SA, G0>::run(p, smem);
 }
 
 }  // namespace beam
