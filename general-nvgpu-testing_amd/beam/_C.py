@@ -84,6 +84,8 @@ def _load() -> ctypes.CDLL:
     L.beam_gemmrc_ln.argtypes = [vp, vp, vp, vp, ctypes.c_float, vp, i, i, i, i, cfgp, vp, sz, vp]
     L.beam_gemmrc_ln_workspace_bytes_ex.argtypes = [i, i, cfgp, i]
     L.beam_gemmrc_ln_workspace_bytes_ex.restype = sz
+    L.beam_gemmrc_ln_workspace_bytes_for.argtypes = [i, i, i, cfgp, i]
+    L.beam_gemmrc_ln_workspace_bytes_for.restype = sz
     L.beam_gemmrc_ln_ex.argtypes = [vp, vp, vp, vp, ctypes.c_float, vp, i, i, i, i, cfgp, i, vp, sz, vp]
     L.beam_set_ln_spin_limit.argtypes = [i]
     L.beam_gemmrc_ln_workspace_reset.argtypes = [vp]
@@ -296,10 +298,8 @@ def _get_ln_workspace(nbytes: int) -> DeviceArray:
     if _ln_workspace is None or _ln_workspace.nbytes < nbytes:
         if _ln_workspace is not None:
             _check(lib.beam_sync(None))
-            lib.beam_gemmrc_ln_workspace_reset(_ln_workspace.ptr)
             _ln_workspace.free()
-        _ln_workspace = DeviceArray((max(nbytes, 1 << 20),), itemsize=1)
-        lib.beam_gemmrc_ln_workspace_reset(_ln_workspace.ptr)
+        _ln_workspace = DeviceArray((max(nbytes, 1 << 20),), itemsize=1)  # whatever it holds: the library checks
     return _ln_workspace
 
 
@@ -363,9 +363,11 @@ LN_AUTO, LN_TWOPASS, LN_FUSED = 0, 1, 2
 
 
 def gemmrc_ln(a, b, c, gamma, beta, eps: float = 1e-5, config: Optional[TileConfig] = None,
-              mode: int = LN_AUTO) -> None:
+              mode: int = LN_AUTO, check: bool = False) -> None:
     """c = LayerNorm_N(a @ b.T) * gamma + beta, statistics from the fp32 accumulators.
-    mode: LN_AUTO (fused single kernel when N / block_n <= 64), LN_TWOPASS, LN_FUSED."""
+    mode: LN_AUTO (fused single kernel when N / block_n <= 64), LN_TWOPASS, LN_FUSED.
+    check: wait for the result and raise BeamError if the fused kernel gave up waiting for a band (its
+    workgroups need the device to themselves; the rows concerned are NaN then)."""
     pa, pb, pc, M, N, K, d, st = _problem(a, b, c)
     pg, sg, dg, _ = _describe(gamma)
     pbt, sbt, dbt, _ = _describe(beta)
@@ -373,9 +375,15 @@ def gemmrc_ln(a, b, c, gamma, beta, eps: float = 1e-5, config: Optional[TileConf
         raise BeamError(1, "gamma and beta must be [N] of the same dtype as a, b, c")
     cfg = config.to_c() if config is not None else None
     cfgp = ctypes.byref(cfg) if cfg else None
-    need = lib.beam_gemmrc_ln_workspace_bytes_ex(M, N, cfgp, mode)
+    need = lib.beam_gemmrc_ln_workspace_bytes_for(M, N, K, cfgp, mode)
     ws = _get_ln_workspace(need)
     _check(lib.beam_gemmrc_ln_ex(pa, pb, pg, pbt, eps, pc, M, N, K, d, cfgp, mode, ws.ptr, ws.nbytes, st))
+    if check:
+        flag = ctypes.c_int(0)
+        _check(lib.beam_gemmrc_ln_timed_out(ws.ptr, st, ctypes.byref(flag)))
+        if flag.value:
+            raise BeamError(4, "fused GEMM+LayerNorm gave up waiting for a band of workgroups (device shared with "
+                               "other work?); use mode=LN_TWOPASS")
 
 
 def gemmrc_ln_timed_out() -> bool:

@@ -17,6 +17,12 @@ hipError_t launch_ln_apply(const float* X, const float* stats, const void* gamma
                            void* Y, int M, int N, int tiles_n, int block_n, float eps, int dtype,
                            hipStream_t stream);
 
+// Stream-ordered preparation of a fused GEMM+LayerNorm workspace (header of 64 ints + two statistics sets of
+// set_floats_total / 2 floats each) for its next launch: validates the header on the device and either
+// advances the epoch or re-initialises everything.
+hipError_t launch_ln_prepare(int* header, float* sets, size_t set_floats_total, int geom_lo, int geom_hi, int expected,
+                             hipStream_t stream);
+
 // y[i] (16-bit) = silu(x[i]) for i in [0, count); x and y 16-byte aligned.
 hipError_t launch_silu(const void* x, void* y, size_t count, int dtype, hipStream_t stream);
 

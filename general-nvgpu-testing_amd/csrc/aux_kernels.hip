@@ -5,6 +5,7 @@
 #include <type_traits>
 
 #include "elementwise.h"
+#include "tile_map.h"
 
 namespace beam {
 
@@ -138,6 +139,34 @@ __global__ void __launch_bounds__(256) silu_kernel(const T* __restrict__ x, T* _
   if (i < count) y[i] = silu_16<T>(x[i]);
 }
 
+// Before every fused GEMM+LayerNorm launch: decide, on the device, whether the workspace is in the state the
+// previous fused launch left it in -- header intact, same geometry, and every workgroup of that launch
+// finished (each of them has marked its slots of the other statistics set "not published") -- and then
+// just move on to the next epoch; otherwise mark both sets "not published" (M2 = -1) and start at epoch 0.
+// One workgroup: the decision and the header update are then trivially ordered around the fill.
+__global__ void __launch_bounds__(1024) ln_prepare_kernel(int* hdr, float* sets, size_t set_floats_total, int geom_lo,
+                                                           int geom_hi, int expected) {
+  __shared__ int valid;
+  if (threadIdx.x == 0)
+    valid = hdr[kLnHdrMagic] == kLnMagic && hdr[kLnHdrGeometry] == geom_lo && hdr[kLnHdrGeometry + 1] == geom_hi &&
+            hdr[kLnHdrExpected] == expected && hdr[kLnHdrDone] == expected;
+  __syncthreads();
+  if (!valid) {
+    const f32x4 unpublished = {-1.0f, -1.0f, -1.0f, -1.0f};
+    for (size_t i = threadIdx.x; i < set_floats_total / 4; i += blockDim.x) ((f32x4*)sets)[i] = unpublished;
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) {
+    hdr[kLnHdrTimeout] = 0;
+    hdr[kLnHdrMagic] = kLnMagic;
+    hdr[kLnHdrGeometry] = geom_lo;
+    hdr[kLnHdrGeometry + 1] = geom_hi;
+    hdr[kLnHdrEpoch] = valid ? hdr[kLnHdrEpoch] + 1 : 0;
+    hdr[kLnHdrDone] = 0;
+    hdr[kLnHdrExpected] = expected;
+  }
+}
+
 __global__ void zero_u16_kernel(unsigned short* p, size_t n) {
   for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) p[i] = 0;
 }
@@ -167,6 +196,13 @@ hipError_t launch_silu(const void* x, void* y, size_t count, int dtype, hipStrea
 
 hipError_t launch_fill_floats(float* floats, size_t n, float value, hipStream_t stream) {
   hipLaunchKernelGGL(fill_floats_kernel, dim3(256), dim3(256), 0, stream, floats, n, value);
+  return hipGetLastError();
+}
+
+hipError_t launch_ln_prepare(int* header, float* sets, size_t set_floats_total, int geom_lo, int geom_hi, int expected,
+                             hipStream_t stream) {
+  hipLaunchKernelGGL(ln_prepare_kernel, dim3(1), dim3(1024), 0, stream, header, sets, set_floats_total, geom_lo, geom_hi,
+                     expected);
   return hipGetLastError();
 }
 

@@ -6,7 +6,6 @@
 #include <cstdio>
 #include <cstring>
 #include <atomic>
-#include <map>
 #include <mutex>
 #include <thread>
 #include <vector>
@@ -49,16 +48,8 @@ struct Device {
 };
 Device g_dev;
 std::mutex g_dev_mu;
-// Per workspace: tile geometry of the fused GEMM+LayerNorm launches it has seen and their number
-// (selects the statistics set).
-struct LnWorkspaceState {
-  long geometry;
-  unsigned launches;
-};
-std::map<const void*, LnWorkspaceState> g_ln_geometry;
-// polls of a band counter (about a microsecond each) before a fused LayerNorm workgroup gives up
+// polls of statistics slots (about a microsecond each) before a thread of a fused LayerNorm workgroup gives up
 std::atomic<int> g_ln_spin_limit{4 << 20};
-std::mutex g_ln_mu;
 
 const std::vector<KernelSet>& kernel_sets() {
   static const std::vector<KernelSet> sets = [] {
@@ -577,15 +568,20 @@ int beam_gemmrc_splitk(const void* A, const void* B, void* C, int M, int N, int 
   return BEAM_OK;
 }
 
-// Fused GEMM+LayerNorm workspace: [band counters (tiles_m) + timeout flag | statistics].
-// Fused GEMM+LayerNorm workspace: [timeout flag, 256 bytes | statistics set 0 | statistics set 1];
-// launches alternate between the sets and each marks the other one "unpublished" for its successor.
+// Fused GEMM+LayerNorm workspace: [header, 256 bytes | statistics set 0 | statistics set 1].  The header
+// (tile_map.h: kLnHdr*) carries a magic word, the geometry the sets are laid out for, the epoch whose parity
+// selects the set of a launch, and how many workgroups of the latest launch have finished; a small kernel in
+// front of every fused launch checks it on the device and re-initialises the workspace when anything is off
+// (first use, another geometry, a buffer handed out again by an allocator, an interrupted launch).  The
+// library keeps no host-side state about workspaces.
 static size_t ln_fused_header_bytes() { return 256; }
 static size_t ln_fused_set_bytes(size_t tiles_m, size_t tiles_n, int block_m) {
   return align_up(tiles_m * tiles_n * (size_t)block_m * 2 * sizeof(float), 256);
 }
 
 static bool ln_fused_applies(const beam_tile_cfg& c, const KernelSet& ks, int N) {
+  // The residency argument of the fused kernel (tile_map.h: band_block_tile) is made for 8 XCDs of 32 CUs.
+  if (g_dev.cus != kNumXcd * 32) return false;
   // a band's column tiles are spread over the 8 XCDs; each XCD must hold its share (<= 32) at once,
   // and the band's statistics ((tiles_n + 1) * block_m pairs) are gathered into the kernel's LDS
   const int tiles_n = (N + c.block_n - 1) / c.block_n;
@@ -598,17 +594,46 @@ static int ln_resolve_mode(int mode, const beam_tile_cfg& c, const KernelSet& ks
   return mode;
 }
 
-size_t beam_gemmrc_ln_workspace_bytes_ex(int M, int N, const beam_tile_cfg* cfg, int mode) {
-  if (M <= 0 || N <= 0) return 0;
-  beam_tile_cfg c;
-  const KernelSet* ks;
-  if (resolve_cfg(cfg, M, N, 64, &c, &ks)) return 0;
-  if (c.pipeline == 2) c.pipeline = 0;
+// Bytes for tile `c` in `mode` (already resolved: two-pass or fused).
+static size_t ln_workspace_need(int M, int N, const beam_tile_cfg& c, int mode) {
   const size_t tiles_m = (size_t)(M + c.block_m - 1) / c.block_m;
   const size_t tiles_n = (size_t)(N + c.block_n - 1) / c.block_n;
-  if (ln_resolve_mode(mode, c, *ks, N) == BEAM_LN_FUSED)
-    return ln_fused_header_bytes() + 2 * ln_fused_set_bytes(tiles_m, tiles_n, c.block_m);
+  if (mode == BEAM_LN_FUSED) return ln_fused_header_bytes() + 2 * ln_fused_set_bytes(tiles_m, tiles_n, c.block_m);
   return align_up((size_t)M * N * sizeof(float), 256) + align_up((size_t)M * tiles_n * 2 * sizeof(float), 256);
+}
+
+// The tile a GEMM+LayerNorm call runs with: the caller's, or the default for (M, N, K); never the deep pipeline.
+static int ln_resolve_cfg(const beam_tile_cfg* cfg, int M, int N, int K, beam_tile_cfg* c, const KernelSet** ks) {
+  int rc = resolve_cfg(cfg, M, N, K, c, ks);
+  if (rc) return rc;
+  if (c->pipeline == 2) c->pipeline = 0;  // the deep pipeline exists for the store / split-K kernels only
+  return BEAM_OK;
+}
+
+size_t beam_gemmrc_ln_workspace_bytes_for(int M, int N, int K, const beam_tile_cfg* cfg, int mode) {
+  if (M <= 0 || N <= 0 || K < 0) return 0;
+  (void)beam_init();  // AUTO depends on the device
+  beam_tile_cfg c;
+  const KernelSet* ks;
+  if (ln_resolve_cfg(cfg, M, N, K, &c, &ks)) return 0;
+  return ln_workspace_need(M, N, c, ln_resolve_mode(mode, c, *ks, N));
+}
+
+size_t beam_gemmrc_ln_workspace_bytes_ex(int M, int N, const beam_tile_cfg* cfg, int mode) {
+  if (M <= 0 || N <= 0) return 0;
+  if (cfg) return beam_gemmrc_ln_workspace_bytes_for(M, N, 64, cfg, mode);  // a given tile does not depend on K
+  // Without a tile the library picks one from (M, N, K), and K is not known here: the largest need over
+  // every tile it can pick.
+  (void)beam_init();
+  size_t need = 0;
+  for (int i = 0; i < beam_num_configs(); ++i) {
+    beam_tile_cfg c;
+    const KernelSet* ks;
+    if (beam_get_config(i, &c) || resolve_cfg(&c, M, N, 64, &c, &ks)) continue;
+    const size_t n = ln_workspace_need(M, N, c, ln_resolve_mode(mode, c, *ks, N));
+    need = n > need ? n : need;
+  }
+  return need;
 }
 
 size_t beam_gemmrc_ln_workspace_bytes(int M, int N, const beam_tile_cfg* cfg) {
@@ -629,22 +654,18 @@ int beam_gemmrc_ln_ex(const void* A, const void* B, const void* gamma, const voi
   hipStream_t st = (hipStream_t)stream;
   beam_tile_cfg c;
   const KernelSet* ks;
-  if ((rc = resolve_cfg(cfg, M, N, K, &c, &ks))) return rc;
-  if (c.pipeline == 2) c.pipeline = 0;  // the deep pipeline exists for the store / split-K kernels only
+  if ((rc = ln_resolve_cfg(cfg, M, N, K, &c, &ks))) return rc;
   if (mode == BEAM_LN_FUSED && !ln_fused_applies(c, *ks, N))
-    return fail(BEAM_ERR_UNSUPPORTED, "fused LayerNorm: too many column tiles for this tile shape (N=%d, block_n=%d)", N, c.block_n);
-  // A fused launch depends on how many launches its workspace has seen (the two statistics sets
-  // alternate), which a captured graph would freeze: under stream capture AUTO takes the two-pass
-  // path and an explicit FUSED is refused.
+    return fail(BEAM_ERR_UNSUPPORTED, "fused LayerNorm: needs a device of %d CUs and at most 64 column tiles (N=%d, block_n=%d, %d CUs)",
+                kNumXcd * 32, N, c.block_n, g_dev.cus);
+  // The fused kernel's workgroups wait for one another; whether a replayed graph meets the residency that
+  // wait relies on (other graph branches may share the device) is the caller's business: under stream
+  // capture AUTO takes the two-pass path, an explicit FUSED is honoured.
   hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
   if (st != nullptr) (void)hipStreamIsCapturing(st, &capturing);
-  if (capturing != hipStreamCaptureStatusNone) {
-    if (mode == BEAM_LN_FUSED)
-      return fail(BEAM_ERR_UNSUPPORTED, "fused GEMM+LayerNorm cannot be captured in a graph (use BEAM_LN_TWOPASS or BEAM_LN_AUTO)");
-    mode = BEAM_LN_TWOPASS;
-  }
+  if (capturing != hipStreamCaptureStatusNone && mode == BEAM_LN_AUTO) mode = BEAM_LN_TWOPASS;
   mode = ln_resolve_mode(mode, c, *ks, N);
-  const size_t need = beam_gemmrc_ln_workspace_bytes_ex(M, N, &c, mode);
+  const size_t need = ln_workspace_need(M, N, c, mode);
   if (!ws || ws_bytes < need)
     return fail(BEAM_ERR_WORKSPACE, "GEMM+LayerNorm needs %zu bytes of workspace, got %zu", need, ws_bytes);
   if ((uintptr_t)ws & 255) return fail(BEAM_ERR_UNSUPPORTED, "workspace must be 256-byte aligned");
@@ -652,25 +673,13 @@ int beam_gemmrc_ln_ex(const void* A, const void* B, const void* gamma, const voi
   // K == 0: the kernels run with an empty K range and produce x = 0, i.e. y = beta.
   if (mode == BEAM_LN_FUSED) {
     p.C = Y;
-    // The first launch on a workspace (or after its geometry changed) marks both statistics sets
-    // unpublished; afterwards each launch finds its set prepared by the previous one.  Launches that
-    // share a workspace must be ordered (same stream): overlapping ones would race on the sets.
+    // Launches that share a workspace must be ordered (same stream): overlapping ones would race on the sets.
     const size_t set_bytes = ln_fused_set_bytes(p.tiles_m, p.tiles_n, c.block_m);
-    const long geometry = ((long)p.tiles_m << 32) | ((long)p.tiles_n << 12) | c.block_m;
-    unsigned launches = 0;
-    {
-      std::lock_guard<std::mutex> lk(g_ln_mu);
-      auto it = g_ln_geometry.find(ws);
-      if (it != g_ln_geometry.end() && it->second.geometry == geometry) launches = it->second.launches;
-      g_ln_geometry[ws] = LnWorkspaceState{geometry, launches + 1};
-    }
     float* sets = (float*)((char*)ws + ln_fused_header_bytes());
-    if (launches == 0) {
-      BEAM_HIP(launch_zero_ints((int*)ws, 1, st));
-      BEAM_HIP(launch_fill_floats(sets, 2 * set_bytes / sizeof(float), -1.0f, st));
-    }
-    p.stats = (float*)((char*)sets + (launches & 1u) * set_bytes);
-    p.next_stats = (float*)((char*)sets + ((launches + 1) & 1u) * set_bytes);
+    BEAM_HIP(launch_ln_prepare((int*)ws, sets, 2 * set_bytes / sizeof(float), p.tiles_m, (p.tiles_n << 12) | c.block_m,
+                               p.tiles_m * p.tiles_n, st));
+    p.stats = sets;
+    p.next_stats = (float*)((char*)sets + set_bytes);
     p.timeout_flag = (int*)ws;
     p.gamma = gamma;
     p.beta = beta;
@@ -701,10 +710,6 @@ int beam_gemmrc_ln_ex(const void* A, const void* B, const void* gamma, const voi
     BEAM_HIP(ks->launch[dtype][kEpiLnFused][c.pipeline](p, dim3(grid, 1, 1), st));
     return BEAM_OK;
   }
-  {
-    std::lock_guard<std::mutex> lk(g_ln_mu);
-    g_ln_geometry.erase(ws);  // no fused launch is pending on this workspace any more
-  }
   p.ws = (float*)ws;
   p.stats = (float*)((char*)ws + align_up((size_t)M * N * sizeof(float), 256));
   BEAM_HIP(ks->launch[dtype][kEpiLnStats][c.pipeline](p, dim3((unsigned)(p.tiles_m * p.tiles_n), 1, 1), st));
@@ -719,13 +724,13 @@ int beam_gemmrc_ln(const void* A, const void* B, const void* gamma, const void* 
 }
 
 int beam_gemmrc_ln_workspace_reset(const void* ws) {
-  std::lock_guard<std::mutex> lk(g_ln_mu);
-  g_ln_geometry.erase(ws);
+  if (!ws) return fail(BEAM_ERR_INVALID, "null workspace");
+  BEAM_HIP(hipMemset(const_cast<void*>(ws), 0, ln_fused_header_bytes()));  // no magic word: the next launch starts over
   return BEAM_OK;
 }
 
 int beam_set_ln_spin_limit(int polls) {
-  if (polls < 0) return fail(BEAM_ERR_INVALID, "spin limit must be >= 0");
+  if (polls < -1) return fail(BEAM_ERR_INVALID, "spin limit must be >= -1");
   g_ln_spin_limit.store(polls);
   return BEAM_OK;
 }
@@ -733,16 +738,9 @@ int beam_set_ln_spin_limit(int polls) {
 int beam_gemmrc_ln_timed_out(const void* ws, void* stream, int* timed_out) {
   if (!ws || !timed_out) return fail(BEAM_ERR_INVALID, "null argument");
   BEAM_HIP(hipStreamSynchronize((hipStream_t)stream));
-  {
-    std::lock_guard<std::mutex> lk(g_ln_mu);
-    if (g_ln_geometry.find(ws) == g_ln_geometry.end()) {  // no fused launch has used this workspace
-      *timed_out = 0;
-      return BEAM_OK;
-    }
-  }
-  int flag = 0;
-  BEAM_HIP(hipMemcpy(&flag, ws, sizeof(int), hipMemcpyDeviceToHost));
-  *timed_out = flag;
+  int hdr[2] = {0, 0};
+  BEAM_HIP(hipMemcpy(hdr, ws, sizeof hdr, hipMemcpyDeviceToHost));
+  *timed_out = (hdr[kLnHdrMagic] == kLnMagic) ? hdr[kLnHdrTimeout] : 0;  // no fused launch has prepared this workspace
   return BEAM_OK;
 }
 

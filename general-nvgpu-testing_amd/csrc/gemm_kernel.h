@@ -96,9 +96,14 @@ struct GemmParams {
   void* C;       // 16-bit [M][N]                                  (kEpiStore)
   float* ws;     // fp32 [splits][M][N] (kEpiPartial) or fp32 [M][N] (kEpiLnStats)
   float* stats;  // fp32 [M][tiles_n][2] = (mean, M2) over the tile's columns (kEpiLnStats)
-                 // fp32 [tiles_m][tiles_n][BM][2], every M2 = -1 ("not published") on entry (kEpiLnFused)
-  float* next_stats;    // the statistics set the NEXT launch on this workspace will use: reset here
-  int* timeout_flag;    // set to 1 if a bounded wait ran out (never expected)        (kEpiLnFused)
+                 // kEpiLnFused: statistics set 0, fp32 [tiles_m][tiles_n][BM][2]; launches alternate between
+                 // two sets by the parity of the workspace's epoch; every M2 of a launch's set is -1 ("not
+                 // published") when it starts, and it leaves the other set like that for its successor
+  float* next_stats;    // kEpiLnFused: statistics set 1
+  // kEpiLnFused: the workspace header, kept by ln_prepare_kernel (aux_kernels.hip):
+  //   [0] set to 1 if a bounded wait ran out (never expected)   [4] epoch of this launch
+  //   [5] workgroups of this launch that have finished
+  int* timeout_flag;
   const void* gamma;    // 16-bit [N]                                                   (kEpiLnFused)
   const void* beta;     // 16-bit [N]
   float eps;
@@ -991,8 +996,11 @@ struct GemmTile {
       //    write-back / invalidate (a __threadfence() per workgroup costs tens of microseconds here).
       //    A slot whose M2 is negative has not been published yet: M2 of real data is never negative.
       const size_t my_slot = ((size_t)tc.tm * p.tiles_n + tc.tn) * BM;
-      unsigned long long* my_stats = (unsigned long long*)p.stats + my_slot;
-      unsigned long long* my_next = (unsigned long long*)p.next_stats + my_slot;
+      const bool odd_epoch = (p.timeout_flag[kLnHdrEpoch] & 1) != 0;  // uniform; written before this launch began
+      float* const cur_set = odd_epoch ? p.next_stats : p.stats;
+      float* const other_set = odd_epoch ? p.stats : p.next_stats;
+      unsigned long long* my_stats = (unsigned long long*)cur_set + my_slot;
+      unsigned long long* my_next = (unsigned long long*)other_set + my_slot;
       // (tile_row_stats left row rl's pair with the thread that publishes it: same rl = tid stride)
       for (int rl = tid; rl < BM; rl += NT) {
         const float mean = red[rl * 2 + 0];
@@ -1008,8 +1016,9 @@ struct GemmTile {
       // 3. gather the band's statistics into LDS: one 8-byte device-scope load per (tile, row), all in
       //    flight together, each repeated (bounded) until its tile has published
       float* gathered = part;  // [tiles_n][BM][2]; tiles_n <= 64 keeps it within the LDS the kernel owns
-      const unsigned long long* band_stats = (const unsigned long long*)p.stats + (size_t)tc.tm * p.tiles_n * BM;
+      const unsigned long long* band_stats = (const unsigned long long*)cur_set + (size_t)tc.tm * p.tiles_n * BM;
       const int n_slots = p.tiles_n * BM;
+      int polls = 0;  // one budget for all the slots of this thread: a thread that ran out of it polls no more
       for (int q0 = tid; q0 < n_slots; q0 += 8 * NT) {
         unsigned long long v[8];
 #pragma unroll
@@ -1021,10 +1030,14 @@ struct GemmTile {
         for (int u = 0; u < 8; ++u) {
           const int q = q0 + u * NT;
           if (q >= n_slots) break;
-          int polls = 0;
-          while ((long long)v[u] < 0) {  // sign bit of M2: not published yet
+          // sign bit of M2: not published yet (a negative limit: treat everything as unpublished -- how the
+          // host forces this path in a test)
+          while ((long long)v[u] < 0 || p.spin_limit < 0) {
             if (++polls > p.spin_limit) {
-              *p.timeout_flag = 1;
+              // Give up: raise the flag and poison the row's statistics, so that the rows concerned come out
+              // as NaN instead of as plausible numbers.
+              p.timeout_flag[kLnHdrTimeout] = 1;
+              v[u] = 0x7fc000007fc00000ull;
               break;
             }
             __builtin_amdgcn_s_sleep(4);
@@ -1080,6 +1093,9 @@ struct GemmTile {
                        v[e] = (T)((acc[i][j][e] - st.mean) * st.rstd * (float)gv[j][e] + (float)bv[j][e]);
                      return v;
                    });
+      // One more workgroup has published its statistics and marked its slots of the other set: the next
+      // launch's preparation trusts the workspace only if every workgroup of this one got here.
+      if (tid == 0) __hip_atomic_fetch_add(p.timeout_flag + kLnHdrDone, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     } else {
       if (EPI == kEpiLnStats) {
         // Per-row statistics over the columns this workgroup owns, from the fp32 accumulators.

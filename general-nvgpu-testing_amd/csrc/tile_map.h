@@ -11,11 +11,7 @@
 //       cuda/cute_kernels/cute_gemm_128x128.cu:55-65  (Swizzle<3,3,3>)
 #pragma once
 
-#if defined(__HIPCC__) || defined(__CUDACC__)
 #define BEAM_HD __host__ __device__ inline
-#else
-#define BEAM_HD inline
-#endif
 
 namespace beam {
 
@@ -52,6 +48,15 @@ BEAM_HD int kmajor_swizzle(int k, int block_n) {
 BEAM_HD int kmajor_lds_offset(int k, int n, int block_n) {
   return k * block_n * 2 + ((((n >> 3) ^ kmajor_swizzle(k, block_n))) << 4) + ((n & 7) << 1);
 }
+
+// Words of the fused GEMM+LayerNorm workspace header (256 bytes in front of the two statistics sets).
+constexpr int kLnHdrTimeout = 0;   // 1: a workgroup gave up waiting for a band's statistics
+constexpr int kLnHdrMagic = 1;     // kLnMagic once the workspace has been prepared
+constexpr int kLnHdrGeometry = 2;  // two words: (tiles_m, tiles_n, block_m) the sets are laid out for
+constexpr int kLnHdrEpoch = 4;     // launches so far; its parity selects the statistics set
+constexpr int kLnHdrDone = 5;      // workgroups of the latest launch that have finished
+constexpr int kLnHdrExpected = 6;  // ... out of this many
+constexpr int kLnMagic = 0x4c4e3032;
 
 struct TileCoord {
   int tm;  // tile index along M

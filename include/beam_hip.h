@@ -120,29 +120,42 @@ int beam_gemmrc_ln(const void* A, const void* B, const void* gamma, const void* 
 
 /* The two ways the library computes it, selectable for testing and tuning:
  *   BEAM_LN_FUSED   one kernel: each workgroup keeps its fp32 accumulators in registers, the column
- *                   tiles of a row band exchange per-row (mean, M2) pairs through the workspace and a
- *                   per-band arrival counter, then every workgroup normalises and stores its own tile.
- *                   Needs all column tiles of a band resident at once: N / block_n <= 64.
+ *                   tiles of a row band exchange per-row (mean, M2) pairs through the workspace (every
+ *                   workgroup publishes its own and polls, boundedly, for the others'), then every
+ *                   workgroup normalises and stores its own tile.  Needs all column tiles of a band
+ *                   resident at once: N / block_n <= 64, a device of 256 CUs in 8 XCDs, and the device
+ *                   not shared with other work while it runs.
  *   BEAM_LN_TWOPASS the GEMM kernel stores fp32 X and per-tile statistics, a second kernel normalises.
- *   BEAM_LN_AUTO    fused when it applies, else two-pass (what beam_gemmrc_ln does). */
+ *   BEAM_LN_AUTO    fused when it applies, else two-pass (what beam_gemmrc_ln does); two-pass under
+ *                   stream capture. */
 typedef enum beam_ln_mode { BEAM_LN_AUTO = 0, BEAM_LN_TWOPASS = 1, BEAM_LN_FUSED = 2 } beam_ln_mode;
+/* Workspace bytes.  _for is exact for the call beam_gemmrc_ln_ex(M, N, K, cfg, mode) will make; the
+ * forms without K return, for cfg == NULL, the largest need over every tile the library could pick
+ * for some K (with a tile given they are exact as well). */
+size_t beam_gemmrc_ln_workspace_bytes_for(int M, int N, int K, const beam_tile_cfg* cfg, int mode);
 size_t beam_gemmrc_ln_workspace_bytes_ex(int M, int N, const beam_tile_cfg* cfg, int mode);
 int beam_gemmrc_ln_ex(const void* A, const void* B, const void* gamma, const void* beta, float eps,
                       void* Y, int M, int N, int K, int dtype, const beam_tile_cfg* cfg, int mode,
                       void* ws, size_t ws_bytes, void* stream);
 /* The fused path keeps state in its workspace between launches (each launch prepares the statistics
- * slots of the next one), and the library remembers per workspace pointer that it did.  If anything
- * else writes to a workspace that fused launches have used (or it is freed and the address reused),
- * call this before the next fused launch; that launch then re-initialises the workspace itself.
- * Launches sharing one workspace must be ordered on one stream. */
+ * slots of the next one), described by a 256-byte header in the workspace itself: magic word,
+ * geometry, launch count and how many workgroups of the latest launch finished.  A small kernel in
+ * front of every fused launch checks the header on the device and re-initialises the workspace if
+ * anything is off, so a fresh buffer, a buffer the allocator hands out again, a different problem
+ * shape or an interrupted launch need nothing from the caller; the library keeps no host-side record
+ * of workspaces.  What the check cannot see is a foreign write into the statistics that leaves the
+ * header intact: after such a write call this (it clears the header, synchronously).  Launches
+ * sharing one workspace must be ordered on one stream. */
 int beam_gemmrc_ln_workspace_reset(const void* ws);
-/* Waits for `stream`, then *timed_out = 1 if a fused call on this workspace gave up waiting for a
- * band (its output is then invalid).  Only possible if the device could not hold a whole band of
- * workgroups at once, e.g. because another process occupied most of it. */
+/* Waits for `stream`, then *timed_out = 1 if the latest fused call on this workspace gave up
+ * waiting for a band: the rows concerned are then NaN in Y.  Only possible if the device could not
+ * hold a whole band of workgroups at once, e.g. because another process occupied most of it.  The
+ * flag is cleared at the start of every fused call. */
 int beam_gemmrc_ln_timed_out(const void* ws, void* stream, int* timed_out);
-/* Bound of that wait, in polls of the band counter (roughly a microsecond each; default 4 Mi).
- * 0 makes every workgroup give up at once: the kernel still ends normally and the flag is set,
- * which is how the failure path is exercised without hanging anything. */
+/* Bound of that wait: polls of statistics slots per thread (roughly a microsecond each; default
+ * 4 Mi).  0 makes every thread that finds a slot unpublished give up at once; -1 makes every wait give
+ * up whatever it finds: the kernel still ends normally and the flag is set, which is how the failure
+ * path is exercised without hanging anything. */
 int beam_set_ln_spin_limit(int polls);
 
 /* ---- GEMM with an independent elementwise job hidden in its K loop ------------------------ */

@@ -1,7 +1,9 @@
 """A captured sequence of operators replays as a HIP graph with the eager results.
 
 The graph holds gemmrc, split-K (two kernels), GEMM+SiLU, the [K][N] matmul, a K = 0 call (its clear is a
-kernel, not a memset node) and a two-pass GEMM+LayerNorm (what BEAM_LN_AUTO turns into under capture).
+kernel, not a memset node), a two-pass GEMM+LayerNorm (what BEAM_LN_AUTO turns into under capture) and an
+explicitly fused one (its workspace keeps its launch count on the device, so replays and the eager calls in
+between simply take turns on it).
 It is replayed several times with the inputs changed and eager work of the library in between; every
 replay must reproduce, bit for bit, what the same calls give eagerly on the same inputs.
 """
@@ -27,12 +29,13 @@ def test_graph_replay_matches_eager(gpu, beamc):
     a, b, bkn, x = (beamc.DeviceArray(s, F16) for s in ((M, K), (N, K), (K, N), (n,)))
     g = beamc.DeviceArray.from_numpy(beamc.host_normal((N,), F16, 99, 1000, 1.0, 0.1), F16)
     bt = beamc.DeviceArray.from_numpy(beamc.host_normal((N,), F16, 99, 1001, 0.0, 0.1), F16)
-    outs = {k: beamc.DeviceArray((M, N), F16) for k in ("gemm", "splitk", "pair", "nn", "k0", "ln")}
+    outs = {k: beamc.DeviceArray((M, N), F16) for k in ("gemm", "splitk", "pair", "nn", "k0", "ln", "lnf")}
     y = beamc.DeviceArray((n,), F16)
     cfg = beamc.TileConfig(64, 64, 32, 32, 0, 0).to_c()
     s_eff = L.beam_splitk_effective(M, N, K, ctypes.byref(cfg), 4)
     ws_sk = beamc.DeviceArray((max(L.beam_splitk_workspace_bytes(M, N, s_eff), 256),), F16, 1)
     ws_ln = beamc.DeviceArray((L.beam_gemmrc_ln_workspace_bytes_ex(M, N, None, beamc.LN_TWOPASS),), F16, 1)
+    ws_lnf = beamc.DeviceArray((L.beam_gemmrc_ln_workspace_bytes_ex(M, N, None, beamc.LN_FUSED),), F16, 1)
 
     def upload():
         for d, shape, scale in ((a, (M, K), K ** -0.5), (b, (N, K), K ** -0.5), (bkn, (K, N), K ** -0.5), (x, (n,), 2.0)):
@@ -47,6 +50,8 @@ def test_graph_replay_matches_eager(gpu, beamc):
         chk(L.beam_gemmrc(a.ptr, b.ptr, outs["k0"].ptr, M, N, 0, F16, None, stream))
         chk(L.beam_gemmrc_ln_ex(a.ptr, b.ptr, g.ptr, bt.ptr, 1e-5, outs["ln"].ptr, M, N, K, F16, None, beamc.LN_AUTO if stream else beamc.LN_TWOPASS,
                                 ws_ln.ptr, ws_ln.nbytes, stream))
+        chk(L.beam_gemmrc_ln_ex(a.ptr, b.ptr, g.ptr, bt.ptr, 1e-5, outs["lnf"].ptr, M, N, K, F16, None, beamc.LN_FUSED,
+                                ws_lnf.ptr, ws_lnf.nbytes, stream))
 
     def snapshot():
         return {k: v.to_numpy().copy() for k, v in list(outs.items()) + [("y", y)]}
@@ -62,9 +67,6 @@ def test_graph_replay_matches_eager(gpu, beamc):
     chk(L.beam_sync(None))
     chk(L.beam_graph_begin_capture(stream))
     sequence(stream)
-    rc = L.beam_gemmrc_ln_ex(a.ptr, b.ptr, g.ptr, bt.ptr, 1e-5, outs["ln"].ptr, M, N, K, F16, None, beamc.LN_FUSED,
-                             ws_ln.ptr, ws_ln.nbytes, stream)
-    assert rc == 2, "an explicit fused LayerNorm must be refused under capture"
     graph = ctypes.c_void_p()
     chk(L.beam_graph_end_capture(stream, ctypes.byref(graph)))
     try:
@@ -80,8 +82,11 @@ def test_graph_replay_matches_eager(gpu, beamc):
             got = snapshot()
             for k in want:
                 assert (got[k] == want[k]).all(), f"replay {replay}: {k} differs from the eager result"
+            timed_out = ctypes.c_int(1)
+            chk(L.beam_gemmrc_ln_timed_out(ws_lnf.ptr, stream, ctypes.byref(timed_out)))
+            assert timed_out.value == 0
     finally:
         chk(L.beam_graph_destroy(graph))
         chk(L.beam_stream_destroy(stream))
-        for t in [a, b, bkn, x, g, bt, y, ws_sk, ws_ln] + list(outs.values()):
+        for t in [a, b, bkn, x, g, bt, y, ws_sk, ws_ln, ws_lnf] + list(outs.values()):
             t.free()

@@ -8,6 +8,15 @@ from test_gpu_gemm import F16, BF16
 pytestmark = pytest.mark.gpu
 
 LN_TOL = 2e-3
+# fp16: what is left of the error once the rounding of the output itself (half an ulp: at most |y| * 2^-11)
+# is taken off, i.e. the error of the statistics and the normalisation
+LN_OWN_TOL = 2e-4
+
+
+def f16_error_beyond_rounding(got_bits, ref32):
+    got = np.ascontiguousarray(got_bits, dtype=np.uint16).view(np.float16).astype(np.float64).ravel()
+    ref = np.asarray(ref32, dtype=np.float64).ravel()
+    return float((np.abs(got - ref) - np.abs(ref) * 2.0 ** -11).max())
 
 
 def make_ln_inputs(beamc, M, N, K, dtype, seed):
@@ -38,6 +47,8 @@ def check_ln(oracle, got_bits, ref32, dtype, what):
         # fp16 rounding alone is within 2e-3 only below 8.0; the inputs are chosen so that holds
         assert r["max_abs_ref"] < 8.0, f"{what}: |y| reaches {r['max_abs_ref']}"
         assert r["max_abs_err"] <= LN_TOL, f"{what}: {r['max_abs_err']:.4g} > {LN_TOL}"
+        own = f16_error_beyond_rounding(got_bits, ref32)
+        assert own <= LN_OWN_TOL, f"{what}: error beyond the output's rounding {own:.4g} > {LN_OWN_TOL}"
     else:
         assert r["max_bf16_excess"] <= LN_TOL, f"{what}: {r['max_bf16_excess']:.4g} > {LN_TOL}"
 
@@ -118,21 +129,88 @@ def test_ln_invariants(gpu, beamc, oracle):
 
 
 def test_ln_fused_timeout_is_reported_not_hung(gpu, beamc):
-    """With a zero poll budget every workgroup gives up waiting at once: the kernel still ends normally,
-    the flag is raised, and the next call with the normal budget is correct again."""
+    """Spin limit -1 makes every wait of the fused kernel give up at once, whatever has been published: the
+    kernel still ends normally, the flag is raised, the rows come out as NaN (not as plausible numbers), the
+    checking form of the call raises -- and the next call with the normal budget is correct again with no
+    reset in between."""
     M, N, K = 512, 4096, 256
     a, b, g_, bt = make_ln_inputs(beamc, M, N, K, F16, 26)
     good = run_ln(beamc, a, b, g_, bt, F16, mode=beamc.LN_FUSED)
+    da, db = beamc.DeviceArray.from_numpy(a), beamc.DeviceArray.from_numpy(b)
+    dg, dbt = beamc.DeviceArray.from_numpy(g_), beamc.DeviceArray.from_numpy(bt)
+    y = beamc.DeviceArray((M, N))
     try:
-        assert beamc.lib.beam_set_ln_spin_limit(0) == 0
-        da, db = beamc.DeviceArray.from_numpy(a), beamc.DeviceArray.from_numpy(b)
-        dg, dbt = beamc.DeviceArray.from_numpy(g_), beamc.DeviceArray.from_numpy(bt)
-        y = beamc.DeviceArray((M, N))
+        assert beamc.lib.beam_set_ln_spin_limit(-1) == 0
         beamc.gemmrc_ln(da, db, y, dg, dbt, mode=beamc.LN_FUSED)
         beamc.sync()
         assert beamc.gemmrc_ln_timed_out()
+        assert np.isnan(y.to_numpy().view(np.float16)).all()
+        with pytest.raises(beamc.BeamError):
+            beamc.gemmrc_ln(da, db, y, dg, dbt, mode=beamc.LN_FUSED, check=True)
     finally:
         beamc.lib.beam_set_ln_spin_limit(4 << 20)
-    beamc.lib.beam_gemmrc_ln_workspace_reset(beamc._ln_workspace.ptr)
-    again = run_ln(beamc, a, b, g_, bt, F16, mode=beamc.LN_FUSED)
-    assert (again == good).all()
+    beamc.gemmrc_ln(da, db, y, dg, dbt, mode=beamc.LN_FUSED, check=True)  # the flag was cleared by this call
+    assert (y.to_numpy() == good).all()
+    for x in (da, db, dg, dbt, y):
+        x.free()
+
+
+def _ln_ex(beamc, da, db, dg, dbt, y, M, N, K, dtype, ws, mode):
+    import ctypes
+    rc = beamc.lib.beam_gemmrc_ln_ex(da.ptr, db.ptr, dg.ptr, dbt.ptr, ctypes.c_float(1e-5), y.ptr, M, N, K, dtype, None, mode,
+                                     ws.ptr, ws.nbytes, None)
+    assert rc == 0, beamc.lib.beam_last_error().decode()
+
+
+def test_ln_fused_workspace_describes_itself(gpu, beamc, oracle):
+    """The fused kernel's workspace carries its own state: a buffer freed and handed out again, overwritten
+    with bytes that read as published statistics (0x3f...: sign bit clear), or used for another shape before,
+    needs no reset call -- the launch notices on the device and starts over."""
+    M, N, K = 768, 2048, 256
+    a, b, g_, bt = make_ln_inputs(beamc, M, N, K, F16, 31)
+    ref = oracle.gemmrc_ln(a, b, g_, bt, 1e-5, F16)
+    da, db = beamc.DeviceArray.from_numpy(a), beamc.DeviceArray.from_numpy(b)
+    dg, dbt = beamc.DeviceArray.from_numpy(g_), beamc.DeviceArray.from_numpy(bt)
+    y = beamc.DeviceArray((M, N))
+    need = beamc.lib.beam_gemmrc_ln_workspace_bytes_for(M, N, K, None, beamc.LN_FUSED)
+    assert need > 0
+
+    def launch_and_check(ws, what):
+        y.fill_bytes(0xEE)
+        _ln_ex(beamc, da, db, dg, dbt, y, M, N, K, F16, ws, beamc.LN_FUSED)
+        beamc.sync()
+        check_ln(oracle, y.to_numpy(), ref, F16, what)
+
+    ws = beamc.DeviceArray((need,), itemsize=1)
+    launch_and_check(ws, "fresh workspace")
+    launch_and_check(ws, "second launch on it")
+    ws.free()
+    ws = beamc.DeviceArray((need,), itemsize=1)  # usually the same address again
+    ws.fill_bytes(0x3F)
+    launch_and_check(ws, "re-allocated workspace full of 0x3f")
+    launch_and_check(ws, "launch after that")
+    # another shape on the same buffer in between (same bytes needed or fewer), then the first one again
+    M2, N2 = 512, 1024
+    a2, b2, g2, bt2 = make_ln_inputs(beamc, M2, N2, K, F16, 32)
+    ref2 = oracle.gemmrc_ln(a2, b2, g2, bt2, 1e-5, F16)
+    da2, db2 = beamc.DeviceArray.from_numpy(a2), beamc.DeviceArray.from_numpy(b2)
+    dg2, dbt2 = beamc.DeviceArray.from_numpy(g2), beamc.DeviceArray.from_numpy(bt2)
+    y2 = beamc.DeviceArray((M2, N2))
+    assert beamc.lib.beam_gemmrc_ln_workspace_bytes_for(M2, N2, K, None, beamc.LN_FUSED) <= need
+    _ln_ex(beamc, da2, db2, dg2, dbt2, y2, M2, N2, K, F16, ws, beamc.LN_FUSED)
+    beamc.sync()
+    check_ln(oracle, y2.to_numpy(), ref2, F16, "other shape on the same workspace")
+    launch_and_check(ws, "first shape again")
+    for x in (da, db, dg, dbt, y, da2, db2, dg2, dbt2, y2, ws):
+        x.free()
+
+
+def test_ln_default_call_never_lacks_workspace(gpu, beamc, oracle):
+    """M=1024, N=8192, K=2048 without a tile: the library's tile for that K takes the two-pass path (32 column
+    tiles of 256 fit the fused kernel, but the tile chosen is another); the Python wrapper sizes its buffer for
+    exactly that call."""
+    M, N, K = 1024, 8192, 2048
+    a, b, g_, bt = make_ln_inputs(beamc, M, N, K, F16, 33)
+    ref = oracle.gemmrc_ln(a, b, g_, bt, 1e-5, F16)
+    got = run_ln(beamc, a, b, g_, bt, F16)
+    check_ln(oracle, got, ref, F16, "default call 1024 x 8192 x 2048")

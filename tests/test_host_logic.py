@@ -271,3 +271,22 @@ def test_roofline_calculator():
     b, h, sq, d = 2, 24, 4096 + 333, 64
     assert R.attn_flops(b, h, sq, d) == 2 * (b * h * sq * d * sq + b * h * sq * sq * d) == 241041911808
     assert abs(R.attn_bound_ms(mi, "bf16", b, h, sq, d) - 241041911808 / 2516.6e12 * 1e3) < 1e-9
+
+
+def test_ln_workspace_query_covers_every_default_call(beamc):
+    """The size queries without K must cover whatever tile the library picks once it knows K (a call without a
+    tile): for every shape, query(M, N) >= exact need(M, N, K), and with a tile given the two agree."""
+    L = beamc.lib
+    for M in (64, 300, 1024, 4096, 16384):
+        for N in (40, 1000, 4096, 8192, 20000):
+            loose = L.beam_gemmrc_ln_workspace_bytes_ex(M, N, None, beamc.LN_AUTO)
+            assert loose == L.beam_gemmrc_ln_workspace_bytes(M, N, None)
+            for K in (8, 64, 200, 2048, 32768):
+                exact = L.beam_gemmrc_ln_workspace_bytes_for(M, N, K, None, beamc.LN_AUTO)
+                assert 0 < exact <= loose, (M, N, K, exact, loose)
+            for cfg in (beamc.TileConfig(128, 128, 64, 64), beamc.TileConfig(256, 256, 128, 64)):
+                import ctypes
+                c = cfg.to_c()
+                for mode in (beamc.LN_AUTO, beamc.LN_TWOPASS):
+                    assert L.beam_gemmrc_ln_workspace_bytes_ex(M, N, ctypes.byref(c), mode) == \
+                        L.beam_gemmrc_ln_workspace_bytes_for(M, N, 4096, ctypes.byref(c), mode)
