@@ -79,6 +79,9 @@ def _load() -> ctypes.CDLL:
     L.beam_splitk_workspace_bytes.restype = sz
     L.beam_gemmrc_splitk.argtypes = [vp, vp, vp, i, i, i, i, cfgp, i, vp, sz, vp]
     L.beam_splitk_effective.argtypes = [i, i, i, cfgp, i]
+    L.beam_splitk_noalloc_max_bytes.argtypes = []
+    L.beam_splitk_noalloc_max_bytes.restype = sz
+    L.beam_gemmrc_splitk_noalloc.argtypes = [vp, vp, vp, i, i, i, i, cfgp, i, vp]
     L.beam_gemmrc_ln_workspace_bytes.argtypes = [i, i, cfgp]
     L.beam_gemmrc_ln_workspace_bytes.restype = sz
     L.beam_gemmrc_ln.argtypes = [vp, vp, vp, vp, ctypes.c_float, vp, i, i, i, i, cfgp, vp, sz, vp]

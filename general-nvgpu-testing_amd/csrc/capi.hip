@@ -51,6 +51,37 @@ std::mutex g_dev_mu;
 // polls of statistics slots (about a microsecond each) before a thread of a fused LayerNorm workgroup gives up
 std::atomic<int> g_ln_spin_limit{4 << 20};
 
+// Split-K workspace of beam_gemmrc_splitk_noalloc: device memory that exists from the moment the library's
+// code is loaded on a GPU until the process ends, so the entry point never allocates.  In host code the
+// array's name is only a handle for hipGetSymbolAddress; what kernels and copies get is the per-device
+// address looked up below (every GPU has its own copy at its own address).
+constexpr size_t kScratchBytes = (size_t)16 << 20;
+constexpr int kMaxDevices = 64;
+void* g_scratch_ptr[kMaxDevices] = {};
+std::mutex g_scratch_mu;
+
+}  // namespace
+
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+
+namespace {
+
+// Address of `scratch` on the current device (looked up once per device, with that device current).
+int scratch_on_current_device(void** out) {
+  int dev = -1;
+  BEAM_HIP(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kMaxDevices) return fail(BEAM_ERR_UNSUPPORTED, "device index %d beyond %d", dev, kMaxDevices - 1);
+  std::lock_guard<std::mutex> lk(g_scratch_mu);
+  if (!g_scratch_ptr[dev]) {
+    void* ptr = nullptr;
+    BEAM_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+    if (!ptr) return fail(BEAM_ERR_HIP, "hipGetSymbolAddress returned a null address for the scratch array");
+    g_scratch_ptr[dev] = ptr;
+  }
+  *out = g_scratch_ptr[dev];
+  return BEAM_OK;
+}
+
 const std::vector<KernelSet>& kernel_sets() {
   static const std::vector<KernelSet> sets = [] {
     std::vector<KernelSet> v;
@@ -238,7 +269,8 @@ int beam_init(void) {
     return fail(BEAM_ERR_DEVICE, "device 0 is %s; this library holds gfx950 code only", prop.gcnArchName);
   }
   g_dev.status = BEAM_OK;
-  return BEAM_OK;
+  void* ignored;
+  return scratch_on_current_device(&ignored);  // the no-allocation entry point's memory, looked up at set-up
 }
 
 int beam_device_info(char* name, int len, int* compute_units, int* clock_khz, size_t* mem_bytes) {
@@ -566,6 +598,26 @@ int beam_gemmrc_splitk(const void* A, const void* B, void* C, int M, int N, int 
   BEAM_HIP(ks->launch[dtype][kEpiPartial][c.pipeline](p, dim3((unsigned)(p.tiles_m * p.tiles_n * s), 1, 1), st));
   BEAM_HIP(launch_splitk_reduce((const float*)ws, C, (size_t)M * N, s, dtype, st));
   return BEAM_OK;
+}
+
+size_t beam_splitk_noalloc_max_bytes(void) { return kScratchBytes; }
+
+int beam_gemmrc_splitk_noalloc(const void* A, const void* B, void* C, int M, int N, int K, int dtype,
+                               const beam_tile_cfg* cfg, int split_k, void* stream) {
+  int rc = beam_init();
+  if (rc) return rc;
+  if (M > 0 && N > 0 && K > 0) {
+    const int s = beam_splitk_effective(M, N, K, cfg, split_k);
+    if (s < 0) return BEAM_ERR_UNSUPPORTED;  // the message is already set
+    const size_t need = s > 1 ? beam_splitk_workspace_bytes(M, N, s) : 0;
+    if (need > kScratchBytes)
+      return fail(BEAM_ERR_WORKSPACE, "split-K of %d x %d in %d slices needs %zu bytes; the built-in workspace of the "
+                  "no-allocation entry point holds %zu (use beam_gemmrc_splitk with a workspace of your own)", M, N, s, need,
+                  kScratchBytes);
+  }
+  void* ws = nullptr;
+  if ((rc = scratch_on_current_device(&ws))) return rc;
+  return beam_gemmrc_splitk(A, B, C, M, N, K, dtype, cfg, split_k, ws, kScratchBytes, stream);
 }
 
 // Fused GEMM+LayerNorm workspace: [header, 256 bytes | statistics set 0 | statistics set 1].  The header

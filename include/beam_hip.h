@@ -105,6 +105,16 @@ int beam_gemmrc_splitk(const void* A, const void* B, void* C, int M, int N, int 
                        void* stream);
 /* The effective split factor beam_gemmrc_splitk would use for these arguments. */
 int beam_splitk_effective(int M, int N, int K, const beam_tile_cfg* cfg, int split_k);
+/* beam_gemmrc_splitk without a workspace argument and without any allocation: the fp32 partial sums go
+ * into device memory built into the library (a fixed array of beam_splitk_noalloc_max_bytes() = 16 MiB
+ * per GPU, present from the first call into the library until the process ends).  No counterpart in
+ * the reference; it is for callers that cannot allocate: code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc.  Same results as beam_gemmrc_splitk, bit for bit.
+ * split_k * M * N * 4 bytes beyond the array's size -> BEAM_ERR_WORKSPACE.  All calls on one GPU share
+ * the array: calls that overlap in time on one GPU (different streams) race; order them. */
+size_t beam_splitk_noalloc_max_bytes(void);
+int beam_gemmrc_splitk_noalloc(const void* A, const void* B, void* C, int M, int N, int K, int dtype,
+                               const beam_tile_cfg* cfg, int split_k, void* stream);
 
 /* ---- fused GEMM + LayerNorm --------------------------------------------------------------- */
 
