@@ -759,6 +759,14 @@ int beam_gemmrc_ln_ex(const void* A, const void* B, const void* gamma, const voi
     } else {
       grid = (unsigned)band_block_grid(p.tiles_m, p.group_m, p.group_n);
     }
+    // The 256 x 256 tile runs on the kernel of gemm_w4.h where that one's preconditions hold (asked for by
+    // name, or as the library's own choice).
+    const bool w4_fits = c.pipeline == 0 && c.block_m == 256 && c.block_n == 256 && K % kBK == 0 && K >= kW4MinK && N % 8 == 0 &&
+                         N <= (1 << 21) && (((uintptr_t)Y | (uintptr_t)gamma | (uintptr_t)beta) & 15) == 0;
+    if (w4_fits && (!cfg || (c.wave_m == 128 && c.wave_n == 128))) {
+      BEAM_HIP(launch_gemm_w4_ln(p, dtype, dim3(grid, 1, 1), st));
+      return BEAM_OK;
+    }
     BEAM_HIP(ks->launch[dtype][kEpiLnFused][c.pipeline](p, dim3(grid, 1, 1), st));
     return BEAM_OK;
   }

@@ -4,9 +4,9 @@
 
 namespace beam {
 
-template <typename T, bool C_NT>
+template <typename T, bool C_NT, bool LN = false>
 static hipError_t launch_w4_t(const GemmParams& p, dim3 grid, hipStream_t stream) {
-  auto kern = gemmrc_w4_kernel<T, C_NT>;
+  auto kern = gemmrc_w4_kernel<T, C_NT, LN>;
   static bool configured = false;  // benign race: the attribute call is idempotent
   if (!configured) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -21,6 +21,10 @@ static hipError_t launch_w4_t(const GemmParams& p, dim3 grid, hipStream_t stream
 hipError_t launch_gemm_w4(const GemmParams& p, int dtype, dim3 grid, hipStream_t stream) {
   if (p.c_streaming) return dtype == BEAM_BF16 ? launch_w4_t<__bf16, true>(p, grid, stream) : launch_w4_t<_Float16, true>(p, grid, stream);
   return dtype == BEAM_BF16 ? launch_w4_t<__bf16, false>(p, grid, stream) : launch_w4_t<_Float16, false>(p, grid, stream);
+}
+
+hipError_t launch_gemm_w4_ln(const GemmParams& p, int dtype, dim3 grid, hipStream_t stream) {
+  return dtype == BEAM_BF16 ? launch_w4_t<__bf16, false, true>(p, grid, stream) : launch_w4_t<_Float16, false, true>(p, grid, stream);
 }
 
 }  // namespace beam

@@ -124,7 +124,10 @@ __host__ __device__ inline int w4_b_row(int b, int r) { return 32 * (b >> 1) + 4
 // four issue: loads issued faster than that stall the wavefront, and with it its MFMAs, at issue.
 // C_NT: C is stored non-temporal (an output larger than the last-level cache: its lines then do not push
 // operand panels out of the caches).
-template <typename T, bool C_NT = false, int SB = 4, int SA = 8, int G0 = 2>
+// LN: the fused GEMM+LayerNorm of gemm_kernel.h (kEpiLnFused) with this K loop: one output tile per
+// workgroup in the band order of tile_map.h, and after the K loop the same exchange of per-row (mean, M2)
+// pairs between the column tiles of a row band, normalisation in registers, Y stored once.
+template <typename T, bool C_NT = false, bool LN = false, int SB = 4, int SA = 8, int G0 = 2>
 struct GemmW4 {
   using Traits = ElemTraits<T>;
   using vec8 = typename Traits::vec8;
@@ -172,7 +175,13 @@ struct GemmW4 {
     const int n_k = K / kBK;
     const int total_tiles = p.tiles_m * p.tiles_n;
     const int first_tile = blockIdx.x, tile_step = gridDim.x;
-    const int my_tiles = (total_tiles - first_tile + tile_step - 1) / tile_step;
+    TileCoord ln_tile{0, 0};
+    if constexpr (LN) {
+      ln_tile = p.group_n > 0 ? band_block_tile(blockIdx.x, p.tiles_m, p.tiles_n, p.group_m, p.group_n)
+                              : band_xcd_tile(blockIdx.x, p.tiles_m, p.tiles_n, p.group_m);
+      if (ln_tile.tm < 0) return;  // the band grids are padded
+    }
+    const int my_tiles = LN ? 1 : (total_tiles - first_tile + tile_step - 1) / tile_step;
     const int g_total = my_tiles * n_k;  // K tiles this workgroup multiplies
 
     // ---- global -> LDS -----------------------------------------------------------------------
@@ -192,7 +201,10 @@ struct GemmW4 {
 
     // Operand rows of the workgroup's j-th output tile as (address, bytes) of a buffer descriptor; empty
     // past its last tile: such loads are issued and counted like any other and touch no memory.
-    auto tile_coord = [&](int j) { return tile_of_workgroup(first_tile + j * tile_step, p.tiles_m, p.tiles_n, p.group_m); };
+    auto tile_coord = [&](int j) {
+      if constexpr (LN) return ln_tile;
+      else return tile_of_workgroup(first_tile + j * tile_step, p.tiles_m, p.tiles_n, p.group_m);
+    };
     auto rows_of_a = [&](int j, TileCoord tc) {
       if (j >= my_tiles) return make_rsrc(p.A, 0u);
       const int row0 = tc.tm * BM;
@@ -372,7 +384,7 @@ struct GemmW4 {
         if constexpr (half == 1 && m == LAST_READ + 1) rd_a = rd_a + SLOT == B_REGION ? 0 : rd_a + SLOT;
         if constexpr (half == 1 && m == LAST_READ + 2) rd_b = rd_b + SLOT == LDS_BYTES ? B_REGION : rd_b + SLOT;
         if constexpr (half == 1 && m > LAST_A && m <= LAST_A + 3) advance(ld_a, wrap_a, next_a, 0, B_REGION, m - LAST_A - 1);
-        if constexpr (FIRST && gap >= 10 && gap < 10 + 8 * FM && ((gap - 10) & 1) == 0) {
+        if constexpr (FIRST && !LN && gap >= 10 && gap < 10 + 8 * FM && ((gap - 10) & 1) == 0) {
           // pair q of row block i goes into gap 10 + 8 i + 2 q
           store_pair(std::integral_constant<int, (gap - 10) / 8>{}, std::integral_constant<int, ((gap - 10) / 2) % 4>{});
         }
@@ -419,18 +431,200 @@ struct GemmW4 {
         Mfma::template fma<m>(fb1[m & 7], fa1[m >> 3]);
       });
       asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
-      w4_static_for<0, FM * FN / 2>([&](auto o_tag) __attribute__((always_inline)) {
-        constexpr int o = decltype(o_tag)::value;
-        store_pair(std::integral_constant<int, o / 4>{}, std::integral_constant<int, o % 4>{});
-      });
+      if constexpr (!LN) {
+        w4_static_for<0, FM * FN / 2>([&](auto o_tag) __attribute__((always_inline)) {
+          constexpr int o = decltype(o_tag)::value;
+          store_pair(std::integral_constant<int, o / 4>{}, std::integral_constant<int, o % 4>{});
+        });
+      } else {
+        layer_norm_epilogue(p, smem, ln_tile, out);
+      }
     }
+  }
+
+  // ---- LayerNorm over the row band (LN) -------------------------------------------------------------
+  // The same five steps as the kEpiLnFused epilogue of gemm_kernel.h, for this kernel's accumulator layout:
+  // row block i of a lane is 32 values (blocks 8 i .. 8 i + 7) of row 128 wm + 16 i + r, in the four groups of
+  // 8 columns 128 wn + 32 q + 8 g; a row of the tile is spread over 4 lane groups x 2 wavefronts = 8 slots.
+  template <typename OutTileT>
+  static __device__ __forceinline__ void layer_norm_epilogue(const GemmParams& p, char* smem, TileCoord tc, const OutTileT& out) {
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave & 1, wn = wave >> 1;
+    const int r = lane & 15, g = lane >> 4;
+    const int N = p.N;
+    const int col0 = tc.tn * BN;
+    constexpr int SLOTS = 8, PITCH = SLOTS + 1;  // (a row of `part` is padded by one pair: see gemm_kernel.h)
+    // gamma / beta of this lane's four column groups: issued now, used in step 5
+    bool q_valid[4];
+    vec8 gv[4], bv[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int n = col0 + wn * 128 + 32 * q + 8 * g;
+      q_valid[q] = n < N;  // N is a multiple of 8: a group of 8 columns exists whole or not at all
+      gv[q] = *(const vec8*)((const T*)p.gamma + (q_valid[q] ? n : 0));
+      bv[q] = *(const vec8*)((const T*)p.beta + (q_valid[q] ? n : 0));
+    }
+    const int my_cols = 8 * ((int)q_valid[0] + (int)q_valid[1] + (int)q_valid[2] + (int)q_valid[3]);
+    const bool full = col0 + BN <= N;
+    __syncthreads();  // every wavefront is done with the operand slots: LDS is free
+    float* red = (float*)smem;   // [BM][2] tile statistics, later (mean, rstd) of the whole row
+    float* part = red + BM * 2;  // [BM][PITCH][2], later the gathered pairs of the band [tiles_n][BM][2]
+    // 1. per-lane (mean, M2) over the lane's columns of each of its rows, dropped into LDS
+    w4_static_for<0, FM>([&](auto i_tag) __attribute__((always_inline)) {
+      constexpr int i = decltype(i_tag)::value;
+      float x[32];
+      w4_static_for<0, 32>([&](auto t_tag) __attribute__((always_inline)) {
+        constexpr int t = decltype(t_tag)::value;
+        x[t] = w4_acc_read<4 * (8 * i) + t>();  // block 8 i + t / 4, element t % 4
+      });
+      float sum = 0.0f, m2 = 0.0f;
+#pragma unroll
+      for (int t = 0; t < 32; ++t) sum += (full || q_valid[t >> 3]) ? x[t] : 0.0f;
+      const float mean = full ? sum * (1.0f / 32.0f) : (my_cols > 0 ? sum / (float)my_cols : 0.0f);
+#pragma unroll
+      for (int t = 0; t < 32; ++t) {
+        const float d = x[t] - mean;
+        m2 += (full || q_valid[t >> 3]) ? d * d : 0.0f;
+      }
+      const int rl = wm * 128 + 16 * i + r;
+      part[(rl * PITCH + wn * 4 + g) * 2 + 0] = mean;
+      part[(rl * PITCH + wn * 4 + g) * 2 + 1] = m2;
+    });
+    __syncthreads();
+    // 2. one thread per row merges the 8 slots in a fixed order (Chan's update) ...
+    {
+      const int rl = tid;  // 256 threads, 256 rows
+      float mean = 0.0f, m2 = 0.0f, n_acc = 0.0f;
+      if (full) {
+        // every slot covers 32 columns: the mean of the slot means, then M2 about it -- the merge below for
+        // equal counts, in the same fixed order, without its divisions
+        float mw[SLOTS], qw[SLOTS];
+#pragma unroll
+        for (int slot = 0; slot < SLOTS; ++slot) {
+          mw[slot] = part[(rl * PITCH + slot) * 2 + 0];
+          qw[slot] = part[(rl * PITCH + slot) * 2 + 1];
+          mean += mw[slot];
+        }
+        mean *= 1.0f / (float)SLOTS;
+#pragma unroll
+        for (int slot = 0; slot < SLOTS; ++slot) {
+          const float d = mw[slot] - mean;
+          m2 += qw[slot] + 32.0f * d * d;
+        }
+      }
+#pragma unroll
+      for (int slot = 0; slot < (full ? 0 : SLOTS); ++slot) {
+        int cnt = 0;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) cnt += (col0 + (slot >> 2) * 128 + 32 * q + 8 * (slot & 3) < N) ? 8 : 0;
+        if (cnt == 0) continue;
+        const float mw = part[(rl * PITCH + slot) * 2 + 0];
+        const float qw = part[(rl * PITCH + slot) * 2 + 1];
+        const float nb = (float)cnt;
+        const float tot = n_acc + nb;
+        const float delta = mw - mean;
+        mean += delta * (nb / tot);
+        m2 += qw + delta * delta * (n_acc * nb / tot);
+        n_acc = tot;
+      }
+      // ... and publishes the tile's pair: one 8-byte device-scope atomic store; a slot whose M2 is negative
+      // has not been published (see gemm_kernel.h for why this needs no cache-wide fence)
+      const bool odd_epoch = (p.timeout_flag[kLnHdrEpoch] & 1) != 0;
+      float* const cur_set = odd_epoch ? p.next_stats : p.stats;
+      float* const other_set = odd_epoch ? p.stats : p.next_stats;
+      const size_t my_slot = ((size_t)tc.tm * p.tiles_n + tc.tn) * BM;
+      m2 = fmaxf(m2, 0.0f);
+      const unsigned long long pair = (unsigned long long)__float_as_uint(mean) | ((unsigned long long)__float_as_uint(m2) << 32);
+      __hip_atomic_store((unsigned long long*)cur_set + my_slot + rl, pair, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const unsigned long long unpublished = (unsigned long long)__float_as_uint(-1.0f) << 32;
+      __hip_atomic_store((unsigned long long*)other_set + my_slot + rl, unpublished, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __syncthreads();  // `part` is free again
+      // 3. gather the band's pairs into LDS, polling (boundedly) what is not published yet
+      float* gathered = part;
+      const unsigned long long* band_stats = (const unsigned long long*)cur_set + (size_t)tc.tm * p.tiles_n * BM;
+      const int n_slots = p.tiles_n * BM;
+      int polls = 0;
+      for (int q0 = tid; q0 < n_slots; q0 += 8 * NT) {
+        unsigned long long v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          const int q = q0 + u * NT;
+          v[u] = __hip_atomic_load(band_stats + (q < n_slots ? q : q0), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          const int q = q0 + u * NT;
+          if (q >= n_slots) break;
+          while ((long long)v[u] < 0 || p.spin_limit < 0) {
+            if (++polls > p.spin_limit) {
+              p.timeout_flag[kLnHdrTimeout] = 1;
+              v[u] = 0x7fc000007fc00000ull;
+              break;
+            }
+            __builtin_amdgcn_s_sleep(4);
+            v[u] = __hip_atomic_load(band_stats + q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          }
+          ((unsigned long long*)gathered)[q] = v[u];
+        }
+      }
+      __syncthreads();
+      // 4. merge in tile order -> (mean, rstd) of the whole row
+      mean = 0.0f;
+      m2 = 0.0f;
+      n_acc = 0.0f;
+      const bool even_tiles = (N % BN) == 0;  // every column tile is full: equal weights
+      if (even_tiles) {
+        for (int t = 0; t < p.tiles_n; ++t) mean += gathered[((size_t)t * BM + rl) * 2 + 0];
+        mean *= 1.0f / (float)p.tiles_n;
+        for (int t = 0; t < p.tiles_n; ++t) {
+          const float d = gathered[((size_t)t * BM + rl) * 2 + 0] - mean;
+          m2 += gathered[((size_t)t * BM + rl) * 2 + 1] + (float)BN * d * d;
+        }
+      }
+      for (int t = 0; t < (even_tiles ? 0 : p.tiles_n); ++t) {
+        int cw = N - t * BN;
+        cw = cw > BN ? BN : cw;
+        const float mw = gathered[((size_t)t * BM + rl) * 2 + 0];
+        const float qw = gathered[((size_t)t * BM + rl) * 2 + 1];
+        const float nb = (float)cw;
+        const float tot = n_acc + nb;
+        const float delta = mw - mean;
+        mean += delta * (nb / tot);
+        m2 += qw + delta * delta * (n_acc * nb / tot);
+        n_acc = tot;
+      }
+      red[rl * 2 + 0] = mean;
+      red[rl * 2 + 1] = even_tiles ? __builtin_amdgcn_rsqf(m2 * (1.0f / (float)N) + p.eps) : 1.0f / sqrtf(m2 / (float)N + p.eps);
+    }
+    __syncthreads();
+    // 5. normalise the accumulators and store Y: a pair of blocks is one 16-byte store per lane
+    w4_static_for<0, FM>([&](auto i_tag) __attribute__((always_inline)) {
+      constexpr int i = decltype(i_tag)::value;
+      const int rl = wm * 128 + 16 * i + r;
+      const float mean = red[rl * 2 + 0], rstd = red[rl * 2 + 1];
+      const int skip = i * 16 * N * 2;
+      const int left = out.bytes - skip;
+      const __amdgpu_buffer_rsrc_t rsrc = make_rsrc(out.base + skip, left > 0 ? (unsigned)left : 0u);
+      w4_static_for<0, 4>([&](auto q_tag) __attribute__((always_inline)) {
+        constexpr int q = decltype(q_tag)::value;
+        vec8 v;
+        w4_static_for<0, 8>([&](auto e_tag) __attribute__((always_inline)) {
+          constexpr int e = decltype(e_tag)::value;
+          v[e] = (T)((w4_acc_read<4 * (8 * i + 2 * q) + e>() - mean) * rstd * (float)gv[q][e] + (float)bv[q][e]);
+        });
+        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(i32x4, v), rsrc, (int)out.voff[q], 0, 0);
+      });
+    });
+    // One more workgroup has published its statistics and marked its slots of the other set.
+    if (tid == 0) __hip_atomic_fetch_add(p.timeout_flag + kLnHdrDone, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
 };
 
-template <typename T, bool C_NT = false, int SB = 4, int SA = 8, int G0 = 2>
+template <typename T, bool C_NT = false, bool LN = false, int SB = 4, int SA = 8, int G0 = 2>
 __global__ void __launch_bounds__(256) gemmrc_w4_kernel(const GemmParams p) {
   extern __shared__ __attribute__((aligned(1024))) char smem[];
-  GemmW4<T, C_NT, SB, SA, G0>::run(p, smem);
+  GemmW4<T, C_NT, LN, SB, SA, G0>::run(p, smem);
 }
 
 }  // namespace beam

@@ -54,14 +54,16 @@ def check_ln(oracle, got_bits, ref32, dtype, what):
 
 
 @pytest.mark.parametrize("shape", [(256, 512, 256), (1024, 1024, 512), (300, 1000, 200), (64, 4096, 128),
-                                   (17, 40, 64), (16384, 2048, 128), (4200, 1000, 72)])
+                                   (17, 40, 64), (16384, 2048, 128), (4200, 1000, 72), (300, 1000, 256), (700, 1304, 192)])
 def test_ln_small(gpu, beamc, oracle, shape):
     M, N, K = shape
     for dtype in (F16, BF16):
         a, b, g, bt = make_ln_inputs(beamc, M, N, K, dtype, 21)
         ref = oracle.gemmrc_ln(a, b, g, bt, 1e-5, dtype)
+        # (256 x 256 / 128 x 128 is the 4-wavefront kernel where K is a multiple of 64 from 192 on, the
+        # 8-wavefront family's tile of that shape elsewhere)
         for cfg in [None, beamc.TileConfig(128, 128, 64, 64), beamc.TileConfig(64, 64, 32, 32),
-                    beamc.TileConfig(256, 256, 128, 64)]:
+                    beamc.TileConfig(256, 256, 128, 64), beamc.TileConfig(256, 256, 128, 128)]:
             for mode in (beamc.LN_TWOPASS, beamc.LN_FUSED):
                 got = run_ln(beamc, a, b, g, bt, dtype, config=cfg, mode=mode)
                 check_ln(oracle, got, ref, dtype, f"{shape} dtype {dtype} {cfg.name if cfg else 'default'} mode {mode}")
