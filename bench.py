@@ -7,9 +7,11 @@ A step is one gemmrc launch (C = A . B^T, fp32 accumulation, fp16 output) on inp
 resident in HBM (N(0,1)/sqrt(K) values from the seeded host generator).  One JSON line is
 printed: whole-job TFLOP/s, the MFMA roofline fraction of the kernel measured with HIP events on
 the launch stream, and the CPU oracle timed on this host's cores beside it (a reported baseline,
-also used to check the GPU result of the timed run).  `extra` carries the two companion targets:
-split-K at 256x256x32768 (us, against the best non-split tile) and fused GEMM+LayerNorm at 4096^3
-(against the plain GEMM).
+also used to check the GPU result of the timed run).  `value` is what the --warmup / --steps asked for
+give (after idle the first ~50 launches run on a clock that is still settling); `extra.headline_steady`
+is the same kernel once it has settled.  `extra` also carries the two companion targets, split-K at
+256x256x32768 (us, against the best non-split tile) and fused GEMM+LayerNorm at 4096^3 (against the plain
+GEMM), and the shape/dtype sweep.
 """
 import argparse
 import json
@@ -25,10 +27,24 @@ METRIC = "fp16 GEMM TFLOP/s + % MFMA peak at 8192^3; split-K µs at 256x256x3276
 # published as 2.5 PFLOP/s.
 PEAK_TFLOPS = 2500.0
 HBM_PEAK_GBS = 8000.0
-# HBM/fabric bytes per launch of the headline kernel, from the counter runs summarised in
-# profiles/gemmrc_256x256_fp16_8192cube.txt (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000, the factors of
-# profiles/copy_256MiB_counter_calibration.txt).  Counters cannot be read from inside this script.
-PROFILED_TRAFFIC_BYTES = 1.749e9
+# HBM/fabric bytes per launch of the headline kernel come from counter runs (FETCH_SIZE, WRITE_SIZE, scaled by
+# what the same counters read for a copy of known size); counters cannot be read from inside this script, so
+# the figure is taken from the committed summary of those runs, whose "traffic =" line names it.
+HEADLINE_PROFILE = os.path.join(ROOT, "profiles", "gemmrc_256x256_fp16_8192cube.txt")
+
+
+def profiled_traffic_bytes():
+    """Bytes per launch from the "traffic = <number> MB per launch" line of the headline profile, or None."""
+    import re
+    try:
+        with open(HEADLINE_PROFILE) as f:
+            for line in f:
+                m = re.search(r"traffic\s*=\s*([0-9.]+)\s*MB per launch", line)
+                if m:
+                    return float(m.group(1)) * 1e6
+    except OSError:
+        pass
+    return None
 
 
 def time_region(_C, fn, steps):
@@ -112,6 +128,24 @@ def splitk_graph_us(_C, a, b, c, cfg, s, calls=50, replays=10, operand_sets=1):
         a2.free()
         b2.free()
     return ms.value * 1e3 / (calls * replays)
+
+
+def extra_splitk_small(_C):
+    """The second split-K shape of the configuration list, 64 x 128 x 65536, as the library runs it when left
+    the choice, against the library's tile without a split."""
+    M, N, K = 64, 128, 65536
+    a = _C.DeviceArray.from_numpy(_C.host_uniform((M, K), _C.F16, 12, 0))
+    b = _C.DeviceArray.from_numpy(_C.host_uniform((N, K), _C.F16, 12, 1))
+    c = _C.DeviceArray((M, N))
+    cfg, s = _C.default_config(M, N, K, split=True)
+    split_ms = min(_C.bench(1, a, b, c, config=None, split_k=0, warmup=20, iters=100) for _ in range(2))
+    plain_ms = min(_C.bench(0, a, b, c, config=None, warmup=5, iters=20) for _ in range(2))
+    for x in (a, b, c):
+        x.free()
+    bytes_alg = 2.0 * (M * K + N * K + M * N)
+    return {"shape": [M, N, K], "splitk_us": round(split_ms * 1e3, 2), "config": f"{cfg.name},S={s}",
+            "nonsplit_us": round(plain_ms * 1e3, 2), "speedup": round(plain_ms / split_ms, 2),
+            "hbm_GBs": round(bytes_alg / (split_ms * 1e-3) / 1e9, 1)}
 
 
 def extra_splitk(_C):
@@ -200,20 +234,26 @@ def extra_nn(_C):
     return {"shape": [M, N, K], "us": round(ms * 1e3, 1), "TFLOPs": round(2.0 * M * N * K / (ms * 1e-3) / 1e12, 1)}
 
 
-def extra_shapes(_C):
-    """A few shapes of the sweep with the tile the library picks for them."""
+def extra_sweep(_C):
+    """The shape/dtype sweep of the configuration list with the tile the library picks: squares 512 ... 16384,
+    the two LLM shapes and the ragged 3000 x 5000 x 2000, fp16 and bf16 (uniform[-1, 1) values), plus a few
+    squares between the powers of two in fp16."""
+    shapes = [(512, 512, 512), (1024, 1024, 1024), (2048, 2048, 2048), (4096, 4096, 4096), (16384, 16384, 16384),
+              (4096, 11008, 4096), (4096, 4096, 11008), (3000, 5000, 2000)]
+    more_fp16 = [(3072, 3072, 3072), (6144, 6144, 6144), (7168, 7168, 7168), (16384, 16384, 2048)]
     out = []
-    for (M, N, K) in [(2048, 2048, 2048), (3072, 3072, 3072), (4096, 4096, 4096), (6144, 6144, 6144), (7168, 7168, 7168),
-                      (4096, 11008, 4096), (4096, 4096, 11008), (16384, 16384, 2048)]:
-        a = _C.DeviceArray.from_numpy(_C.host_normal((M, K), _C.F16, 5, 0, 0.0, K ** -0.5))
-        b = _C.DeviceArray.from_numpy(_C.host_normal((N, K), _C.F16, 5, 1, 0.0, K ** -0.5))
-        c = _C.DeviceArray((M, N))
-        cfg, _ = _C.default_config(M, N, K, split=False)
-        ms = min(_C.bench(_C.OP_GEMM, a, b, c, warmup=50, iters=100) for _ in range(2))
-        for t in (a, b, c):
-            t.free()
-        out.append({"shape": [M, N, K], "tile": cfg.name, "us": round(ms * 1e3, 1),
-                    "TFLOPs": round(2.0 * M * N * K / (ms * 1e-3) / 1e12, 1)})
+    for dtype, name, todo in ((_C.F16, "fp16", shapes + more_fp16), (_C.BF16, "bf16", shapes)):
+        for (M, N, K) in todo:
+            a = _C.DeviceArray.from_numpy(_C.host_uniform((M, K), dtype, 5, 0), dtype)
+            b = _C.DeviceArray.from_numpy(_C.host_uniform((N, K), dtype, 5, 1), dtype)
+            c = _C.DeviceArray((M, N), dtype)
+            cfg, _ = _C.default_config(M, N, K, split=False)
+            big = 2.0 * M * N * K > 2e12
+            ms = min(_C.bench(_C.OP_GEMM, a, b, c, warmup=10 if big else 50, iters=20 if big else 100) for _ in range(2))
+            for t in (a, b, c):
+                t.free()
+            out.append({"shape": [M, N, K], "dtype": name, "tile": cfg.name, "us": round(ms * 1e3, 1),
+                        "TFLOPs": round(2.0 * M * N * K / (ms * 1e-3) / 1e12, 1)})
     return out
 
 
@@ -265,6 +305,20 @@ def main():
     value = flops * args.steps / wall / 1e12
     kern_ms = ev_ms / args.steps
     achieved = flops / (kern_ms * 1e-3) / 1e12
+    # The same kernel once the clock has settled, whatever --warmup and --steps were: launches until two
+    # successive batches of 50 agree within 2% (at least 100 launches), then 200 timed.
+    settle_launches, prev = 0, None
+    while settle_launches < 1000:
+        _, batch_ms = time_region(_C, step, 50)
+        settle_launches += 50
+        if prev is not None and settle_launches >= 100 and abs(batch_ms - prev) <= 0.02 * prev:
+            break
+        prev = batch_ms
+    _, steady_ms = time_region(_C, step, 200)
+    steady_ms /= 200
+    steady = {"kernel_ms": round(steady_ms, 4), "TFLOPs": round(flops / (steady_ms * 1e-3) / 1e12, 1),
+              "frac": round(flops / (steady_ms * 1e-3) / 1e12 / PEAK_TFLOPS, 4), "launches_before": args.warmup + args.steps + settle_launches,
+              "timed_launches": 200}
 
     out = {
         "metric": METRIC, "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
@@ -274,7 +328,8 @@ def main():
                    "tile": cfg.name, "device": info["name"], "compute_units": info["compute_units"]},
         "pct_of_peak": round(100.0 * value / PEAK_TFLOPS, 2),
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(achieved / PEAK_TFLOPS, 4), "traffic": PROFILED_TRAFFIC_BYTES,
+                     "frac": round(achieved / PEAK_TFLOPS, 4), "traffic": profiled_traffic_bytes(),
+                     "traffic_source": "profiles/" + os.path.basename(HEADLINE_PROFILE) + " (rocprofv3 counter runs, not this run)",
                      "kernel_ms": round(kern_ms, 4)},
     }
     if not args.no_cpu:
@@ -287,8 +342,11 @@ def main():
     for x in (a, b, c):
         x.free()
     if not args.no_extra:
-        out["extra"] = {"splitk": extra_splitk(_C), "gemm_ln": extra_ln(_C), "gemm_silu": extra_silu(_C),
-                        "matmul_nn": extra_nn(_C), "gemm_bf16": extra_bf16(_C), "fp16_shapes": extra_shapes(_C)}
+        out["extra"] = {"headline_steady": steady, "splitk": extra_splitk(_C), "splitk_64x128x65536": extra_splitk_small(_C),
+                        "gemm_ln": extra_ln(_C), "gemm_silu": extra_silu(_C), "matmul_nn": extra_nn(_C),
+                        "gemm_bf16": extra_bf16(_C), "sweep": extra_sweep(_C)}
+    else:
+        out["extra"] = {"headline_steady": steady}
     print(json.dumps(out))
     if "check" in out and not out["check"]["ok"]:
         sys.exit("bench.py: GPU result outside the tolerance of the CPU oracle")

@@ -8,10 +8,17 @@ Counterpart of the reference's python/beam/tuner.py:19-137:
 * OperatorTuner enumerates candidates (plain tiles and split-K tiles x split factors), times
   each on fresh inputs and memoises (best_op, best_tflops) per problem.
 
-What differs, on purpose: the cache key carries the dtype and is persisted as JSON; inputs are
-seeded; a candidate whose output disagrees with the library's default kernel is discarded
-instead of trusted (the reference's only guard is the >1000 TFLOP/s filter, tuner.py:42-43);
-the search space is the library's gfx950 tile table and split factors {4, 8, 16, 32, 64}.
+What differs, on purpose: the cache key carries the dtype and the architecture and is persisted as JSON
+(a file written on another architecture or another CU count is ignored); inputs are seeded; a candidate
+whose output disagrees with the library's default kernel is discarded instead of trusted (the reference's
+only guard is the >1000 TFLOP/s filter, tuner.py:42-43); a problem on which every candidate fails is not
+cached; the search space is the library's gfx950 tile table x LDS pipeline depth {0: 3+2 slots, 1: 2+2,
+2: as many as fit} x raster group, and for split-K the tiles up to 128 x 128 x pipeline {0, 2} x split
+factors {4, 8, 16, 32, 64}.
+
+    python -m beam.tuner [--dtype fp16|bf16|both] [--cache FILE] M,N,K [M,N,K ...]
+
+tunes the shapes given and prints a table: winner and its TFLOP/s beside the library's default.
 """
 from __future__ import annotations
 
@@ -28,7 +35,17 @@ from . import _C
 # measurement artefact (a launch that failed or did nothing).
 PLAUSIBLE_TFLOPS = 2600.0
 SPLIT_FACTORS = (4, 8, 16, 32, 64)
+PIPELINES = (0, 1, 2)
+ARCH = "gfx950"  # the only architecture libbeam_hip.so holds code for
 _DTYPES = {"fp16": _C.F16, "bf16": _C.BF16}
+
+
+def _compute_units() -> Optional[int]:
+    """CU count of the device, None without one (the cache is then only matched on the architecture)."""
+    try:
+        return int(_C.device_info()["compute_units"])
+    except Exception:
+        return None
 
 
 def _callable_name(func) -> str:
@@ -119,14 +136,17 @@ class OperatorTuner:
     # -- candidate enumeration ------------------------------------------------------------
 
     def _get_gemm_specs(self) -> List[Operator]:
+        """Every compiled tile x LDS pipeline depth; the raster group is varied for the standard depth
+        only (it matters for problems of many tiles, which is where that depth is the one to use)."""
         ret = []
         for cfg in _C.list_configs():
-            for group_m in (2, 4, 8, 16):
-                full = _C.TileConfig(cfg.block_m, cfg.block_n, cfg.wave_m, cfg.wave_n, 0, group_m)
-                ret.append(Operator(
-                    partial(_C.gemmrc_spec, shape_threadblock=[cfg.block_m, cfg.block_n],
-                            shape_warp=[cfg.wave_m, cfg.wave_n], group_m=group_m),
-                    native={"op": 0, "config": full}, name=f"gemmrc_spec[{full.name}]"))
+            for pipeline in PIPELINES:
+                for group_m in ((2, 4, 8, 16) if pipeline == 0 else (0,)):
+                    full = _C.TileConfig(cfg.block_m, cfg.block_n, cfg.wave_m, cfg.wave_n, pipeline, group_m)
+                    ret.append(Operator(
+                        partial(_C.gemmrc_spec, shape_threadblock=[cfg.block_m, cfg.block_n],
+                                shape_warp=[cfg.wave_m, cfg.wave_n], pipeline=pipeline, group_m=group_m),
+                        native={"op": 0, "config": full}, name=f"gemmrc_spec[{full.name}]"))
         return ret
 
     def _get_gemm_splitk_specs(self) -> List[Operator]:
@@ -134,13 +154,14 @@ class OperatorTuner:
         for cfg in _C.list_configs():
             if cfg.block_m * cfg.block_n > 128 * 128:
                 continue  # split-K is for problems with few output tiles
-            deep = _C.TileConfig(cfg.block_m, cfg.block_n, cfg.wave_m, cfg.wave_n, 2, 0)
-            for s in SPLIT_FACTORS:
-                ret.append(Operator(
-                    partial(_C.gemmrc_splitk_spec, shape_threadblock=[cfg.block_m, cfg.block_n],
-                            shape_warp=[cfg.wave_m, cfg.wave_n], split_k_slices=s, pipeline=2),
-                    native={"op": 1, "config": deep, "split_k": s},
-                    name=f"gemmrc_splitk_spec[{deep.name},s{s}]"))
+            for pipeline in (0, 2):
+                tile = _C.TileConfig(cfg.block_m, cfg.block_n, cfg.wave_m, cfg.wave_n, pipeline, 0)
+                for s in SPLIT_FACTORS:
+                    ret.append(Operator(
+                        partial(_C.gemmrc_splitk_spec, shape_threadblock=[cfg.block_m, cfg.block_n],
+                                shape_warp=[cfg.wave_m, cfg.wave_n], split_k_slices=s, pipeline=pipeline),
+                        native={"op": 1, "config": tile, "split_k": s},
+                        name=f"gemmrc_splitk_spec[{tile.name},s{s}]"))
         return ret
 
     # -- cache -----------------------------------------------------------------------------
@@ -153,18 +174,26 @@ class OperatorTuner:
         return ret
 
     def _load(self, path: str) -> None:
+        """Entries of a cache file written on this architecture (and, where both are known, this CU count:
+        a partitioned device has other winners); anything else is ignored, not trusted."""
         with open(path) as f:
             blob = json.load(f)
+        if blob.get("arch") != ARCH:
+            return
+        cus = _compute_units()
+        if cus is not None and blob.get("compute_units") not in (None, cus):
+            return
         for key, (name, tflops) in blob.get("entries", {}).items():
             op = self._by_name.get(name)
-            if op is not None:
+            if op is not None and key.endswith(f",{ARCH},)"):
                 self.cache[key] = (op, float(tflops))
 
     def save(self, path: Optional[str] = None) -> None:
         path = path or self.cache_path
         if not path:
             return
-        blob = {"arch": "gfx950", "entries": {k: [str(op), t] for k, (op, t) in self.cache.items()}}
+        blob = {"arch": ARCH, "compute_units": _compute_units(),
+                "entries": {k: [str(op), t] for k, (op, t) in self.cache.items()}}
         tmp = path + ".tmp"
         with open(tmp, "w") as f:
             json.dump(blob, f, indent=1, sort_keys=True)
@@ -197,7 +226,7 @@ class OperatorTuner:
              verbose: bool = False) -> Tuple[Operator, float]:
         M, N, K = (int(x) for x in matmul_shape)
         d = _DTYPES[dtype]
-        hashval = self.get_hash("gemm", [M, N, K, dtype])
+        hashval = self.get_hash("gemm", [M, N, K, dtype, ARCH])
         if hashval in self.cache:
             return self.cache[hashval]
         a, b, c = self._make_inputs(M, N, K, d)
@@ -222,6 +251,40 @@ class OperatorTuner:
                 best_op, best_tflops = op, tflops
         for x in (a, b, c):
             x.free()
+        if best_op is None:  # nothing ran: say so, but do not remember it (the next call tries again)
+            return None, -1
         self.cache[hashval] = (best_op, best_tflops)
         self.save()
         return self.cache[hashval]
+
+
+def _main(argv: Sequence[str]) -> int:
+    import argparse
+    ap = argparse.ArgumentParser(prog="python -m beam.tuner", description="tune gemmrc shapes and print winner against default")
+    ap.add_argument("shapes", nargs="+", help="M,N,K")
+    ap.add_argument("--dtype", default="fp16", choices=["fp16", "bf16", "both"])
+    ap.add_argument("--cache", default=None)
+    ap.add_argument("--rep", type=int, default=20)
+    args = ap.parse_args(list(argv))
+    tuner = OperatorTuner(cache_path=args.cache, warmup=5, rep=args.rep)
+    default_op = tuner.gemm_ops[0]
+    print(f"{len(tuner.gemm_ops)} candidates")
+    print("| shape | dtype | tuned operator | tuned TFLOP/s | default tile | default TFLOP/s | tuned / default |")
+    print("|---|---|---|---|---|---|---|")
+    for text in args.shapes:
+        M, N, K = (int(x) for x in text.split(","))
+        for dtype in (("fp16", "bf16") if args.dtype == "both" else (args.dtype,)):
+            op, tf = tuner.tune((M, N, K), dtype=dtype)
+            a, b, c = tuner._make_inputs(M, N, K, _DTYPES[dtype])
+            base = max(default_op.get_performance(a, b, c, warmup=20, rep=max(args.rep, 50)) for _ in range(2))
+            again = max(op.get_performance(a, b, c, warmup=20, rep=max(args.rep, 50)) for _ in range(2)) if op else -1
+            for x in (a, b, c):
+                x.free()
+            cfg, _ = _C.default_config(M, N, K, split=False)
+            print(f"| {M}x{N}x{K} | {dtype} | {op} | {again:.1f} | {cfg.name} | {base:.1f} | {again / base:.3f} |", flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    import sys
+    sys.exit(_main(sys.argv[1:]))

@@ -143,14 +143,17 @@ int choose_default(int M, int N, int K, int split_req, beam_tile_cfg* cfg, int* 
 
 // split_req: -1 the caller cannot run K slices (no workspace); 0 it can, and leaves the number to
 // the library; > 0 it asks for that many.  The default tile is chosen for that situation.
+// w4_ok: the caller has a form of the 4-wavefront kernel (gemm_w4.h); for the others the library's own choice
+// of that tile means the 8-wavefront 256 x 256 tile.
 int resolve_cfg(const beam_tile_cfg* in, int M, int N, int K, beam_tile_cfg* out, const KernelSet** ks,
-                int split_req = -1) {
+                int split_req = -1, bool w4_ok = false) {
   if (in) {
     *out = *in;
   } else {
     int s;
     int rc = choose_default(M, N, K, split_req, out, &s);
     if (rc) return rc;
+    if (!w4_ok && out->block_m == 256 && out->block_n == 256 && out->wave_m == 128 && out->wave_n == 128) out->wave_n = 64;
   }
   if (out->pipeline < 0 || out->pipeline > 2) return fail(BEAM_ERR_UNSUPPORTED, "pipeline %d: 0 (3 A + 2 B LDS slots), 1 (2 + 2) or 2 (deep)", out->pipeline);
   if (out->group_m <= 0) out->group_m = default_group_m(out->block_m, out->block_n);
@@ -380,6 +383,14 @@ int choose_default(int M, int N, int K, int split_req, beam_tile_cfg* cfg, int* 
     }
   }
   *cfg = c;
+  // From one full round of workgroups on, the 256 x 256 tile runs as four wavefronts of 128 x 128 (the kernel of
+  // gemm_w4.h; 8192^3 fp16, same machine, in turn: 1490-1515 against 1455-1465 TFLOP/s) where that kernel's
+  // shape conditions hold.
+  if (c_split == 1 && c.block_m == 256 && c.block_n == 256 && tiles(256, 256) >= cus && K % kBK == 0 && K >= kW4MinK && N % 8 == 0 &&
+      N <= (1 << 21)) {
+    cfg->wave_m = 128;
+    cfg->wave_n = 128;
+  }
   if (split_req < 0 && tiles(c.block_m, c.block_n) < cus / 2 && K >= 2048)
     cfg->pipeline = 2;  // few workgroups per CU: a long prefetch queue keeps HBM busy
   if (split_k) *split_k = c_split;
@@ -403,7 +414,7 @@ int beam_gemmrc(const void* A, const void* B, void* C, int M, int N, int K, int 
   }
   beam_tile_cfg c;
   const KernelSet* ks;
-  if ((rc = resolve_cfg(cfg, M, N, K, &c, &ks))) return rc;
+  if ((rc = resolve_cfg(cfg, M, N, K, &c, &ks, -1, true))) return rc;
   GemmParams p = base_params(A, B, M, N, K, c);
   p.C = C;
   const long tiles = (long)p.tiles_m * p.tiles_n;
@@ -411,12 +422,16 @@ int beam_gemmrc(const void* A, const void* B, void* C, int M, int N, int K, int 
   // The 256 x 256 tile of four 128 x 128 wavefronts has a kernel of its own (gemm_w4.h), built for problems
   // of a round of workgroups or more: one workgroup per CU walks its tiles with the operand ring running
   // through the tile boundaries.  It is what the tile {256, 256, 128, 128} means wherever its preconditions
-  // hold, and what a call without a tile gets in place of the 8-wavefront 256 x 256 tile from one full
-  // round of workgroups on (8192^3 fp16, same machine, in turn: 1490-1515 against 1455-1465 TFLOP/s).
+  // hold (elsewhere that tile is the 4-wavefront member of the gemm_kernel.h family), and what
+  // beam_default_config names from one full round of workgroups on.
   const bool w4_fits = c.pipeline == 0 && K % kBK == 0 && K >= kW4MinK && N % 8 == 0 && ((uintptr_t)C & 15) == 0 && N <= (1 << 21);
   const bool w4_named = c.block_m == 256 && c.block_n == 256 && c.wave_m == 128 && c.wave_n == 128;
-  const bool w4_default = !cfg && c.block_m == 256 && c.block_n == 256 && tiles >= cus;
-  if (w4_fits && (w4_named || w4_default)) {
+  if (w4_named && !w4_fits && !cfg) {  // the library's own choice, but C is only 8-byte aligned: the 8-wavefront tile
+    c.wave_m = 128;
+    c.wave_n = 64;
+    if ((rc = resolve_cfg(&c, M, N, K, &c, &ks))) return rc;
+  }
+  if (w4_fits && w4_named) {
     // Non-temporal stores of C pay when C is larger than the 256 MB last-level cache (and the K loops
     // are not so short that the writes are the bound).
     p.c_streaming = (size_t)M * N * 2 >= ((size_t)256 << 20) && K >= 1024;
@@ -656,7 +671,7 @@ static size_t ln_workspace_need(int M, int N, const beam_tile_cfg& c, int mode) 
 
 // The tile a GEMM+LayerNorm call runs with: the caller's, or the default for (M, N, K); never the deep pipeline.
 static int ln_resolve_cfg(const beam_tile_cfg* cfg, int M, int N, int K, beam_tile_cfg* c, const KernelSet** ks) {
-  int rc = resolve_cfg(cfg, M, N, K, c, ks);
+  int rc = resolve_cfg(cfg, M, N, K, c, ks, -1, true);
   if (rc) return rc;
   if (c->pipeline == 2) c->pipeline = 0;  // the deep pipeline exists for the store / split-K kernels only
   return BEAM_OK;
@@ -717,6 +732,16 @@ int beam_gemmrc_ln_ex(const void* A, const void* B, const void* gamma, const voi
   if (st != nullptr) (void)hipStreamIsCapturing(st, &capturing);
   if (capturing != hipStreamCaptureStatusNone && mode == BEAM_LN_AUTO) mode = BEAM_LN_TWOPASS;
   mode = ln_resolve_mode(mode, c, *ks, N);
+  // The 256 x 256 tile runs on the kernel of gemm_w4.h where that one's preconditions hold (asked for by
+  // name, or as the library's own choice); where they do not, the library's own choice falls back to the
+  // 8-wavefront tile of the same shape.
+  const bool w4_fits = mode == BEAM_LN_FUSED && c.pipeline == 0 && c.block_m == 256 && c.block_n == 256 && K % kBK == 0 &&
+                       K >= kW4MinK && N % 8 == 0 && N <= (1 << 21) &&
+                       (((uintptr_t)Y | (uintptr_t)gamma | (uintptr_t)beta) & 15) == 0;
+  if (!cfg && !w4_fits && c.block_m == 256 && c.block_n == 256 && c.wave_m == 128 && c.wave_n == 128) {
+    c.wave_n = 64;
+    if ((rc = resolve_cfg(&c, M, N, K, &c, &ks))) return rc;
+  }
   const size_t need = ln_workspace_need(M, N, c, mode);
   if (!ws || ws_bytes < need)
     return fail(BEAM_ERR_WORKSPACE, "GEMM+LayerNorm needs %zu bytes of workspace, got %zu", need, ws_bytes);
@@ -759,10 +784,6 @@ int beam_gemmrc_ln_ex(const void* A, const void* B, const void* gamma, const voi
     } else {
       grid = (unsigned)band_block_grid(p.tiles_m, p.group_m, p.group_n);
     }
-    // The 256 x 256 tile runs on the kernel of gemm_w4.h where that one's preconditions hold (asked for by
-    // name, or as the library's own choice).
-    const bool w4_fits = c.pipeline == 0 && c.block_m == 256 && c.block_n == 256 && K % kBK == 0 && K >= kW4MinK && N % 8 == 0 &&
-                         N <= (1 << 21) && (((uintptr_t)Y | (uintptr_t)gamma | (uintptr_t)beta) & 15) == 0;
     if (w4_fits && (!cfg || (c.wave_m == 128 && c.wave_n == 128))) {
       BEAM_HIP(launch_gemm_w4_ln(p, dtype, dim3(grid, 1, 1), st));
       return BEAM_OK;

@@ -77,7 +77,7 @@ def test_tuner_picks_max_and_memoises(tuner_mod, monkeypatch, tmp_path):
     t.tune((512, 256, 1024), dtype="bf16")
     assert len(calls) == 2 * n                                               # dtype is part of the key
     blob = json.load(open(path))
-    assert blob["arch"] == "gfx950" and blob["entries"]["gemm(512,256,1024,fp16,)"][0] == "fast"
+    assert blob["arch"] == "gfx950" and blob["entries"]["gemm(512,256,1024,fp16,gfx950,)"][0] == "fast"
     # a second tuner loads the persisted result and does not re-measure
     t2 = tuner_mod.OperatorTuner(cache_path=path, verify=False)
     t2.gemm_ops = t.gemm_ops
@@ -85,6 +85,18 @@ def test_tuner_picks_max_and_memoises(tuner_mod, monkeypatch, tmp_path):
     t2._load(path)
     calls.clear()
     assert str(t2.tune((512, 256, 1024))[0]) == "fast" and not calls
+    # ... but not a file written on another architecture, or for another CU count
+    for change in ({"arch": "gfx942"}, {"compute_units": 12345}):
+        other = dict(blob)
+        other.update(change)
+        monkeypatch.setattr(tuner_mod, "_compute_units", lambda: 256)
+        json.dump(other, open(path, "w"))
+        t3 = tuner_mod.OperatorTuner(cache_path=path, verify=False)
+        assert not t3.cache
+    # a problem on which nothing runs is reported, not remembered
+    t4 = tuner_mod.OperatorTuner(verify=False)
+    t4.gemm_ops = [FakeOp(named("broken", lambda a, b, c: None))]
+    assert t4.tune((8, 8, 8)) == (None, -1) and not t4.cache
 
 
 def test_candidate_space(beamc):
@@ -96,3 +108,10 @@ def test_candidate_space(beamc):
     assert sum(n.startswith("gemmrc_splitk_spec") for n in names) >= 5 * len(tuner.SPLIT_FACTORS)
     assert any("256x256" in n for n in names)
     assert tuner.SPLIT_FACTORS == (4, 8, 16, 32, 64)
+    # the LDS pipeline depth is an axis of the search: every tile appears with all three depths
+    plain = [o for o in t.gemm_ops if str(o).startswith("gemmrc_spec[")]
+    depths = {}
+    for o in plain:
+        c = o.native["config"]
+        depths.setdefault((c.block_m, c.block_n, c.wave_m, c.wave_n), set()).add(c.pipeline)
+    assert len(depths) == len(beamc.list_configs()) and all(d == {0, 1, 2} for d in depths.values())
