@@ -45,7 +45,8 @@ class _Problem(ctypes.Structure):
                 ("gamma", ctypes.c_void_p), ("beta", ctypes.c_void_p), ("eps", ctypes.c_float),
                 ("M", ctypes.c_int), ("N", ctypes.c_int), ("K", ctypes.c_int), ("dtype", ctypes.c_int),
                 ("split_k", ctypes.c_int), ("ws", ctypes.c_void_p), ("ws_bytes", ctypes.c_size_t),
-                ("side_x", ctypes.c_void_p), ("side_y", ctypes.c_void_p), ("side_count", ctypes.c_longlong)]
+                ("side_x", ctypes.c_void_p), ("side_y", ctypes.c_void_p), ("side_count", ctypes.c_longlong),
+                ("ln_mode", ctypes.c_int)]
 
 
 def library_path() -> str:
@@ -484,7 +485,7 @@ OP_GEMM, OP_SPLITK, OP_GEMM_LN, OP_GEMM_SILU, OP_SILU, OP_MATMUL_NN = 0, 1, 2, 3
 
 
 def bench(op: int, a, b, c, config: Optional[TileConfig] = None, split_k: int = 0, gamma=None, beta=None,
-          eps: float = 1e-5, warmup: int = 5, iters: int = 20, x=None, y=None) -> float:
+          eps: float = 1e-5, warmup: int = 5, iters: int = 20, x=None, y=None, ln_mode: int = 0) -> float:
     """Average milliseconds per call (HIP events around `iters` back-to-back launches)."""
     if op == OP_MATMUL_NN:  # b is [K, N]
         pa, (M, K), d, st = _describe(a)
@@ -496,7 +497,7 @@ def bench(op: int, a, b, c, config: Optional[TileConfig] = None, split_k: int = 
         pa, pb, pc, M, N, K, d, st = _problem(a, b, c)
     cfg = config.to_c() if config is not None else None
     cfgp = ctypes.byref(cfg) if cfg is not None else None
-    q = _Problem(pa, pb, pc, None, None, eps, M, N, K, d, split_k, None, 0, None, None, 0)
+    q = _Problem(pa, pb, pc, None, None, eps, M, N, K, d, split_k, None, 0, None, None, 0, ln_mode)
     if op in (OP_GEMM_SILU, OP_SILU):
         q.side_x, q.side_y, q.side_count, _, _ = _flat_pair(x, y, d)
     ws = None
@@ -507,7 +508,7 @@ def bench(op: int, a, b, c, config: Optional[TileConfig] = None, split_k: int = 
         ws = _get_workspace(max(lib.beam_splitk_workspace_bytes(M, N, s), 1))
     elif op == 2:
         q.gamma, q.beta = _describe(gamma)[0], _describe(beta)[0]
-        ws = _get_ln_workspace(lib.beam_gemmrc_ln_workspace_bytes(M, N, cfgp))
+        ws = _get_ln_workspace(lib.beam_gemmrc_ln_workspace_bytes_for(M, N, K, cfgp, ln_mode))
     if ws is not None:
         q.ws, q.ws_bytes = ws.ptr, ws.nbytes
     ms = ctypes.c_float()

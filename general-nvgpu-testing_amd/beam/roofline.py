@@ -1,6 +1,6 @@
 """Roofline arithmetic for tiled GEMMs, with an MI355X row.
 
-Counterpart of the reference's python/scripts/gemm_flops.py:1-90 and python/scripts/attn_flops.py:1-16 (GPUSpec :4-13, spec list
+Counterpart of the reference's python/scripts/gemm_flops.py:1-90 (GPUSpec :4-13, spec list
 :26-32, print_gemm_bound :37-76): the time a GEMM needs at the matrix-unit peak, the time its
 tiles need at the memory bandwidth when every tile fetches its operands once, and their ratio.
 Differences: a function that returns the numbers (the reference only prints), bytes counted with
@@ -30,11 +30,8 @@ class GPUSpec:
 BITWIDTH_MAP = {"tf32": 32, "fp16": 16, "bf16": 16, "fp8": 8, "int8": 8, "int4": 4}
 
 GPU_SPEC_LIST = [
+    # one row of the reference's list, kept so that its worked example can be reproduced as a check
     GPUSpec("A100_{PCIe,SXM}_HBM2", 1555, 19.5, 156, 312, 624, 0, 164, 108),
-    GPUSpec("A100_PCIe_HBM2e", 1935, 19.5, 156, 312, 624, 0, 164, 108),
-    GPUSpec("A100_SXM_HBM2e", 2039, 19.5, 156, 312, 624, 0, 164, 108),
-    GPUSpec("H100_SXM", 3350, 67, 989 / 2, 1979 / 2, 3958 / 2, 3958 / 2, 228, 132),
-    GPUSpec("H100_NVL", 3900, 60, 835 / 2, 1671 / 2, 3341 / 2, 3341 / 2, 228, 132),
     # MI355X (gfx950): 256 CUs x 4 SIMDs x 1024 fp16 FLOP/clk x 2.4 GHz; HBM3E 8 TB/s; no tf32 unit
     # (the fp32 matrix rate is 157.3 TFLOP/s).
     GPUSpec("MI355X", 8000, 157.3, 0, 2516.6, 5033.2, 5033.2, 160, 256),
@@ -79,22 +76,6 @@ def print_gemm_bound(spec: GPUSpec, dtype: str, n: int, k: int, m: int, micro_n:
     return r
 
 
-def attn_flops(batch_size: int, num_heads: int, seq_len: int, head_dim: int) -> int:
-    """FLOPs of one attention layer's two batched GEMMs, Q.K^T ([b,h,s,d] x [b,h,d,s]) and P.V
-    ([b,h,s,s] x [b,h,s,d]), 2 per multiply-add: 4*b*h*s*s*d.  Same count as the reference's
-    python/scripts/attn_flops.py:1-7 (its example, :11: b=2, h=24, s=4429, d=64)."""
-    return 4 * batch_size * num_heads * seq_len * seq_len * head_dim
-
-
-def attn_bound_ms(spec: GPUSpec, dtype: str, batch_size: int, num_heads: int, seq_len: int, head_dim: int) -> float:
-    """Time of those two GEMMs at the matrix-unit peak of `spec`."""
-    rate = getattr(spec, "fp16" if dtype == "bf16" else dtype)
-    if rate <= 0:
-        raise ValueError(f"{spec.name} has no {dtype} matrix rate")
-    return attn_flops(batch_size, num_heads, seq_len, head_dim) / (rate * 1e12) * 1e3
-
-
 if __name__ == "__main__":
     print_gemm_bound(GPU_NAME_SPEC_MAP["MI355X"], "fp16", 8192, 8192, 8192, 256, 8192, 256)
     print_gemm_bound(GPU_NAME_SPEC_MAP["MI355X"], "fp16", 256, 32768, 256, 64, 2048, 64)
-    print(f"FLOPS: {attn_flops(2, 24, 4096 + 333, 64)}")

@@ -23,6 +23,15 @@ hipError_t launch_ln_apply(const float* X, const float* stats, const void* gamma
 hipError_t launch_ln_prepare(int* header, float* sets, size_t set_floats_total, int geom_lo, int geom_hi, int expected,
                              hipStream_t stream);
 
+// gemmrc without any condition on K, N or alignment (slow; what the tiled kernels refuse runs here):
+// C[M][N] = A[M][K] . B^T with B as [N][K], or as [K][N] when b_kmajor; C 16-bit, or fp32 when out_fp32.
+// Grid dimension y = ceil(M / 64) must stay below 65536.
+hipError_t launch_generic_gemm(const void* A, const void* B, void* C, int M, int N, int K, int dtype, bool b_kmajor,
+                               bool out_fp32, hipStream_t stream);
+// Y[m][:] (16-bit) = LayerNorm of the fp32 row X[m][:], statistics computed here (generic path).
+hipError_t launch_ln_rows(const float* X, const void* gamma, const void* beta, void* Y, int M, int N, float eps, int dtype,
+                          hipStream_t stream);
+
 // y[i] (16-bit) = silu(x[i]) for i in [0, count); x and y 16-byte aligned.
 hipError_t launch_silu(const void* x, void* y, size_t count, int dtype, hipStream_t stream);
 

@@ -139,6 +139,93 @@ __global__ void __launch_bounds__(256) silu_kernel(const T* __restrict__ x, T* _
   if (i < count) y[i] = silu_16<T>(x[i]);
 }
 
+// gemmrc for problems the tiled kernels do not take: K not a multiple of 8 (rows of A and B are then not
+// 16-byte aligned), operands or output at odd addresses, and the [K][N] layout with N not a multiple of 8.
+// A plain LDS-tiled fp32 kernel: 64 x 64 outputs per workgroup, 16 K elements per step, 4 x 4 outputs per
+// thread, every access bounds-checked element by element.  Same arithmetic contract (16-bit inputs, fp32
+// accumulation, one rounding), far from the same speed; it exists so that no well-formed problem is refused
+// (the reference's Triton matmul masks any edge: python/beam/triton_kernels/gemm.py:62-63,75).
+// OUT32: write fp32 (the input of the row-wise LayerNorm below) instead of the 16-bit type.
+template <typename T, bool B_KMAJOR, bool OUT32>
+__global__ void __launch_bounds__(256) generic_gemm_kernel(const T* __restrict__ A, const T* __restrict__ B, void* __restrict__ Cv,
+                                                            int M, int N, int K) {
+  constexpr int TS = 64, KS = 16;
+  __shared__ float as[KS][TS + 1], bs[KS][TS + 1];
+  const int tid = threadIdx.x;
+  const int row0 = blockIdx.y * TS, col0 = blockIdx.x * TS;
+  const int ty = tid / 16, tx = tid % 16;
+  float acc[4][4] = {};
+  for (int k0 = 0; k0 < K; k0 += KS) {
+    // 64 rows x 16 k of each operand: thread t fetches row t / 4, k (t % 4) * 4 .. + 3
+    const int lr = tid / 4, lk = (tid % 4) * 4;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int k = k0 + lk + e;
+      const int m = row0 + lr, n = col0 + lr;
+      as[lk + e][lr] = (m < M && k < K) ? (float)A[(size_t)m * K + k] : 0.0f;
+      bs[lk + e][lr] = (n < N && k < K) ? (float)(B_KMAJOR ? B[(size_t)k * N + n] : B[(size_t)n * K + k]) : 0.0f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < KS; ++k) {
+      float a[4], b[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) a[i] = as[k][ty * 4 + i];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) b[j] = bs[k][tx * 4 + j];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] += a[i] * b[j];
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int m = row0 + ty * 4 + i;
+    if (m >= M) continue;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int n = col0 + tx * 4 + j;
+      if (n >= N) continue;
+      if (OUT32) ((float*)Cv)[(size_t)m * N + n] = acc[i][j];
+      else ((T*)Cv)[(size_t)m * N + n] = (T)acc[i][j];
+    }
+  }
+}
+
+// Row-wise LayerNorm of fp32 X for the generic path: one workgroup per row; mean, then M2 about it (two passes
+// over the row, no cancellation), then y = (x - mean) * rstd * gamma + beta.  Scalar accesses: no alignment
+// is assumed of anything.
+template <typename T>
+__global__ void __launch_bounds__(256) ln_rows_kernel(const float* __restrict__ X, const T* __restrict__ gamma,
+                                                       const T* __restrict__ beta, T* __restrict__ Y, int N, float eps) {
+  __shared__ float red[256];
+  const float* x = X + (size_t)blockIdx.x * N;
+  T* y = Y + (size_t)blockIdx.x * N;
+  auto block_sum = [&](float v) {
+    red[threadIdx.x] = v;
+    __syncthreads();
+    for (int s = 128; s > 0; s >>= 1) {
+      if ((int)threadIdx.x < s) red[threadIdx.x] += red[threadIdx.x + s];
+      __syncthreads();
+    }
+    const float total = red[0];
+    __syncthreads();
+    return total;
+  };
+  float s = 0.0f;
+  for (int n = threadIdx.x; n < N; n += 256) s += x[n];
+  const float mean = block_sum(s) / (float)N;
+  float q = 0.0f;
+  for (int n = threadIdx.x; n < N; n += 256) {
+    const float d = x[n] - mean;
+    q += d * d;
+  }
+  const float rstd = 1.0f / sqrtf(block_sum(q) / (float)N + eps);
+  for (int n = threadIdx.x; n < N; n += 256) y[n] = (T)((x[n] - mean) * rstd * (float)gamma[n] + (float)beta[n]);
+}
+
 // Before every fused GEMM+LayerNorm launch: decide, on the device, whether the workspace is in the state the
 // previous fused launch left it in -- header intact, same geometry, and every workgroup of that launch
 // finished (each of them has marked its slots of the other statistics set "not published") -- and then
@@ -196,6 +283,36 @@ hipError_t launch_silu(const void* x, void* y, size_t count, int dtype, hipStrea
 
 hipError_t launch_fill_floats(float* floats, size_t n, float value, hipStream_t stream) {
   hipLaunchKernelGGL(fill_floats_kernel, dim3(256), dim3(256), 0, stream, floats, n, value);
+  return hipGetLastError();
+}
+
+hipError_t launch_generic_gemm(const void* A, const void* B, void* C, int M, int N, int K, int dtype, bool b_kmajor,
+                               bool out_fp32, hipStream_t stream) {
+  const dim3 grid((unsigned)((N + 63) / 64), (unsigned)((M + 63) / 64), 1);
+#define BEAM_GENERIC(T, KM, O32) \
+  hipLaunchKernelGGL((generic_gemm_kernel<T, KM, O32>), grid, dim3(256), 0, stream, (const T*)A, (const T*)B, C, M, N, K)
+#define BEAM_GENERIC_T(T)                                   \
+  do {                                                      \
+    if (b_kmajor && out_fp32) BEAM_GENERIC(T, true, true);  \
+    else if (b_kmajor) BEAM_GENERIC(T, true, false);        \
+    else if (out_fp32) BEAM_GENERIC(T, false, true);        \
+    else BEAM_GENERIC(T, false, false);                     \
+  } while (0)
+  if (dtype == BEAM_BF16) BEAM_GENERIC_T(__bf16);
+  else BEAM_GENERIC_T(_Float16);
+#undef BEAM_GENERIC_T
+#undef BEAM_GENERIC
+  return hipGetLastError();
+}
+
+hipError_t launch_ln_rows(const float* X, const void* gamma, const void* beta, void* Y, int M, int N, float eps, int dtype,
+                          hipStream_t stream) {
+  if (dtype == BEAM_BF16)
+    hipLaunchKernelGGL(ln_rows_kernel<__bf16>, dim3((unsigned)M), dim3(256), 0, stream, X, (const __bf16*)gamma, (const __bf16*)beta,
+                       (__bf16*)Y, N, eps);
+  else
+    hipLaunchKernelGGL(ln_rows_kernel<_Float16>, dim3((unsigned)M), dim3(256), 0, stream, X, (const _Float16*)gamma,
+                       (const _Float16*)beta, (_Float16*)Y, N, eps);
   return hipGetLastError();
 }
 

@@ -112,17 +112,20 @@ static_assert((unsigned long long)kMaxK * 512ull < kOobOffset && kMaxK % 8 == 0,
 // Elements of a side-job array: its byte size must stay below the out-of-range offset the kernels use.
 constexpr long long kMaxSideElems = (long long)(kOobOffset / 16) * 8;
 
-int check_problem(const void* A, const void* B, const void* C, int M, int N, int K, int dtype) {
+// Validates a gemmrc problem.  *generic is set when it is well formed but outside what the tiled kernels take
+// (rows of A / B that are not multiples of 16 bytes, i.e. K % 8 != 0; operands not 16-byte or output not
+// 8-byte aligned; K beyond the descriptor range): such problems run on the plain kernel of aux_kernels.hip.
+int check_problem(const void* A, const void* B, const void* C, int M, int N, int K, int dtype, bool* generic) {
+  *generic = false;
   if (M < 0 || N < 0 || K < 0) return fail(BEAM_ERR_INVALID, "negative dimension (M=%d N=%d K=%d)", M, N, K);
   if (dtype != BEAM_F16 && dtype != BEAM_BF16) return fail(BEAM_ERR_UNSUPPORTED, "dtype %d: only fp16 (0) and bf16 (1)", dtype);
   if (M == 0 || N == 0) return BEAM_OK;
   if (!C) return fail(BEAM_ERR_INVALID, "null output pointer");
   if (K > 0 && (!A || !B)) return fail(BEAM_ERR_INVALID, "null input pointer");
-  if (K > kMaxK) return fail(BEAM_ERR_UNSUPPORTED, "K=%d exceeds %d", K, kMaxK);
-  if (K % 8 != 0) return fail(BEAM_ERR_UNSUPPORTED, "K=%d: rows must be multiples of 16 bytes (K %% 8 == 0)", K);
-  if (((uintptr_t)A | (uintptr_t)B) & 15) return fail(BEAM_ERR_UNSUPPORTED, "A and B must be 16-byte aligned");
-  if ((uintptr_t)C & 7) return fail(BEAM_ERR_UNSUPPORTED, "C must be 8-byte aligned");
+  if (((uintptr_t)A | (uintptr_t)B | (uintptr_t)C) & 1) return fail(BEAM_ERR_INVALID, "A, B and C must be aligned to their 16-bit elements");
   if ((size_t)M * (size_t)N >= ((size_t)1 << 40)) return fail(BEAM_ERR_UNSUPPORTED, "M*N too large");
+  if ((M + 63) / 64 > 65535) return fail(BEAM_ERR_UNSUPPORTED, "M=%d too large", M);
+  *generic = K > kMaxK || K % 8 != 0 || ((((uintptr_t)A | (uintptr_t)B) & 15) != 0) || (((uintptr_t)C & 7) != 0);
   return BEAM_OK;
 }
 
@@ -403,13 +406,18 @@ extern "C" {
 
 int beam_gemmrc(const void* A, const void* B, void* C, int M, int N, int K, int dtype,
                 const beam_tile_cfg* cfg, void* stream) {
-  int rc = check_problem(A, B, C, M, N, K, dtype);
+  bool generic;
+  int rc = check_problem(A, B, C, M, N, K, dtype, &generic);
   if (rc) return rc;
   if (M == 0 || N == 0) return BEAM_OK;
   if ((rc = beam_init())) return rc;
   hipStream_t st = (hipStream_t)stream;
   if (K == 0) {
     BEAM_HIP(launch_zero_u16(C, (size_t)M * N, st));
+    return BEAM_OK;
+  }
+  if (generic) {  // whatever tile was named: the tiled kernels cannot take this problem
+    BEAM_HIP(launch_generic_gemm(A, B, C, M, N, K, dtype, false, false, st));
     return BEAM_OK;
   }
   beam_tile_cfg c;
@@ -458,15 +466,19 @@ int beam_gemmrc(const void* A, const void* B, void* C, int M, int N, int K, int 
 
 int beam_matmul_nn(const void* A, const void* B, void* C, int M, int N, int K, int dtype, const beam_tile_cfg* cfg,
                    void* stream) {
-  int rc = check_problem(A, B, C, M, N, K, dtype);
+  bool generic;
+  int rc = check_problem(A, B, C, M, N, K, dtype, &generic);
   if (rc) return rc;
   if (M == 0 || N == 0) return BEAM_OK;
-  if (N % 8 != 0) return fail(BEAM_ERR_UNSUPPORTED, "N=%d: rows of B must be multiples of 16 bytes (N %% 8 == 0)", N);
-  if (N > (1 << 24)) return fail(BEAM_ERR_UNSUPPORTED, "N=%d exceeds %d (64 rows of B per buffer descriptor)", N, 1 << 24);
   if ((rc = beam_init())) return rc;
   hipStream_t st = (hipStream_t)stream;
   if (K == 0) {
     BEAM_HIP(launch_zero_u16(C, (size_t)M * N, st));
+    return BEAM_OK;
+  }
+  // rows of B ([K][N]) that are not multiples of 16 bytes, or more than a descriptor spans: the plain kernel
+  if (generic || N % 8 != 0 || N > (1 << 24)) {
+    BEAM_HIP(launch_generic_gemm(A, B, C, M, N, K, dtype, true, false, st));
     return BEAM_OK;
   }
   beam_tile_cfg c;
@@ -494,7 +506,8 @@ int beam_silu(const void* X, void* Y, long long count, int dtype, void* stream) 
 
 int beam_parallel_gemmrc_silu(const void* A, const void* B, void* C, int M, int N, int K, const void* X, void* Y,
                               long long count, int dtype, const beam_tile_cfg* cfg, void* stream) {
-  int rc = check_problem(A, B, C, M, N, K, dtype);
+  bool generic;
+  int rc = check_problem(A, B, C, M, N, K, dtype, &generic);
   if (rc) return rc;
   if (count < 0) return fail(BEAM_ERR_INVALID, "negative element count %lld", count);
   if (count > 0) {
@@ -503,7 +516,7 @@ int beam_parallel_gemmrc_silu(const void* A, const void* B, void* C, int M, int 
     if (count > kMaxSideElems)
       return fail(BEAM_ERR_UNSUPPORTED, "count=%lld exceeds %lld elements (one buffer descriptor)", count, kMaxSideElems);
   }
-  if (M == 0 || N == 0 || K == 0) {  // no K loop to hide anything in: the two halves run one after the other
+  if (M == 0 || N == 0 || K == 0 || generic) {  // no (tiled) K loop to hide anything in: the two halves run one after the other
     if ((rc = beam_gemmrc(A, B, C, M, N, K, dtype, cfg, stream))) return rc;
     return beam_silu(X, Y, count, dtype, stream);
   }
@@ -577,19 +590,25 @@ int beam_splitk_effective(int M, int N, int K, const beam_tile_cfg* cfg, int spl
   beam_tile_cfg c;
   const KernelSet* ks;
   if (M <= 0 || N <= 0 || K < 0) return 1;
+  if (K % 8 != 0 || K > kMaxK) return 1;  // the plain kernel: no slices
   if (resolve_cfg(cfg, M, N, K, &c, &ks, split_k > 0 ? split_k : 0)) return -1;
   return effective_split(M, N, K, c, split_k);
 }
 
 int beam_gemmrc_splitk(const void* A, const void* B, void* C, int M, int N, int K, int dtype,
                        const beam_tile_cfg* cfg, int split_k, void* ws, size_t ws_bytes, void* stream) {
-  int rc = check_problem(A, B, C, M, N, K, dtype);
+  bool generic;
+  int rc = check_problem(A, B, C, M, N, K, dtype, &generic);
   if (rc) return rc;
   if (M == 0 || N == 0) return BEAM_OK;
   if ((rc = beam_init())) return rc;
   hipStream_t st = (hipStream_t)stream;
   if (K == 0) {
     BEAM_HIP(launch_zero_u16(C, (size_t)M * N, st));
+    return BEAM_OK;
+  }
+  if (generic) {  // one pass of the plain kernel, no slices (beam_splitk_effective says 1 for K % 8 != 0)
+    BEAM_HIP(launch_generic_gemm(A, B, C, M, N, K, dtype, false, false, st));
     return BEAM_OK;
   }
   beam_tile_cfg c;
@@ -661,6 +680,12 @@ static int ln_resolve_mode(int mode, const beam_tile_cfg& c, const KernelSet& ks
   return mode;
 }
 
+// GEMM+LayerNorm problems that run on the plain kernels, and the workspace they need (fp32 X).
+static bool ln_is_generic(bool gemm_generic, const void* gamma, const void* beta) {
+  return gemm_generic || ((((uintptr_t)gamma | (uintptr_t)beta) & 7) != 0);
+}
+static size_t ln_generic_need(int M, int N) { return align_up((size_t)M * N * sizeof(float), 256); }
+
 // Bytes for tile `c` in `mode` (already resolved: two-pass or fused).
 static size_t ln_workspace_need(int M, int N, const beam_tile_cfg& c, int mode) {
   const size_t tiles_m = (size_t)(M + c.block_m - 1) / c.block_m;
@@ -679,6 +704,7 @@ static int ln_resolve_cfg(const beam_tile_cfg* cfg, int M, int N, int K, beam_ti
 
 size_t beam_gemmrc_ln_workspace_bytes_for(int M, int N, int K, const beam_tile_cfg* cfg, int mode) {
   if (M <= 0 || N <= 0 || K < 0) return 0;
+  if (K % 8 != 0 || K > kMaxK) return ln_generic_need(M, N);
   (void)beam_init();  // AUTO depends on the device
   beam_tile_cfg c;
   const KernelSet* ks;
@@ -688,7 +714,11 @@ size_t beam_gemmrc_ln_workspace_bytes_for(int M, int N, int K, const beam_tile_c
 
 size_t beam_gemmrc_ln_workspace_bytes_ex(int M, int N, const beam_tile_cfg* cfg, int mode) {
   if (M <= 0 || N <= 0) return 0;
-  if (cfg) return beam_gemmrc_ln_workspace_bytes_for(M, N, 64, cfg, mode);  // a given tile does not depend on K
+  // a given tile does not depend on K (but a problem the tiled kernels refuse -- odd K, odd addresses -- needs fp32 X)
+  if (cfg) {
+    const size_t tiled = beam_gemmrc_ln_workspace_bytes_for(M, N, 64, cfg, mode), plain = ln_generic_need(M, N);
+    return tiled > plain ? tiled : plain;
+  }
   // Without a tile the library picks one from (M, N, K), and K is not known here: the largest need over
   // every tile it can pick.
   (void)beam_init();
@@ -710,15 +740,27 @@ size_t beam_gemmrc_ln_workspace_bytes(int M, int N, const beam_tile_cfg* cfg) {
 int beam_gemmrc_ln_ex(const void* A, const void* B, const void* gamma, const void* beta, float eps, void* Y,
                       int M, int N, int K, int dtype, const beam_tile_cfg* cfg, int mode, void* ws,
                       size_t ws_bytes, void* stream) {
-  int rc = check_problem(A, B, Y, M, N, K, dtype);
+  bool generic;
+  int rc = check_problem(A, B, Y, M, N, K, dtype, &generic);
   if (rc) return rc;
   if (M == 0 || N == 0) return BEAM_OK;
   if (!gamma || !beta) return fail(BEAM_ERR_INVALID, "null gamma/beta");
-  if (((uintptr_t)gamma | (uintptr_t)beta) & 7) return fail(BEAM_ERR_UNSUPPORTED, "gamma and beta must be 8-byte aligned");
+  if (((uintptr_t)gamma | (uintptr_t)beta) & 1) return fail(BEAM_ERR_INVALID, "gamma and beta must be aligned to their 16-bit elements");
   if (!(eps >= 0.0f)) return fail(BEAM_ERR_INVALID, "eps must be >= 0");
   if (mode < BEAM_LN_AUTO || mode > BEAM_LN_FUSED) return fail(BEAM_ERR_INVALID, "unknown LayerNorm mode %d", mode);
   if ((rc = beam_init())) return rc;
   hipStream_t st = (hipStream_t)stream;
+  if (ln_is_generic(generic, gamma, beta)) {
+    // What the tiled kernels cannot take: the plain GEMM into fp32 X, then a row-wise LayerNorm (whatever mode was named).
+    const size_t need = ln_generic_need(M, N);
+    if (!ws || ws_bytes < need)
+      return fail(BEAM_ERR_WORKSPACE, "GEMM+LayerNorm needs %zu bytes of workspace, got %zu", need, ws_bytes);
+    if ((uintptr_t)ws & 15) return fail(BEAM_ERR_UNSUPPORTED, "workspace must be 16-byte aligned");
+    if (K == 0) BEAM_HIP(launch_fill_floats((float*)ws, (size_t)M * N, 0.0f, st));
+    else BEAM_HIP(launch_generic_gemm(A, B, ws, M, N, K, dtype, false, true, st));
+    BEAM_HIP(launch_ln_rows((const float*)ws, gamma, beta, Y, M, N, eps, dtype, st));
+    return BEAM_OK;
+  }
   beam_tile_cfg c;
   const KernelSet* ks;
   if ((rc = ln_resolve_cfg(cfg, M, N, K, &c, &ks))) return rc;
@@ -836,8 +878,8 @@ int beam_bench(int op, const beam_problem* q, const beam_tile_cfg* cfg, int warm
         return beam_gemmrc_splitk(q->A, q->B, q->C, q->M, q->N, q->K, q->dtype, cfg, q->split_k, q->ws,
                                   q->ws_bytes, stream);
       case BEAM_OP_GEMM_LN:
-        return beam_gemmrc_ln(q->A, q->B, q->gamma, q->beta, q->eps, q->C, q->M, q->N, q->K, q->dtype, cfg,
-                              q->ws, q->ws_bytes, stream);
+        return beam_gemmrc_ln_ex(q->A, q->B, q->gamma, q->beta, q->eps, q->C, q->M, q->N, q->K, q->dtype, cfg, q->ln_mode,
+                                 q->ws, q->ws_bytes, stream);
       case BEAM_OP_GEMM_SILU:
         return beam_parallel_gemmrc_silu(q->A, q->B, q->C, q->M, q->N, q->K, q->side_x, q->side_y, q->side_count,
                                          q->dtype, cfg, stream);

@@ -16,6 +16,7 @@
 //             [--wave TMxTN] [--pipeline 0|1] [--group G] [--splitk S] [--iters I] [--warmup W]
 //             [--count ELEMENTS]   (silu: GEMM, SiLU alone and GEMM with the SiLU in its K loop)
 //             [--data normal|zeros] (zeros: all-zero operands, for telling schedule limits from power limits)
+//             [--ln-mode auto|twopass|fused]   (--op ln)
 //   beam_host --tune --m M --n N --k K [--dtype fp16|bf16]
 //   beam_host --copy MiB      device-to-device copy of known size (calibrates profiler byte counters)
 #include <cmath>
@@ -369,7 +370,8 @@ BEAM_TEST(error_paths) {
   DevBuf da(64 * 64 * 2), db(64 * 64 * 2), dc(64 * 64 * 2);
   beam_tile_cfg bad = {96, 96, 48, 48, 0, 0};
   if (beam_gemmrc(da.p, db.p, dc.p, 64, 64, 64, BEAM_F16, &bad, nullptr) != BEAM_ERR_UNSUPPORTED) c.fail("bad tile accepted");
-  if (beam_gemmrc(da.p, db.p, dc.p, 64, 64, 60, BEAM_F16, nullptr, nullptr) != BEAM_ERR_UNSUPPORTED) c.fail("K % 8 accepted");
+  if (beam_gemmrc(da.p, db.p, dc.p, 64, 64, 60, BEAM_F16, nullptr, nullptr) != BEAM_OK) c.fail("K % 8 != 0 refused (the plain kernel takes it)");
+  if (beam_gemmrc((char*)da.p + 1, db.p, dc.p, 64, 64, 56, BEAM_F16, nullptr, nullptr) != BEAM_ERR_INVALID) c.fail("odd address accepted");
   if (beam_gemmrc(da.p, db.p, dc.p, 64, 64, 64, 9, nullptr, nullptr) != BEAM_ERR_UNSUPPORTED) c.fail("bad dtype accepted");
   if (beam_gemmrc(nullptr, db.p, dc.p, 64, 64, 64, BEAM_F16, nullptr, nullptr) != BEAM_ERR_INVALID) c.fail("null A accepted");
   beam_tile_cfg small = {64, 64, 32, 32, 0, 0};
@@ -425,7 +427,7 @@ struct Problem {
   }
 };
 
-int time_op(int op, Problem& p, const beam_tile_cfg* cfg, int split_k, int warmup, int iters, float* ms) {
+int time_op(int op, Problem& p, const beam_tile_cfg* cfg, int split_k, int warmup, int iters, float* ms, int ln_mode = 0) {
   beam_problem q;
   std::memset(&q, 0, sizeof q);
   q.A = p.a.p;
@@ -439,13 +441,14 @@ int time_op(int op, Problem& p, const beam_tile_cfg* cfg, int split_k, int warmu
   q.K = p.K;
   q.dtype = p.dtype;
   q.split_k = split_k;
+  q.ln_mode = ln_mode;
   size_t need = 0;
   if (op == BEAM_OP_SPLITK) {
     const int s = beam_splitk_effective(p.M, p.N, p.K, cfg, split_k);
     if (s < 0) return BEAM_ERR_UNSUPPORTED;
     need = beam_splitk_workspace_bytes(p.M, p.N, s);
   } else if (op == BEAM_OP_GEMM_LN) {
-    need = beam_gemmrc_ln_workspace_bytes(p.M, p.N, cfg);
+    need = beam_gemmrc_ln_workspace_bytes_for(p.M, p.N, p.K, cfg, ln_mode);
   }
   DevBuf ws(need ? need : 256);
   q.ws = ws.p;
@@ -511,7 +514,9 @@ int cli_bench(const Args& a) {
     return cli_bench_silu(a, p, cfg);
   }
   float ms = 0;
-  int rc = time_op(op, p, &cfg, split, a.num("warmup", 5), a.num("iters", 20), &ms);
+  const std::string lnm = a.str("ln-mode", "auto");  // --op ln: auto | twopass | fused
+  const int ln_mode = lnm == "twopass" ? BEAM_LN_TWOPASS : lnm == "fused" ? BEAM_LN_FUSED : BEAM_LN_AUTO;
+  int rc = time_op(op, p, &cfg, split, a.num("warmup", 5), a.num("iters", 20), &ms, ln_mode);
   if (rc != BEAM_OK) {
     std::fprintf(stderr, "bench failed (%d): %s\n", rc, beam_last_error());
     return 1;

@@ -226,6 +226,7 @@ typedef struct beam_problem {
   const void* side_x;   /* BEAM_OP_GEMM_SILU, BEAM_OP_SILU                            */
   void* side_y;
   long long side_count;
+  int ln_mode;          /* BEAM_OP_GEMM_LN: a beam_ln_mode (0 = BEAM_LN_AUTO)          */
 } beam_problem;
 
 /* `warmup` untimed calls, then `iters` back-to-back calls bracketed by HIP events on `stream`;

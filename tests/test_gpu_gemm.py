@@ -249,11 +249,9 @@ def test_error_codes(gpu, beamc):
     with pytest.raises(beamc.BeamError) as e:
         beamc.gemmrc(a, b, beamc.DeviceArray((64, 32)))
     assert e.value.status == 1
-    a2 = beamc.DeviceArray((64, 12))
-    b2 = beamc.DeviceArray((64, 12))
     with pytest.raises(beamc.BeamError) as e:
-        beamc.gemmrc(a2, b2, c)
-    assert e.value.status == 2      # K % 8 != 0 has no kernel: reported, never silent
+        beamc.gemmrc_spec(a, b, c, shape_threadblock=[64, 64], shape_warp=[32, 32], pipeline=3)
+    assert e.value.status == 2
     # empty problems are no-ops, K == 0 clears C
     beamc.gemmrc(beamc.DeviceArray((0, 64)), b, beamc.DeviceArray((0, 64)))
     c.fill_bytes(0x55)

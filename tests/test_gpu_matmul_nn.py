@@ -104,9 +104,6 @@ def test_full_size_equals_gemmrc_on_transpose(gpu, beamc, oracle):
 def test_error_paths(gpu, beamc):
     a = beamc.DeviceArray((64, 64), F16)
     b = beamc.DeviceArray((64, 36), F16)
-    with pytest.raises(beamc.BeamError) as e:
-        beamc.matmul(a, b)  # N % 8 != 0
-    assert e.value.status == 2
     b2 = beamc.DeviceArray((32, 64), F16)
     with pytest.raises(beamc.BeamError):
         beamc.matmul(a, b2)  # inner dimensions differ

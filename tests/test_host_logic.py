@@ -218,8 +218,14 @@ def test_argument_validation_without_gpu(beamc):
     cfg = beamc.TileConfig(128, 128, 64, 64).to_c()
     assert L.beam_gemmrc(1 << 20, 1 << 20, 1 << 20, -1, 4, 8, 0, ctypes.byref(cfg), None) == 1
     assert L.beam_gemmrc(1 << 20, 1 << 20, 1 << 20, 4, 4, 8, 7, ctypes.byref(cfg), None) == 2      # dtype
-    assert L.beam_gemmrc(1 << 20, 1 << 20, 1 << 20, 4, 4, 12, 0, ctypes.byref(cfg), None) == 2     # K % 8
-    assert L.beam_gemmrc((1 << 20) + 2, 1 << 20, 1 << 20, 4, 4, 8, 0, ctypes.byref(cfg), None) == 2  # alignment
+    # K % 8 != 0 and operands off a 16-byte boundary are problems like any other (a plain kernel takes them):
+    # without a device the call gets as far as looking for one.  (With a device these made-up addresses must
+    # not reach a kernel: the two calls are made only where there is none.)
+    if L.beam_init() != 0:
+        assert L.beam_gemmrc(1 << 20, 1 << 20, 1 << 20, 4, 4, 12, 0, ctypes.byref(cfg), None) == 4
+        assert L.beam_gemmrc((1 << 20) + 2, 1 << 20, 1 << 20, 4, 4, 8, 0, ctypes.byref(cfg), None) == 4
+    assert L.beam_gemmrc((1 << 20) + 1, 1 << 20, 1 << 20, 4, 4, 8, 0, ctypes.byref(cfg), None) == 1  # not even element aligned
+    assert L.beam_splitk_effective(64, 64, 12, None, 8) == 1                                         # no slices for such K
     assert L.beam_gemmrc(None, 1 << 20, 1 << 20, 4, 4, 8, 0, ctypes.byref(cfg), None) == 1
     assert b"null" in L.beam_last_error()
     assert L.beam_gemmrc(None, None, None, 0, 4, 8, 0, None, None) == 0                             # empty: no-op
@@ -267,10 +273,7 @@ def test_roofline_calculator():
     assert split["ratio"] < 1 and abs(split["memory_ms"] * 1e3 - 4.21) < 0.01  # the 4.2 us HBM floor
     with pytest.raises(ValueError):
         R.gemm_bound(mi, "tf32", 64, 64, 64, 64, 64, 64)
-    # attention: the reference's example (b=2, h=24, s=4429, d=64), counted term by term as it does
-    b, h, sq, d = 2, 24, 4096 + 333, 64
-    assert R.attn_flops(b, h, sq, d) == 2 * (b * h * sq * d * sq + b * h * sq * sq * d) == 241041911808
-    assert abs(R.attn_bound_ms(mi, "bf16", b, h, sq, d) - 241041911808 / 2516.6e12 * 1e3) < 1e-9
+
 
 
 def test_ln_workspace_query_covers_every_default_call(beamc):

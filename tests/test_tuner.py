@@ -53,7 +53,7 @@ def test_tuner_picks_max_and_memoises(tuner_mod, monkeypatch, tmp_path):
     calls = []
 
     class FakeOp(tuner_mod.Operator):
-        def get_performance(self, a, b, c, warmup=5, rep=20):
+        def get_performance(self, a, b, c, warmup=5, rep=20, min_ms=0.0):
             calls.append(str(self))
             return speeds[str(self)]
 
