@@ -15,7 +15,8 @@
 //   beam_host --bench [--op gemm|splitk|ln|silu|nn] --m M --n N --k K [--dtype fp16|bf16] [--tile BMxBN]
 //             [--wave TMxTN] [--pipeline 0|1] [--group G] [--splitk S] [--iters I] [--warmup W]
 //             [--count ELEMENTS]   (silu: GEMM, SiLU alone and GEMM with the SiLU in its K loop)
-//             [--data normal|zeros] (zeros: all-zero operands, for telling schedule limits from power limits)
+//             [--data normal|uniform|zeros] (normal: N(0,1)/sqrt(K); uniform: [-1, 1); zeros: all-zero operands,
+//                                            for telling schedule limits from power limits)
 //             [--ln-mode auto|twopass|fused]   (--op ln)
 //   beam_host --tune --m M --n N --k K [--dtype fp16|bf16]
 //   beam_host --copy MiB      device-to-device copy of known size (calibrates profiler byte counters)
@@ -416,12 +417,17 @@ struct Problem {
   // zeros: A and B all zero instead of N(0,1)/sqrt(K).  The matrix cores draw far less power on zeros, so the
   // same kernel then runs at the full clock: the pair of timings separates what the schedule costs from
   // what the power cap costs.
-  Problem(int m, int n, int k, int d, bool zeros = false)
+  Problem(int m, int n, int k, int d, const std::string& data = "normal")
       : M(m), N(n), K(k), dtype(d), a((size_t)m * k * 2), b((size_t)n * k * 2), c((size_t)m * n * 2), gamma((size_t)n * 2),
         beta((size_t)n * 2) {
-    const float scale = zeros ? 0.0f : 1.0f / std::sqrt((float)k);
-    a.upload(normal16((size_t)m * k, d, 7, 0, 0.0f, scale));
-    b.upload(normal16((size_t)n * k, d, 7, 1, 0.0f, scale));
+    if (data == "uniform") {
+      a.upload(uniform16((size_t)m * k, d, 7, 0));
+      b.upload(uniform16((size_t)n * k, d, 7, 1));
+    } else {
+      const float scale = data == "zeros" ? 0.0f : 1.0f / std::sqrt((float)k);
+      a.upload(normal16((size_t)m * k, d, 7, 0, 0.0f, scale));
+      b.upload(normal16((size_t)n * k, d, 7, 1, 0.0f, scale));
+    }
     gamma.upload(normal16(n, d, 7, 2, 1.0f, 0.1f));
     beta.upload(normal16(n, d, 7, 3, 0.0f, 0.1f));
   }
@@ -507,7 +513,7 @@ int cli_bench(const Args& a) {
   cfg.pipeline = a.num("pipeline", cfg.pipeline);
   cfg.group_m = a.num("group", cfg.group_m);
   split = a.num("splitk", op == BEAM_OP_SPLITK ? 0 : split);
-  Problem p(M, N, K, dtype, a.str("data", "normal") == "zeros");
+  Problem p(M, N, K, dtype, a.str("data", "normal"));
   if (op == BEAM_OP_MATMUL_NN && cfg.pipeline == 2) cfg.pipeline = 0;
   if (opname == "silu") {
     if (cfg.pipeline == 2) cfg.pipeline = 0;
