@@ -396,7 +396,7 @@ struct GemmW4 {
       // Prologue: A and B of K tile 0, A of K tile 1 (oldest first: the first wait is about tile 0).
       TileCoord tc_cur = tile_coord(0);
       const __amdgpu_buffer_rsrc_t rows_a0 = rows_of_a(0, tc_cur), rows_b0 = rows_of_b(0, tc_cur);
-      next_a = rows_a0;  // (never used: the host sends K >= 3 tiles, so FIRST(0) sets them before any wrap)
+      next_a = rows_a0;  // (never used: K >= 3 tiles, so no stream wraps before the loop below sets them)
       next_b = rows_b0;
       ld_a = Stream{rows_a0, 0, wave * 1024};
       ld_b = Stream{rows_b0, 0, B_REGION + wave * 1024};
@@ -415,13 +415,14 @@ struct GemmW4 {
       advance(ld_a, wrap_a, next_a, 0, B_REGION, -1);
 
       for (int j = 0; j < my_tiles; ++j) {
-        k_tile(std::true_type{});
-        // From here on the accumulators belong to tile j, and the streams will move on to tile j + 1
-        // (A in the last but one K tile of tile j, B in the last).
-        out = out_tile_of(j, tc_cur);
+        // The streams move on to tile j + 1 while tile j is multiplied: A in its last but one K tile,
+        // B in its last.  With K = 3 tiles that is this very K tile, so the rows come first.
+        const TileCoord tc_j = tc_cur;
         tc_cur = tile_coord(j + 1 < my_tiles ? j + 1 : j);
         next_a = rows_of_a(j + 1, tc_cur);
         next_b = rows_of_b(j + 1, tc_cur);
+        k_tile(std::true_type{});
+        out = out_tile_of(j, tc_j);  // from here on the accumulators belong to tile j
         for (int h = 1; h < n_k; ++h) k_tile(std::false_type{});
       }
       // Drain: the second half of the last K tile is in set 1; then the last tile's output.

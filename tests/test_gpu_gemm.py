@@ -165,7 +165,7 @@ def test_fp16_sweep(gpu, beamc, oracle, shape):
     assert_close(oracle, got, ref, K, F16, f"{shape}")
 
 
-@pytest.mark.parametrize("shape", [(4200, 4296, 128), (8192, 8200, 64), (2600, 9000, 192), (4096, 4104, 256)])
+@pytest.mark.parametrize("shape", [(4200, 4296, 128), (8192, 8200, 64), (2600, 9000, 192), (4096, 4104, 256), (5000, 5000, 320)])
 def test_more_tiles_than_compute_units(gpu, beamc, oracle, shape):
     """More tiles than CUs: with 3 A + 2 B slots the large tiles run as one workgroup per CU that walks
     its tiles and prefetches the next one's operands during the store.  Ragged M and N (rows and
@@ -181,6 +181,9 @@ def test_more_tiles_than_compute_units(gpu, beamc, oracle, shape):
             once = run_gemm(beamc, a, b, dtype, beamc.TileConfig(*tile, 1, 0))
             assert_close(oracle, walk, ref, K, dtype, f"{shape} {tile}")
             assert (walk == once).all(), (shape, tile)
+        # The default tile: the 4-wavefront kernel where K >= 192 (one workgroup per CU, load streams that
+        # run ahead across tile boundaries: at K = 192 the A stream changes tile in a tile's first K tile).
+        assert_close(oracle, run_gemm(beamc, a, b, dtype), ref, K, dtype, f"{shape} default")
 
 
 def _decode(bits, dtype):
