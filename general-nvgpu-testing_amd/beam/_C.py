@@ -92,6 +92,7 @@ def _load() -> ctypes.CDLL:
     L.beam_gemmrc_ln_workspace_bytes_for.restype = sz
     L.beam_gemmrc_ln_ex.argtypes = [vp, vp, vp, vp, ctypes.c_float, vp, i, i, i, i, cfgp, i, vp, sz, vp]
     L.beam_set_ln_spin_limit.argtypes = [i]
+    L.beam_set_verbose.argtypes = [i]
     L.beam_gemmrc_ln_workspace_reset.argtypes = [vp]
     L.beam_gemmrc_ln_timed_out.argtypes = [vp, vp, ctypes.POINTER(i)]
     L.beam_parallel_gemmrc_silu.argtypes = [vp, vp, vp, i, i, i, vp, vp, ctypes.c_longlong, i, cfgp, vp]

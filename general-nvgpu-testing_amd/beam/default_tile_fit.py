@@ -1,0 +1,153 @@
+"""The cost model behind the library's default tile (beam_default_config), its timing table and its fit.
+
+The library picks a tile for a problem without measuring anything: every CU works through
+ceil(tiles / CUs) workgroups, `occ` of them at a time (what LDS allows); a workgroup costs a fixed
+start-up / epilogue time plus its flops at the per-CU rate of its tile shape, which is higher when
+several workgroups share the CU.  Three constants per candidate tile (rate alone, rate with a full CU,
+fixed cost) are fitted to `default_tile_timings.json`: microseconds per launch of every candidate on 39
+shapes from 512^3 to 8192^3 (square, skinny, short-K), fp16, N(0,1)/sqrt(K) operands, best of two rounds
+of 40 launches each, on one MI355X.  `PARAMS` below are the constants compiled into the library
+(csrc/capi.hip, kCandidates); a test keeps the two in step.
+
+    python -m beam.default_tile_fit              model's pick per shape against the table, mean / worst regret
+    python -m beam.default_tile_fit --refit      coordinate search from PARAMS (what produced them)
+    python -m beam.default_tile_fit --collect F  re-measure the table on the GPU at hand into file F
+
+This stands where the reference has fixed default shapes (cuda/cutlass_kernels/cutlass_gemmrc.cu:22-24).
+"""
+import json
+import math
+import os
+import random
+import sys
+
+CUS = 256
+TIMINGS = os.path.join(os.path.dirname(os.path.abspath(__file__)), "default_tile_timings.json")
+
+# name -> (block_m, block_n, workgroups a CU holds at once)
+CANDIDATES = {
+    "256x256_w128x64": (256, 256, 1), "224x256_w112x64": (224, 256, 1), "192x256_w96x64": (192, 256, 1),
+    "256x128_w64x64": (256, 128, 1), "128x256_w64x64": (128, 256, 1), "128x128_w64x64": (128, 128, 2),
+    "128x128_w64x32_deep": (128, 128, 1), "128x64_w64x32": (128, 64, 2), "128x64_w64x32_deep": (128, 64, 1),
+    "64x64_w32x32": (64, 64, 4), "64x64_w32x32_deep": (64, 64, 1), "64x128_w32x64": (64, 128, 2),
+    "64x128_w32x64_deep": (64, 128, 1),
+}
+# name -> (TFLOP/s per CU alone, with a full CU, fixed microseconds per workgroup slot)
+PARAMS = {
+    "256x256_w128x64": (6.04, 6.04, 8.0), "224x256_w112x64": (5.95, 5.95, 8.0), "192x256_w96x64": (5.22, 5.22, 8.0),
+    "256x128_w64x64": (4.99, 4.99, 6.0), "128x256_w64x64": (4.8, 4.8, 6.0), "128x128_w64x64": (3.8, 4.4, 3.42),
+    "128x128_w64x32_deep": (4.05, 4.05, 4.0), "128x64_w64x32": (2.6, 3.4, 3.5), "128x64_w64x32_deep": (3.2, 3.2, 4.2),
+    "64x64_w32x32": (1.87, 2.9, 2.7), "64x64_w32x32_deep": (2.4, 2.4, 4.0), "64x128_w32x64": (3.15, 3.4, 3.5),
+    "64x128_w32x64_deep": (3.3, 3.3, 4.0),
+}
+
+
+def load_timings(path=TIMINGS):
+    with open(path) as f:
+        return json.load(f)
+
+
+def predict(params, M, N, K):
+    """(modelled microseconds, candidate name) of the model's pick for a call without a workspace."""
+    best = None
+    for name, (bm, bn, occ) in CANDIDATES.items():
+        alone, full, fixed = params[name]
+        tiles = math.ceil(M / bm) * math.ceil(N / bn)
+        load = math.ceil(tiles / CUS)
+        conc = min(occ, load)
+        rate = alone if occ == 1 else alone + (full - alone) * (conc - 1) / (occ - 1)
+        mflop = 2.0e-6 * bm * bn * K
+        us = math.ceil(load / occ) * fixed + load * mflop / rate
+        if best is None or us < best[0]:
+            best = (us, name)
+    return best
+
+
+def regret(params, timings, rows=None):
+    """(geometric-mean, worst) ratio of the picked candidate's measured time to the best time of any tile."""
+    total, worst = 0.0, 0.0
+    for key, row in timings.items():
+        M, N, K = map(int, key.split("x"))
+        us, name = predict(params, M, N, K)
+        best = row["best_of_all_tiles"][1]
+        r = row["candidates"][name] / best
+        total += math.log(r)
+        worst = max(worst, r)
+        if rows is not None:
+            rows.append((key, name, row["candidates"][name], us, row["best_of_all_tiles"][0], best, r))
+    return math.exp(total / len(timings)), worst
+
+
+def refit(params, timings, steps=4000, seed=1):
+    """Coordinate search: nudge one constant at a time, keep what lowers the worst, then the mean regret."""
+    rng = random.Random(seed)
+    params = dict(params)
+    best = regret(params, timings)
+    for _ in range(steps):
+        name = rng.choice(list(params))
+        idx = rng.randrange(3)
+        old = params[name]
+        new = list(old)
+        new[idx] *= rng.choice([0.9, 0.95, 1.05, 1.1])
+        if CANDIDATES[name][2] == 1 and idx < 2:
+            new[0] = new[1] = new[idx]   # one workgroup per CU: one rate
+        params[name] = tuple(new)
+        r = regret(params, timings)
+        if (r[1], r[0]) < (best[1], best[0]) or (r[0] < best[0] and r[1] <= best[1] * 1.001):
+            best = r
+        else:
+            params[name] = old
+    return params, best
+
+
+def collect(path):
+    """Times every compiled tile (both pipeline depths) on the table's shapes on the GPU at hand."""
+    from . import _C
+    out = {}
+    for key in load_timings():
+        M, N, K = map(int, key.split("x"))
+        a = _C.DeviceArray.from_numpy(_C.host_normal((M, K), _C.F16, 1, 0, 0.0, K ** -0.5))
+        b = _C.DeviceArray.from_numpy(_C.host_normal((N, K), _C.F16, 1, 1, 0.0, K ** -0.5))
+        c = _C.DeviceArray((M, N))
+        res = {}
+        for _ in range(2):
+            for cfg in _C.list_configs():
+                for pipe in (0, 2):
+                    pc = _C.TileConfig(cfg.block_m, cfg.block_n, cfg.wave_m, cfg.wave_n, pipe, 0)
+                    try:
+                        us = _C.bench(0, a, b, c, config=pc, warmup=20, iters=40) * 1e3
+                    except _C.BeamError:
+                        continue
+                    res[pc.name] = min(res.get(pc.name, 1e9), us)
+        for x in (a, b, c):
+            x.free()
+        name = min(res, key=res.get)
+        out[key] = {"candidates": {n: round(res[n], 2) for n in CANDIDATES},
+                    "best_of_all_tiles": [name, round(res[name], 2)]}
+        print(key, out[key]["best_of_all_tiles"], flush=True)
+    with open(path, "w") as f:
+        f.write("{\n" + ",\n".join(f' "{k}": {json.dumps(v)}' for k, v in out.items()) + "\n}\n")
+
+
+def main(argv):
+    if argv[:1] == ["--collect"]:
+        collect(argv[1])
+        return 0
+    timings = load_timings()
+    params = PARAMS
+    if argv[:1] == ["--refit"]:
+        params, _ = refit(PARAMS, timings)
+        for name, p in params.items():
+            print(f"{name:22s} {p[0]:.2f} {p[1]:.2f} {p[2]:.2f}")
+    rows = []
+    mean, worst = regret(params, timings, rows)
+    print("| shape | model's pick | measured us | modelled us | best tile of all | its us | pick / best |")
+    print("|---|---|---|---|---|---|---|")
+    for key, name, t, us, bname, bt, r in rows:
+        print(f"| {key} | {name} | {t:.1f} | {us:.1f} | {bname} | {bt:.1f} | {r:.3f} |")
+    print(f"geometric mean {mean:.4f}, worst {worst:.3f} over {len(rows)} shapes")
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main(sys.argv[1:]))

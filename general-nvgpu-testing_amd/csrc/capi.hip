@@ -6,7 +6,10 @@
 #include <cstdio>
 #include <cstring>
 #include <atomic>
+#include <cstdlib>
 #include <mutex>
+#include <set>
+#include <string>
 #include <thread>
 #include <vector>
 
@@ -595,6 +598,30 @@ int beam_splitk_effective(int M, int N, int K, const beam_tile_cfg* cfg, int spl
   return effective_split(M, N, K, c, split_k);
 }
 
+// The once-per-shape line about a slice count the library chose (beam_set_verbose).
+static std::atomic<int> g_verbose{[] {
+  const char* e = getenv("BEAM_VERBOSE");
+  return e && *e && *e != '0' ? 1 : 0;
+}()};
+
+int beam_set_verbose(int verbose) {
+  g_verbose.store(verbose != 0);
+  return BEAM_OK;
+}
+
+static void log_split_choice_once(int M, int N, int K, int dtype, const beam_tile_cfg& c, int s) {
+  static std::mutex mu;
+  static std::set<std::string> seen;
+  const long tiles = (long)((M + c.block_m - 1) / c.block_m) * ((N + c.block_n - 1) / c.block_n);
+  const int cus = g_dev.cus > 0 ? g_dev.cus : 256;
+  char line[256];
+  snprintf(line, sizeof line, "split-K [%d,%d,%d] %s: tile %dx%d, %d slices of %d K elements, %ld workgroups = %.2f rounds of %d CUs",
+           M, N, K, dtype == BEAM_BF16 ? "bf16" : "fp16", c.block_m, c.block_n, s, split_k_len(K, s), tiles * s,
+           (double)(tiles * s) / cus, cus);
+  std::lock_guard<std::mutex> lock(mu);
+  if (seen.insert(line).second) fprintf(stderr, "[beam] %s\n", line);
+}
+
 int beam_gemmrc_splitk(const void* A, const void* B, void* C, int M, int N, int K, int dtype,
                        const beam_tile_cfg* cfg, int split_k, void* ws, size_t ws_bytes, void* stream) {
   bool generic;
@@ -615,6 +642,7 @@ int beam_gemmrc_splitk(const void* A, const void* B, void* C, int M, int N, int 
   const KernelSet* ks;
   if ((rc = resolve_cfg(cfg, M, N, K, &c, &ks, split_k > 0 ? split_k : 0))) return rc;
   const int s = effective_split(M, N, K, c, split_k);
+  if (split_k <= 0 && g_verbose.load(std::memory_order_relaxed)) log_split_choice_once(M, N, K, dtype, c, s);
   if (s == 1) {  // nothing to reduce: the plain kernel writes C directly
     GemmParams p = base_params(A, B, M, N, K, c);
     p.C = C;

@@ -105,6 +105,12 @@ int beam_gemmrc_splitk(const void* A, const void* B, void* C, int M, int N, int 
                        void* stream);
 /* The effective split factor beam_gemmrc_splitk would use for these arguments. */
 int beam_splitk_effective(int M, int N, int K, const beam_tile_cfg* cfg, int split_k);
+/* verbose != 0: when the library chooses the slice count itself, beam_gemmrc_splitk writes one line to
+ * stderr the first time it sees a (shape, dtype, tile): the tile, the slice count, the workgroups that
+ * makes and how many rounds of the device's CUs they are.  Off by default; the environment variable
+ * BEAM_VERBOSE=1 turns it on at load.  Stands in for the once-per-shape "[INFO] ... split_k(..), CTAs(..),
+ * waves(..)" line of cuda/cutlass_kernels/cutlass_gemmrc_splitk.cu:12-24,87-93. */
+int beam_set_verbose(int verbose);
 /* beam_gemmrc_splitk without a workspace argument and without any allocation: the fp32 partial sums go
  * into device memory built into the library (a fixed array of beam_splitk_noalloc_max_bytes() = 16 MiB
  * per GPU, present from the first call into the library until the process ends).  No counterpart in

@@ -84,3 +84,30 @@ def test_splitk_workspace_errors(gpu, beamc):
     assert rc == 3
     assert b"workspace" in beamc.lib.beam_last_error()
     assert beamc.lib.beam_splitk_workspace_bytes(256, 256, 8) == 8 * 256 * 256 * 4
+
+
+def test_splitk_choice_is_logged_once_per_shape(gpu, beamc, capfd):
+    """With the library choosing the slice count, a verbose library reports its choice once per shape
+    (the reference's once-per-shape "[INFO] ... split_k(..), CTAs(..), waves(..)" line,
+    cuda/cutlass_kernels/cutlass_gemmrc_splitk.cu:12-24,87-93), and a quiet one (the default) never."""
+    M, N, K = 128, 192, 16384
+    a = beamc.DeviceArray.from_numpy(beamc.host_uniform((M, K), F16, 3, 0), F16)
+    b = beamc.DeviceArray.from_numpy(beamc.host_uniform((N, K), F16, 3, 1), F16)
+    c = beamc.DeviceArray((M, N), F16)
+    capfd.readouterr()
+    beamc.gemmrc_splitk(a, b, c)
+    assert "[beam]" not in capfd.readouterr().err
+    assert beamc.lib.beam_set_verbose(1) == 0
+    try:
+        for _ in range(3):
+            beamc.gemmrc_splitk(a, b, c)
+        beamc.gemmrc_splitk(a, b, c, split_k_slices=4)   # a slice count the caller gave is not a decision
+        err = capfd.readouterr().err
+    finally:
+        beamc.lib.beam_set_verbose(0)
+    lines = [l for l in err.splitlines() if l.startswith("[beam] split-K")]
+    assert len(lines) == 1, err
+    s = beamc.lib.beam_splitk_effective(M, N, K, None, 0)
+    assert f"[{M},{N},{K}]" in lines[0] and f"{s} slices" in lines[0] and "workgroups" in lines[0] and "rounds" in lines[0]
+    for x in (a, b, c):
+        x.free()
