@@ -172,10 +172,20 @@ def extra_splitk(_C):
     # what a call that names neither tile nor slice count gets
     auto_cfg, auto_s = _C.default_config(M, N, K, split=True)
     auto_ms = min(_C.bench(1, a, b, c, config=None, split_k=0, warmup=20, iters=100) for _ in range(2))
+    # what the machine allows for this launch shape: empty launches, and the chosen partial kernel with
+    # nothing but its global->LDS loads and fragment reads (no MFMA, no store, no reduction)
+    floor = {"empty_kernel_us": round(min(_C.bench(_C.OP_PROBE_EMPTY, a, b, c, warmup=50, iters=500) for _ in range(2)) * 1e3, 2),
+             "two_empty_kernels_us": round(min(_C.bench(_C.OP_PROBE_EMPTY_PAIR, a, b, c, warmup=50, iters=500) for _ in range(2)) * 1e3, 2)}
+    try:
+        floor["partial_kernel_loads_only_us"] = round(min(
+            _C.bench(_C.OP_PROBE_SPLITK_LOADS, a, b, c, config=None, split_k=0, warmup=20, iters=100) for _ in range(2)) * 1e3, 2)
+    except _C.BeamError as e:   # the probe is built for the tiles the library picks at this shape
+        floor["partial_kernel_loads_only_us"] = None
+        floor["note"] = str(e)
     for x in (a, b, c):
         x.free()
     bytes_alg = 2.0 * (M * K + N * K + M * N)
-    return {"shape": [M, N, K], "splitk_us": round(best_split[1] * 1e3, 2), "splitk_config": best_split[0],
+    return {"shape": [M, N, K], "splitk_us": round(best_split[1] * 1e3, 2), "splitk_config": best_split[0], "floor": floor,
             "splitk_in_graph_us": round(graph_us, 2), "splitk_cold_operands_us": round(cold_us, 2),
             "cold_hbm_GBs": round(2.0 * (M * K + N * K + M * N) / (cold_us * 1e-6) / 1e9, 1),
             "library_choice_us": round(auto_ms * 1e3, 2), "library_choice": f"{auto_cfg.name},S={auto_s}",

@@ -483,6 +483,8 @@ cutlass_parallel_gemmrc_lnr = parallel_gemmrc_silu
 
 
 OP_GEMM, OP_SPLITK, OP_GEMM_LN, OP_GEMM_SILU, OP_SILU, OP_MATMUL_NN = 0, 1, 2, 3, 4, 5
+# launches that measure what the machine allows: an empty kernel, two of them, a split-K launch with only its loads
+OP_PROBE_EMPTY, OP_PROBE_EMPTY_PAIR, OP_PROBE_SPLITK_LOADS = 6, 7, 8
 
 
 def bench(op: int, a, b, c, config: Optional[TileConfig] = None, split_k: int = 0, gamma=None, beta=None,
@@ -502,7 +504,7 @@ def bench(op: int, a, b, c, config: Optional[TileConfig] = None, split_k: int = 
     if op in (OP_GEMM_SILU, OP_SILU):
         q.side_x, q.side_y, q.side_count, _, _ = _flat_pair(x, y, d)
     ws = None
-    if op == 1:
+    if op in (OP_SPLITK, OP_PROBE_SPLITK_LOADS):
         s = lib.beam_splitk_effective(M, N, K, cfgp, split_k)
         if s < 0:
             raise BeamError(2, lib.beam_last_error().decode())

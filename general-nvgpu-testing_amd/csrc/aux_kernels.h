@@ -39,6 +39,8 @@ hipError_t launch_silu(const void* x, void* y, size_t count, int dtype, hipStrea
 hipError_t launch_zero_u16(void* p, size_t n, hipStream_t stream);
 // ints[0 .. n) = 0 (a fill kernel rather than hipMemsetAsync, so that callers may capture it in a graph).
 hipError_t launch_zero_ints(int* ints, int n, hipStream_t stream);
+// A kernel that does nothing, `workgroups` x `threads`: what a launch costs from submission to completion.
+hipError_t launch_empty(int workgroups, int threads, hipStream_t stream);
 // floats[0 .. n) = value
 hipError_t launch_fill_floats(float* floats, size_t n, float value, hipStream_t stream);
 

@@ -254,6 +254,10 @@ __global__ void __launch_bounds__(1024) ln_prepare_kernel(int* hdr, float* sets,
   }
 }
 
+__global__ void empty_kernel(int* p) {
+  if (p && threadIdx.x == 0x7fffffff) *p = 1;  // never true: keeps the argument alive
+}
+
 __global__ void zero_u16_kernel(unsigned short* p, size_t n) {
   for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) p[i] = 0;
 }
@@ -328,6 +332,11 @@ hipError_t launch_zero_u16(void* p, size_t n, hipStream_t stream) {
   if (blocks < 1) blocks = 1;
   if (blocks > 4096) blocks = 4096;
   hipLaunchKernelGGL(zero_u16_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, (unsigned short*)p, n);
+  return hipGetLastError();
+}
+
+hipError_t launch_empty(int workgroups, int threads, hipStream_t stream) {
+  hipLaunchKernelGGL(empty_kernel, dim3((unsigned)workgroups), dim3((unsigned)threads), 0, stream, (int*)nullptr);
   return hipGetLastError();
 }
 

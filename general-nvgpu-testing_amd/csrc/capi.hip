@@ -895,6 +895,29 @@ int beam_gemmrc_ln_timed_out(const void* ws, void* stream, int* timed_out) {
   return BEAM_OK;
 }
 
+// BEAM_OP_PROBE_SPLITK_LOADS: the launch of beam_gemmrc_splitk's partial kernel, resolved the same way.
+static int probe_splitk_loads(const beam_problem* q, const beam_tile_cfg* cfg, hipStream_t st) {
+  bool generic;
+  int rc = check_problem(q->A, q->B, q->C, q->M, q->N, q->K, q->dtype, &generic);
+  if (rc) return rc;
+  if ((rc = beam_init())) return rc;
+  if (generic || q->dtype != BEAM_F16 || q->M == 0 || q->N == 0 || q->K == 0)
+    return fail(BEAM_ERR_UNSUPPORTED, "the load probe is built for fp16 problems of the tiled kernels");
+  beam_tile_cfg c;
+  const KernelSet* ks;
+  if ((rc = resolve_cfg(cfg, q->M, q->N, q->K, &c, &ks, q->split_k > 0 ? q->split_k : 0))) return rc;
+  const bool built = c.pipeline == 2 && c.block_m == 64 && ((c.block_n == 128 && c.wave_m == 32 && c.wave_n == 64) ||
+                                                            (c.block_n == 64 && c.wave_m == 32 && c.wave_n == 32));
+  if (!built) return fail(BEAM_ERR_UNSUPPORTED, "the load probe is built for the deep 64x128 (wave 32x64) and 64x64 (wave 32x32) tiles");
+  const int s = effective_split(q->M, q->N, q->K, c, q->split_k);
+  GemmParams p = base_params(q->A, q->B, q->M, q->N, q->K, c);
+  p.ws = (float*)q->ws;  // never written
+  p.k_slice = split_k_len(q->K, s);
+  p.splits = s;
+  BEAM_HIP(launch_probe_splitk_loads(p, c.block_m, c.block_n, dim3((unsigned)(p.tiles_m * p.tiles_n * s), 1, 1), st));
+  return BEAM_OK;
+}
+
 int beam_bench(int op, const beam_problem* q, const beam_tile_cfg* cfg, int warmup, int iters, void* stream,
                float* avg_ms) {
   if (!q || !avg_ms || iters < 1 || warmup < 0) return fail(BEAM_ERR_INVALID, "bad bench arguments");
@@ -915,6 +938,16 @@ int beam_bench(int op, const beam_problem* q, const beam_tile_cfg* cfg, int warm
         return beam_matmul_nn(q->A, q->B, q->C, q->M, q->N, q->K, q->dtype, cfg, stream);
       case BEAM_OP_SILU:
         return beam_silu(q->side_x, q->side_y, q->side_count, q->dtype, stream);
+      case BEAM_OP_PROBE_EMPTY:
+      case BEAM_OP_PROBE_EMPTY_PAIR: {
+        int rc = beam_init();
+        if (rc) return rc;
+        BEAM_HIP(launch_empty(256, 256, (hipStream_t)stream));
+        if (op == BEAM_OP_PROBE_EMPTY_PAIR) BEAM_HIP(launch_empty(1024, 64, (hipStream_t)stream));
+        return BEAM_OK;
+      }
+      case BEAM_OP_PROBE_SPLITK_LOADS:
+        return probe_splitk_loads(q, cfg, (hipStream_t)stream);
       default:
         return fail(BEAM_ERR_INVALID, "unknown op %d", op);
     }

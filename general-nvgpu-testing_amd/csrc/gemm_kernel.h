@@ -87,8 +87,12 @@ enum Epilogue : int {
   // kEpiStore for a grid smaller than the tile count: a workgroup walks the tiles id, id + grid, ...
   // and has the first operand tiles of the next one in flight while it stores the current one
   kEpiStoreLoop = 5,
+  // Measurement only (beam_bench's BEAM_OP_PROBE_SPLITK_LOADS; not in the launch tables): the K loop of
+  // kEpiPartial with its global->LDS loads and fragment reads but without MFMAs, and nothing stored.
+  // What such a launch costs is the floor that the loads of a split-K launch shape set by themselves.
+  kEpiProbeLoads = 6,
 };
-constexpr int kNumEpilogues = 6;
+constexpr int kNumEpilogues = 6;  // epilogues of the launch tables
 
 struct GemmParams {
   const void* A;
@@ -554,7 +558,8 @@ struct GemmTile {
           // the power cap in a register-only loop, 1% here).  A wavefront that has its SIMD to itself
           // loses 5-7% that way (measured), so 4-wavefront tiles keep the plain order.
           const int j = (NW >= 8 && (i & 1)) ? FN - 1 - jj : jj;
-          acc[i][j] = Traits::mfma(fb_cur[j], fa_cur[i], acc[i][j]);
+          if constexpr (EPI == kEpiProbeLoads) asm volatile("" ::"v"(fb_cur[j]), "v"(fa_cur[i]));  // fragments stay live
+          else acc[i][j] = Traits::mfma(fb_cur[j], fa_cur[i], acc[i][j]);
         }
         if constexpr (SIDE && LD && ROW0 != 0) {  // step 1: this row's share of the side vectors
           // pairs are dealt to every (FM / SIDE_PAIRS)-th row, or several to a row of a short step
@@ -671,7 +676,10 @@ struct GemmTile {
 #pragma unroll
       for (int i = 0; i < FM; ++i)
 #pragma unroll
-        for (int j = 0; j < FN; ++j) acc[i][j] = Traits::mfma(fb1[j], fa1[i], acc[i][j]);
+        for (int j = 0; j < FN; ++j) {
+          if constexpr (EPI == kEpiProbeLoads) asm volatile("" ::"v"(fb1[j]), "v"(fa1[i]));
+          else acc[i][j] = Traits::mfma(fb1[j], fa1[i], acc[i][j]);
+        }
     };
     if (n_tiles > 0) {
       issue_prologue();
@@ -1111,6 +1119,7 @@ struct GemmTile {
           st[1] = row_stats[rl * 2 + 1];
         }
       }
+      if constexpr (EPI == kEpiProbeLoads) return;
       // fp32 tile: split-K partial sums of this slice, or X for the normalisation pass.
       float* W = p.ws + (EPI == kEpiPartial ? (size_t)slice * M * N : (size_t)0);
 #pragma unroll

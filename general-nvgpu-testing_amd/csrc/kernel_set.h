@@ -122,5 +122,9 @@ hipError_t launch_gemm_w4(const GemmParams& p, int dtype, dim3 grid, hipStream_t
 // Its fused GEMM+LayerNorm form: one workgroup per tile, grid and parameters as for the kEpiLnFused kernels;
 // gamma and beta 16-byte aligned as well.
 hipError_t launch_gemm_w4_ln(const GemmParams& p, int dtype, dim3 grid, hipStream_t stream);
+// Measurement only: the split-K partial kernel of the 64 x 128 (wave 32 x 64) or 64 x 64 (wave 32 x 32) tile, deep
+// pipeline, fp16, with its loads and fragment reads but no MFMAs and no stores (kEpiProbeLoads); hipErrorInvalidValue
+// for any other tile.
+hipError_t launch_probe_splitk_loads(const GemmParams& p, int block_m, int block_n, dim3 grid, hipStream_t stream);
 
 }  // namespace beam

@@ -18,6 +18,8 @@
 //             [--data normal|uniform|zeros] (normal: N(0,1)/sqrt(K); uniform: [-1, 1); zeros: all-zero operands,
 //                                            for telling schedule limits from power limits)
 //             [--ln-mode auto|twopass|fused]   (--op ln)
+//             --op probe-empty | probe-empty-pair | probe-splitk-loads: launches that measure what the machine
+//             allows (an empty kernel, two of them, the split-K partial kernel with nothing but its loads)
 //   beam_host --tune --m M --n N --k K [--dtype fp16|bf16]
 //   beam_host --copy MiB      device-to-device copy of known size (calibrates profiler byte counters)
 #include <cmath>
@@ -449,7 +451,7 @@ int time_op(int op, Problem& p, const beam_tile_cfg* cfg, int split_k, int warmu
   q.split_k = split_k;
   q.ln_mode = ln_mode;
   size_t need = 0;
-  if (op == BEAM_OP_SPLITK) {
+  if (op == BEAM_OP_SPLITK || op == BEAM_OP_PROBE_SPLITK_LOADS) {
     const int s = beam_splitk_effective(p.M, p.N, p.K, cfg, split_k);
     if (s < 0) return BEAM_ERR_UNSUPPORTED;
     need = beam_splitk_workspace_bytes(p.M, p.N, s);
@@ -504,15 +506,20 @@ int cli_bench(const Args& a) {
   const int op = opname == "splitk" ? BEAM_OP_SPLITK
                  : opname == "ln"   ? BEAM_OP_GEMM_LN
                  : opname == "nn"   ? BEAM_OP_MATMUL_NN  // B read as [K][N]
-                                    : BEAM_OP_GEMM;
+                 // what the machine allows: empty launches, and a split-K launch with nothing but its loads
+                 : opname == "probe-empty"        ? BEAM_OP_PROBE_EMPTY
+                 : opname == "probe-empty-pair"   ? BEAM_OP_PROBE_EMPTY_PAIR
+                 : opname == "probe-splitk-loads" ? BEAM_OP_PROBE_SPLITK_LOADS
+                                                  : BEAM_OP_GEMM;
+  const bool splitk_like = op == BEAM_OP_SPLITK || op == BEAM_OP_PROBE_SPLITK_LOADS;
   beam_tile_cfg cfg;
   int split = 1;
-  if (beam_default_config(M, N, K, &cfg, op == BEAM_OP_SPLITK ? &split : nullptr) != BEAM_OK) return 2;
+  if (beam_default_config(M, N, K, &cfg, splitk_like ? &split : nullptr) != BEAM_OK) return 2;
   if (a.has("tile") && !parse_pair(a.str("tile", ""), &cfg.block_m, &cfg.block_n)) return 2;
   if (a.has("wave") && !parse_pair(a.str("wave", ""), &cfg.wave_m, &cfg.wave_n)) return 2;
   cfg.pipeline = a.num("pipeline", cfg.pipeline);
   cfg.group_m = a.num("group", cfg.group_m);
-  split = a.num("splitk", op == BEAM_OP_SPLITK ? 0 : split);
+  split = a.num("splitk", splitk_like ? 0 : split);
   Problem p(M, N, K, dtype, a.str("data", "normal"));
   if (op == BEAM_OP_MATMUL_NN && cfg.pipeline == 2) cfg.pipeline = 0;
   if (opname == "silu") {

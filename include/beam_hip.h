@@ -215,7 +215,13 @@ typedef enum beam_op {
   BEAM_OP_GEMM_LN = 2,
   BEAM_OP_GEMM_SILU = 3, /* beam_parallel_gemmrc_silu */
   BEAM_OP_SILU = 4,      /* beam_silu alone            */
-  BEAM_OP_MATMUL_NN = 5  /* beam_matmul_nn             */
+  BEAM_OP_MATMUL_NN = 5, /* beam_matmul_nn             */
+  /* Not operators: launches that measure what the machine allows (no counterpart in the reference). */
+  BEAM_OP_PROBE_EMPTY = 6,        /* one empty kernel of 256 workgroups x 256 threads                */
+  BEAM_OP_PROBE_EMPTY_PAIR = 7,   /* two empty kernels in a row (256 x 256, then 1024 x 64 threads)   */
+  BEAM_OP_PROBE_SPLITK_LOADS = 8  /* the partial kernel of BEAM_OP_SPLITK for the same arguments with its
+                                     loads and LDS reads but no MFMAs and no stores, and no reduction;
+                                     fp16, tiles 64x128 (wave 32x64) and 64x64 (wave 32x32), pipeline 2 */
 } beam_op;
 
 typedef struct beam_problem {
@@ -255,9 +261,9 @@ int beam_event_destroy(void* event);
  * for launch-bound loops of small GEMMs (a split-K call is two kernels of 13 and 5 us).  The reference
  * has no counterpart (it launches on the legacy default stream, cuda/cute_kernels/cute_gemm_128x128.cu:
  * 203).  Rules: call every operator once eagerly before capturing it (the first launch of a kernel
- * configures its LDS size); the fused GEMM+LayerNorm keeps launch-to-launch state in its workspace and is
- * refused under capture (BEAM_LN_AUTO takes the two-pass path there); K = 0 clears C with a kernel, not
- * a memset node.  Streams are created at the default priority. */
+ * configures its LDS size); BEAM_LN_AUTO takes the two-pass path under capture (BEAM_LN_FUSED is honoured:
+ * the workspace's epoch moves on inside the captured launches); K = 0 clears C with a kernel, not a
+ * memset node.  Streams are created at the default priority. */
 int beam_stream_create(void** stream);
 int beam_stream_destroy(void* stream);
 int beam_graph_begin_capture(void* stream);               /* not the default stream */

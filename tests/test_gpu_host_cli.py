@@ -38,3 +38,24 @@ def test_cli_bench_and_info(gpu):
     assert r.returncode == 0 and r.stdout.startswith("nn 512x1024x768"), r.stdout + r.stderr
     r = run("--bench", "--tile", "100x100")
     assert r.returncode != 0
+
+
+def _ms(stdout):
+    return float(stdout.split(":")[-1].split("ms")[0])
+
+
+def test_cli_launch_floor_probes(gpu):
+    """The launches that measure what the machine allows for split-K at 256 x 256 x 32768: an empty kernel, two
+    of them, and the library's partial kernel with nothing but its loads.  They run, leave C alone, and are
+    ordered as they must be: one empty launch <= two, loads only <= the whole split-K call."""
+    shape = ["--m", "256", "--n", "256", "--k", "32768", "--data", "uniform", "--iters", "200", "--warmup", "50"]
+    t = {}
+    for op in ("probe-empty", "probe-empty-pair", "probe-splitk-loads", "splitk"):
+        r = run("--bench", "--op", op, *shape)
+        assert r.returncode == 0 and r.stdout.startswith(op), r.stdout + r.stderr
+        t[op] = _ms(r.stdout)
+    assert 0 < t["probe-empty"] <= t["probe-empty-pair"] * 1.05
+    assert t["probe-empty"] < t["probe-splitk-loads"] <= t["splitk"] * 1.05, t
+    # a tile the probe is not built for is refused, not run as something else
+    r = run("--bench", "--op", "probe-splitk-loads", "--tile", "128x128", "--wave", "64x64", *shape)
+    assert r.returncode != 0 and "probe" in r.stderr
