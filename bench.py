@@ -340,7 +340,9 @@ def main():
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(achieved / PEAK_TFLOPS, 4), "traffic": profiled_traffic_bytes(),
                      "traffic_source": "profiles/" + os.path.basename(HEADLINE_PROFILE) + " (rocprofv3 counter runs, not this run)",
-                     "kernel_ms": round(kern_ms, 4)},
+                     "kernel_ms": round(kern_ms, 4),
+                     # the same kernel, same process, once the clock has settled (see extra.headline_steady)
+                     "achieved_steady": steady["TFLOPs"], "frac_steady": steady["frac"]},
     }
     if not args.no_cpu:
         rec, ref, O = cpu_baseline(a_bits, b_bits, M, N, K)
