@@ -17,11 +17,9 @@ hipError_t launch_ln_apply(const float* X, const float* stats, const void* gamma
                            void* Y, int M, int N, int tiles_n, int block_n, float eps, int dtype,
                            hipStream_t stream);
 
-// Stream-ordered preparation of a fused GEMM+LayerNorm workspace (header of 64 ints + two statistics sets of
-// set_floats_total / 2 floats each) for its next launch: validates the header on the device and either
-// advances the epoch or re-initialises everything.
-hipError_t launch_ln_prepare(int* header, float* sets, size_t set_floats_total, int geom_lo, int geom_hi, int expected,
-                             hipStream_t stream);
+// One thread moves on the replay counter in the header of a fused GEMM+LayerNorm workspace: recorded in front
+// of a fused launch when the stream is being captured (see ln_launch_tag in gemm_kernel.h).
+hipError_t launch_ln_replay_bump(int* header, hipStream_t stream);
 
 // gemmrc without any condition on K, N or alignment (slow; what the tiled kernels refuse runs here):
 // C[M][N] = A[M][K] . B^T with B as [N][K], or as [K][N] when b_kmajor; C 16-bit, or fp32 when out_fp32.

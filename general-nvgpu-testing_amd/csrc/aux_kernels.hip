@@ -226,33 +226,10 @@ __global__ void __launch_bounds__(256) ln_rows_kernel(const float* __restrict__ 
   for (int n = threadIdx.x; n < N; n += 256) y[n] = (T)((x[n] - mean) * rstd * (float)gamma[n] + (float)beta[n]);
 }
 
-// Before every fused GEMM+LayerNorm launch: decide, on the device, whether the workspace is in the state the
-// previous fused launch left it in -- header intact, same geometry, and every workgroup of that launch
-// finished (each of them has marked its slots of the other statistics set "not published") -- and then
-// just move on to the next epoch; otherwise mark both sets "not published" (M2 = -1) and start at epoch 0.
-// One workgroup: the decision and the header update are then trivially ordered around the fill.
-__global__ void __launch_bounds__(1024) ln_prepare_kernel(int* hdr, float* sets, size_t set_floats_total, int geom_lo,
-                                                           int geom_hi, int expected) {
-  __shared__ int valid;
-  if (threadIdx.x == 0)
-    valid = hdr[kLnHdrMagic] == kLnMagic && hdr[kLnHdrGeometry] == geom_lo && hdr[kLnHdrGeometry + 1] == geom_hi &&
-            hdr[kLnHdrExpected] == expected && hdr[kLnHdrDone] == expected;
-  __syncthreads();
-  if (!valid) {
-    const f32x4 unpublished = {-1.0f, -1.0f, -1.0f, -1.0f};
-    for (size_t i = threadIdx.x; i < set_floats_total / 4; i += blockDim.x) ((f32x4*)sets)[i] = unpublished;
-    __syncthreads();
-  }
-  if (threadIdx.x == 0) {
-    hdr[kLnHdrTimeout] = 0;
-    hdr[kLnHdrMagic] = kLnMagic;
-    hdr[kLnHdrGeometry] = geom_lo;
-    hdr[kLnHdrGeometry + 1] = geom_hi;
-    hdr[kLnHdrEpoch] = valid ? hdr[kLnHdrEpoch] + 1 : 0;
-    hdr[kLnHdrDone] = 0;
-    hdr[kLnHdrExpected] = expected;
-  }
-}
+// In front of a fused GEMM+LayerNorm launch that is being recorded into a graph: the launch's arguments, its
+// nonce among them, repeat from replay to replay, so the part of its tag that changes is this counter in the
+// workspace header.  Whatever the word held before, it holds something else afterwards.
+__global__ void ln_replay_bump_kernel(int* hdr) { hdr[kLnHdrReplay] = hdr[kLnHdrReplay] + 1; }
 
 __global__ void empty_kernel(int* p) {
   if (p && threadIdx.x == 0x7fffffff) *p = 1;  // never true: keeps the argument alive
@@ -320,10 +297,8 @@ hipError_t launch_ln_rows(const float* X, const void* gamma, const void* beta, v
   return hipGetLastError();
 }
 
-hipError_t launch_ln_prepare(int* header, float* sets, size_t set_floats_total, int geom_lo, int geom_hi, int expected,
-                             hipStream_t stream) {
-  hipLaunchKernelGGL(ln_prepare_kernel, dim3(1), dim3(1024), 0, stream, header, sets, set_floats_total, geom_lo, geom_hi,
-                     expected);
+hipError_t launch_ln_replay_bump(int* header, hipStream_t stream) {
+  hipLaunchKernelGGL(ln_replay_bump_kernel, dim3(1), dim3(1), 0, stream, header);
   return hipGetLastError();
 }
 

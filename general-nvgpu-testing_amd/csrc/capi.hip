@@ -6,12 +6,15 @@
 #include <cstdio>
 #include <cstring>
 #include <atomic>
+#include <chrono>
 #include <cstdlib>
 #include <mutex>
 #include <set>
 #include <string>
 #include <thread>
 #include <vector>
+
+#include <unistd.h>
 
 #include "../../include/beam_hip.h"
 #include "aux_kernels.h"
@@ -53,6 +56,10 @@ Device g_dev;
 std::mutex g_dev_mu;
 // polls of statistics slots (about a microsecond each) before a thread of a fused LayerNorm workgroup gives up
 std::atomic<int> g_ln_spin_limit{4 << 20};
+// Nonces of fused GEMM+LayerNorm launches: consecutive numbers from a start that differs from process to process
+// (memory recycled from another process of this library then holds tags of another sequence).
+std::atomic<unsigned> g_ln_nonce{(unsigned)std::chrono::steady_clock::now().time_since_epoch().count() * 2654435761u ^
+                                 (unsigned)getpid() * 40503u};
 
 // Split-K workspace of beam_gemmrc_splitk_noalloc: device memory that exists from the moment the library's
 // code is loaded on a GPU until the process ends, so the entry point never allocates.  In host code the
@@ -682,12 +689,11 @@ int beam_gemmrc_splitk_noalloc(const void* A, const void* B, void* C, int M, int
   return beam_gemmrc_splitk(A, B, C, M, N, K, dtype, cfg, split_k, ws, kScratchBytes, stream);
 }
 
-// Fused GEMM+LayerNorm workspace: [header, 256 bytes | statistics set 0 | statistics set 1].  The header
-// (tile_map.h: kLnHdr*) carries a magic word, the geometry the sets are laid out for, the epoch whose parity
-// selects the set of a launch, and how many workgroups of the latest launch have finished; a small kernel in
-// front of every fused launch checks it on the device and re-initialises the workspace when anything is off
-// (first use, another geometry, a buffer handed out again by an allocator, an interrupted launch).  The
-// library keeps no host-side state about workspaces.
+// Fused GEMM+LayerNorm workspace: [header, 256 bytes | (mean, tag) words | (M2, ~tag) words], one word of
+// each kind per (row band, column tile, row).  Nothing in it is ever prepared or cleared: every fused launch
+// gets a nonce that no earlier launch of this process had, and the kernel takes a statistics word for
+// published only if it carries the tag made from that nonce (gemm_kernel.h: ln_launch_tag).  The library keeps
+// no state about workspaces on the host either.
 static size_t ln_fused_header_bytes() { return 256; }
 static size_t ln_fused_set_bytes(size_t tiles_m, size_t tiles_n, int block_m) {
   return align_up(tiles_m * tiles_n * (size_t)block_m * 2 * sizeof(float), 256);
@@ -823,8 +829,9 @@ int beam_gemmrc_ln_ex(const void* A, const void* B, const void* gamma, const voi
     // Launches that share a workspace must be ordered (same stream): overlapping ones would race on the sets.
     const size_t set_bytes = ln_fused_set_bytes(p.tiles_m, p.tiles_n, c.block_m);
     float* sets = (float*)((char*)ws + ln_fused_header_bytes());
-    BEAM_HIP(launch_ln_prepare((int*)ws, sets, 2 * set_bytes / sizeof(float), p.tiles_m, (p.tiles_n << 12) | c.block_m,
-                               p.tiles_m * p.tiles_n, st));
+    // A recorded launch repeats its arguments on every replay: the counter in the header then makes the tag new.
+    if (capturing != hipStreamCaptureStatusNone) BEAM_HIP(launch_ln_replay_bump((int*)ws, st));
+    p.ln_nonce = g_ln_nonce.fetch_add(1, std::memory_order_relaxed) + 1;
     p.stats = sets;
     p.next_stats = (float*)((char*)sets + set_bytes);
     p.timeout_flag = (int*)ws;
@@ -876,7 +883,7 @@ int beam_gemmrc_ln(const void* A, const void* B, const void* gamma, const void* 
 
 int beam_gemmrc_ln_workspace_reset(const void* ws) {
   if (!ws) return fail(BEAM_ERR_INVALID, "null workspace");
-  BEAM_HIP(hipMemset(const_cast<void*>(ws), 0, ln_fused_header_bytes()));  // no magic word: the next launch starts over
+  BEAM_HIP(hipMemset(const_cast<void*>(ws), 0, ln_fused_header_bytes()));  // forgets a recorded time-out; never needed
   return BEAM_OK;
 }
 
@@ -889,9 +896,10 @@ int beam_set_ln_spin_limit(int polls) {
 int beam_gemmrc_ln_timed_out(const void* ws, void* stream, int* timed_out) {
   if (!ws || !timed_out) return fail(BEAM_ERR_INVALID, "null argument");
   BEAM_HIP(hipStreamSynchronize((hipStream_t)stream));
-  int hdr[2] = {0, 0};
+  int hdr[4] = {0, 0, 0, 0};
   BEAM_HIP(hipMemcpy(hdr, ws, sizeof hdr, hipMemcpyDeviceToHost));
-  *timed_out = (hdr[kLnHdrMagic] == kLnMagic) ? hdr[kLnHdrTimeout] : 0;  // no fused launch has prepared this workspace
+  // the header speaks of a fused launch at all, and the launch that gave up is the latest one
+  *timed_out = hdr[kLnHdrMagic] == kLnMagic && hdr[kLnHdrLaunchTag] != 0 && hdr[kLnHdrTimeout] == hdr[kLnHdrLaunchTag];
   return BEAM_OK;
 }
 

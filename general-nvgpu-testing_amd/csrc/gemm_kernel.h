@@ -100,14 +100,11 @@ struct GemmParams {
   void* C;       // 16-bit [M][N]                                  (kEpiStore)
   float* ws;     // fp32 [splits][M][N] (kEpiPartial) or fp32 [M][N] (kEpiLnStats)
   float* stats;  // fp32 [M][tiles_n][2] = (mean, M2) over the tile's columns (kEpiLnStats)
-                 // kEpiLnFused: statistics set 0, fp32 [tiles_m][tiles_n][BM][2]; launches alternate between
-                 // two sets by the parity of the workspace's epoch; every M2 of a launch's set is -1 ("not
-                 // published") when it starts, and it leaves the other set like that for its successor
-  float* next_stats;    // kEpiLnFused: statistics set 1
-  // kEpiLnFused: the workspace header, kept by ln_prepare_kernel (aux_kernels.hip):
-  //   [0] set to 1 if a bounded wait ran out (never expected)   [4] epoch of this launch
-  //   [5] workgroups of this launch that have finished
+                 // kEpiLnFused: 8-byte words [tiles_m][tiles_n][BM] = (mean, tag of the launch that wrote it)
+  float* next_stats;    // kEpiLnFused: 8-byte words [tiles_m][tiles_n][BM] = (M2, ~tag)
+  // kEpiLnFused: the workspace header (tile_map.h: kLnHdr*); never has to be initialised
   int* timeout_flag;
+  unsigned ln_nonce;    // kEpiLnFused: a number no earlier launch of this process had (see ln_launch_tag)
   const void* gamma;    // 16-bit [N]                                                   (kEpiLnFused)
   const void* beta;     // 16-bit [N]
   float eps;
@@ -130,6 +127,82 @@ struct GemmParams {
   int side_width;        // bytes per unit
   int c_streaming;       // kEpiStoreLoop: store C non-temporal
 };
+
+// ---- statistics exchange of the fused GEMM+LayerNorm (both K loops: this file's and gemm_w4.h's) ----------
+// A tile publishes, per row, two 8-byte words: (mean, tag) and (M2, ~tag), each with one device-scope atomic
+// store.  Such stores go straight through the XCD-private L2 to memory and the device-scope loads of the
+// gather come straight from it, so the exchange needs no cache-wide write-back / invalidate (a
+// __threadfence() per workgroup costs tens of microseconds here).  `tag` is different for every launch: the
+// host hands every fused launch a fresh nonce, and a launch recorded in a graph, whose arguments repeat, is
+// preceded by a one-thread kernel that moves on a counter in the workspace header.  A word that does not carry
+// the launch's tag is "not published yet", whatever it holds: memory never used before, statistics of an
+// earlier launch or of another shape, or somebody else's data.  So a workspace needs no preparation, no
+// clearing between launches and no state on the host.  (A stray word passes for published with probability
+// 2^-32 per word, and both words of a row have to.)
+__device__ __forceinline__ unsigned ln_launch_tag(const GemmParams& p) {
+  unsigned x = p.ln_nonce + (unsigned)p.timeout_flag[kLnHdrReplay] * 0x9E3779B1u;  // uniform: nobody writes it during a launch
+  x ^= x >> 16;
+  x *= 0x7feb352du;
+  x ^= x >> 15;
+  x *= 0x846ca68bu;
+  x ^= x >> 16;
+  return x | 1u;  // never 0: a zeroed header then never reads as "timed out"
+}
+
+// Workgroup 0 records which launch the header speaks of.
+__device__ __forceinline__ void ln_sign_header(const GemmParams& p, unsigned tag) {
+  if (blockIdx.x == 0 && threadIdx.x == 0) {
+    p.timeout_flag[kLnHdrMagic] = kLnMagic;
+    p.timeout_flag[kLnHdrLaunchTag] = (int)tag;
+  }
+}
+
+__device__ __forceinline__ void ln_publish(const GemmParams& p, size_t slot, float mean, float m2, unsigned tag) {
+  const unsigned long long w0 = (unsigned long long)__float_as_uint(mean) | ((unsigned long long)tag << 32);
+  const unsigned long long w1 = (unsigned long long)__float_as_uint(m2) | ((unsigned long long)(~tag) << 32);
+  __hip_atomic_store((unsigned long long*)p.stats + slot, w0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __hip_atomic_store((unsigned long long*)p.next_stats + slot, w1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Gathers the (mean, M2) pairs of slots [first, first + n_slots) into `gathered` (LDS, 8 bytes per slot):
+// INFLIGHT slots per thread in flight before the first is examined, each polled (one bounded budget per thread)
+// until both its words carry the tag.  A thread that runs out of budget raises the header's flag and poisons
+// the pair, so that the rows concerned come out as NaN instead of as plausible numbers.
+template <int NT, int INFLIGHT = 8>
+__device__ __forceinline__ void ln_gather(const GemmParams& p, unsigned tag, size_t first, int n_slots, int tid,
+                                          unsigned long long* gathered) {
+  const unsigned long long* w0s = (const unsigned long long*)p.stats + first;
+  const unsigned long long* w1s = (const unsigned long long*)p.next_stats + first;
+  const unsigned not_tag = ~tag;
+  int polls = 0;
+  for (int q0 = tid; q0 < n_slots; q0 += INFLIGHT * NT) {
+    unsigned long long a[INFLIGHT], b[INFLIGHT];
+#pragma unroll
+    for (int u = 0; u < INFLIGHT; ++u) {
+      const int q = q0 + u * NT;
+      a[u] = __hip_atomic_load(w0s + (q < n_slots ? q : q0), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      b[u] = __hip_atomic_load(w1s + (q < n_slots ? q : q0), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+#pragma unroll
+    for (int u = 0; u < INFLIGHT; ++u) {
+      const int q = q0 + u * NT;
+      if (q >= n_slots) break;
+      // (a negative limit: treat everything as unpublished -- how the host forces this path in a test)
+      while ((unsigned)(a[u] >> 32) != tag || (unsigned)(b[u] >> 32) != not_tag || p.spin_limit < 0) {
+        if (++polls > p.spin_limit) {
+          p.timeout_flag[kLnHdrTimeout] = (int)tag;
+          a[u] = 0x7fc00000ull;
+          b[u] = 0x7fc00000ull;
+          break;
+        }
+        __builtin_amdgcn_s_sleep(4);
+        a[u] = __hip_atomic_load(w0s + q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        b[u] = __hip_atomic_load(w1s + q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+      gathered[q] = (a[u] & 0xffffffffull) | (b[u] << 32);
+    }
+  }
+}
 
 // Buffer descriptor word 3 for gfx9-family raw buffers: 32-bit data format, no swizzle.
 constexpr int kRsrcFlags = 0x00020000;
@@ -998,62 +1071,15 @@ struct GemmTile {
       float* red = (float*)smem;   // [BM][2] tile statistics, later (mean, rstd) of the whole row
       float* part = red + BM * 2;  // [BM][4*WAVES_N + 1][2], then reused as `gathered`
       tile_row_stats(part, red);
-      // 2. publish the tile's statistics: stats[band][tile_n][row] = (mean, M2) as one 8-byte
-      //    device-scope atomic store.  Such stores go straight through the XCD-private L2 to memory
-      //    and the device-scope loads below come straight from it, so the exchange needs no cache-wide
-      //    write-back / invalidate (a __threadfence() per workgroup costs tens of microseconds here).
-      //    A slot whose M2 is negative has not been published yet: M2 of real data is never negative.
+      // 2. publish the tile's statistics (ln_publish above: two tagged 8-byte words per row)
+      const unsigned tag = ln_launch_tag(p);
+      ln_sign_header(p, tag);
       const size_t my_slot = ((size_t)tc.tm * p.tiles_n + tc.tn) * BM;
-      const bool odd_epoch = (p.timeout_flag[kLnHdrEpoch] & 1) != 0;  // uniform; written before this launch began
-      float* const cur_set = odd_epoch ? p.next_stats : p.stats;
-      float* const other_set = odd_epoch ? p.stats : p.next_stats;
-      unsigned long long* my_stats = (unsigned long long*)cur_set + my_slot;
-      unsigned long long* my_next = (unsigned long long*)other_set + my_slot;
       // (tile_row_stats left row rl's pair with the thread that publishes it: same rl = tid stride)
-      for (int rl = tid; rl < BM; rl += NT) {
-        const float mean = red[rl * 2 + 0];
-        float m2 = red[rl * 2 + 1];
-        m2 = fmaxf(m2, 0.0f);  // rounding can leave -0.0 or a tiny negative: keep the "published" sign
-        const unsigned long long pair =
-            (unsigned long long)__float_as_uint(mean) | ((unsigned long long)__float_as_uint(m2) << 32);
-        __hip_atomic_store(my_stats + rl, pair, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        // the other set is the one the next launch on this workspace reads: mark it unpublished
-        const unsigned long long unpublished = (unsigned long long)__float_as_uint(-1.0f) << 32;
-        __hip_atomic_store(my_next + rl, unpublished, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      }
-      // 3. gather the band's statistics into LDS: one 8-byte device-scope load per (tile, row), all in
-      //    flight together, each repeated (bounded) until its tile has published
+      for (int rl = tid; rl < BM; rl += NT) ln_publish(p, my_slot + rl, red[rl * 2 + 0], red[rl * 2 + 1], tag);
+      // 3. gather the band's statistics into LDS
       float* gathered = part;  // [tiles_n][BM][2]; tiles_n <= 64 keeps it within the LDS the kernel owns
-      const unsigned long long* band_stats = (const unsigned long long*)cur_set + (size_t)tc.tm * p.tiles_n * BM;
-      const int n_slots = p.tiles_n * BM;
-      int polls = 0;  // one budget for all the slots of this thread: a thread that ran out of it polls no more
-      for (int q0 = tid; q0 < n_slots; q0 += 8 * NT) {
-        unsigned long long v[8];
-#pragma unroll
-        for (int u = 0; u < 8; ++u) {  // eight loads in flight per thread before the first is examined
-          const int q = q0 + u * NT;
-          v[u] = __hip_atomic_load(band_stats + (q < n_slots ? q : q0), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
-#pragma unroll
-        for (int u = 0; u < 8; ++u) {
-          const int q = q0 + u * NT;
-          if (q >= n_slots) break;
-          // sign bit of M2: not published yet (a negative limit: treat everything as unpublished -- how the
-          // host forces this path in a test)
-          while ((long long)v[u] < 0 || p.spin_limit < 0) {
-            if (++polls > p.spin_limit) {
-              // Give up: raise the flag and poison the row's statistics, so that the rows concerned come out
-              // as NaN instead of as plausible numbers.
-              p.timeout_flag[kLnHdrTimeout] = 1;
-              v[u] = 0x7fc000007fc00000ull;
-              break;
-            }
-            __builtin_amdgcn_s_sleep(4);
-            v[u] = __hip_atomic_load(band_stats + q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          }
-          ((unsigned long long*)gathered)[q] = v[u];
-        }
-      }
+      ln_gather<NT>(p, tag, (size_t)tc.tm * p.tiles_n * BM, p.tiles_n * BM, tid, (unsigned long long*)gathered);
       __syncthreads();
       // 4. merge in tile order -> (mean, rstd) per row
       const bool even_tiles = (N % BN) == 0;  // every column tile is full: equal weights
@@ -1101,9 +1127,6 @@ struct GemmTile {
                        v[e] = (T)((acc[i][j][e] - st.mean) * st.rstd * (float)gv[j][e] + (float)bv[j][e]);
                      return v;
                    });
-      // One more workgroup has published its statistics and marked its slots of the other set: the next
-      // launch's preparation trusts the workspace only if every workgroup of this one got here.
-      if (tid == 0) __hip_atomic_fetch_add(p.timeout_flag + kLnHdrDone, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     } else {
       if (EPI == kEpiLnStats) {
         // Per-row statistics over the columns this workgroup owns, from the fp32 accumulators.

@@ -529,46 +529,16 @@ struct GemmW4 {
         m2 += qw + delta * delta * (n_acc * nb / tot);
         n_acc = tot;
       }
-      // ... and publishes the tile's pair: one 8-byte device-scope atomic store; a slot whose M2 is negative
-      // has not been published (see gemm_kernel.h for why this needs no cache-wide fence)
-      const bool odd_epoch = (p.timeout_flag[kLnHdrEpoch] & 1) != 0;
-      float* const cur_set = odd_epoch ? p.next_stats : p.stats;
-      float* const other_set = odd_epoch ? p.stats : p.next_stats;
-      const size_t my_slot = ((size_t)tc.tm * p.tiles_n + tc.tn) * BM;
-      m2 = fmaxf(m2, 0.0f);
-      const unsigned long long pair = (unsigned long long)__float_as_uint(mean) | ((unsigned long long)__float_as_uint(m2) << 32);
-      __hip_atomic_store((unsigned long long*)cur_set + my_slot + rl, pair, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      const unsigned long long unpublished = (unsigned long long)__float_as_uint(-1.0f) << 32;
-      __hip_atomic_store((unsigned long long*)other_set + my_slot + rl, unpublished, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      // ... and publishes the tile's pair (gemm_kernel.h: ln_publish, two tagged 8-byte words per row)
+      const unsigned tag = ln_launch_tag(p);
+      ln_sign_header(p, tag);
+      ln_publish(p, ((size_t)tc.tm * p.tiles_n + tc.tn) * BM + rl, mean, m2, tag);
       __syncthreads();  // `part` is free again
       // 3. gather the band's pairs into LDS, polling (boundedly) what is not published yet
       float* gathered = part;
-      const unsigned long long* band_stats = (const unsigned long long*)cur_set + (size_t)tc.tm * p.tiles_n * BM;
-      const int n_slots = p.tiles_n * BM;
-      int polls = 0;
-      for (int q0 = tid; q0 < n_slots; q0 += 8 * NT) {
-        unsigned long long v[8];
-#pragma unroll
-        for (int u = 0; u < 8; ++u) {
-          const int q = q0 + u * NT;
-          v[u] = __hip_atomic_load(band_stats + (q < n_slots ? q : q0), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
-#pragma unroll
-        for (int u = 0; u < 8; ++u) {
-          const int q = q0 + u * NT;
-          if (q >= n_slots) break;
-          while ((long long)v[u] < 0 || p.spin_limit < 0) {
-            if (++polls > p.spin_limit) {
-              p.timeout_flag[kLnHdrTimeout] = 1;
-              v[u] = 0x7fc000007fc00000ull;
-              break;
-            }
-            __builtin_amdgcn_s_sleep(4);
-            v[u] = __hip_atomic_load(band_stats + q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          }
-          ((unsigned long long*)gathered)[q] = v[u];
-        }
-      }
+      // (four slots in flight, not eight: this kernel has all its ordinary registers in use here, and a compiler
+      // short of them parks values in accumulation registers, i.e. in the accumulators)
+      ln_gather<NT, 4>(p, tag, (size_t)tc.tm * p.tiles_n * BM, p.tiles_n * BM, tid, (unsigned long long*)gathered);
       __syncthreads();
       // 4. merge in tile order -> (mean, rstd) of the whole row
       mean = 0.0f;
@@ -617,8 +587,6 @@ struct GemmW4 {
         __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(i32x4, v), rsrc, (int)out.voff[q], 0, 0);
       });
     });
-    // One more workgroup has published its statistics and marked its slots of the other set.
-    if (tid == 0) __hip_atomic_fetch_add(p.timeout_flag + kLnHdrDone, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
 };
 

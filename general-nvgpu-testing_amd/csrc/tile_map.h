@@ -49,14 +49,16 @@ BEAM_HD int kmajor_lds_offset(int k, int n, int block_n) {
   return k * block_n * 2 + ((((n >> 3) ^ kmajor_swizzle(k, block_n))) << 4) + ((n & 7) << 1);
 }
 
-// Words of the fused GEMM+LayerNorm workspace header (256 bytes in front of the two statistics sets).
-constexpr int kLnHdrTimeout = 0;   // 1: a workgroup gave up waiting for a band's statistics
-constexpr int kLnHdrMagic = 1;     // kLnMagic once the workspace has been prepared
-constexpr int kLnHdrGeometry = 2;  // two words: (tiles_m, tiles_n, block_m) the sets are laid out for
-constexpr int kLnHdrEpoch = 4;     // launches so far; its parity selects the statistics set
-constexpr int kLnHdrDone = 5;      // workgroups of the latest launch that have finished
-constexpr int kLnHdrExpected = 6;  // ... out of this many
-constexpr int kLnMagic = 0x4c4e3032;
+// Words of the fused GEMM+LayerNorm workspace header (256 bytes in front of the two arrays of statistics
+// words).  Nothing in it has to be initialised: every fused launch carries a tag that no earlier launch had,
+// a statistics word counts as published only if it carries that tag, and the header words say which launch
+// wrote them.
+constexpr int kLnHdrTimeout = 0;    // tag of a launch in which a workgroup gave up waiting for a band's statistics
+constexpr int kLnHdrMagic = 1;      // kLnMagic once a fused launch has run on this workspace
+constexpr int kLnHdrLaunchTag = 2;  // tag of the latest launch
+constexpr int kLnHdrReplay = 3;     // counter that a one-thread kernel moves on in front of a captured launch, whose
+                                    // kernel arguments repeat from replay to replay; part of the tag
+constexpr int kLnMagic = 0x4c4e3033;
 
 struct TileCoord {
   int tm;  // tile index along M

@@ -153,20 +153,18 @@ size_t beam_gemmrc_ln_workspace_bytes_ex(int M, int N, const beam_tile_cfg* cfg,
 int beam_gemmrc_ln_ex(const void* A, const void* B, const void* gamma, const void* beta, float eps,
                       void* Y, int M, int N, int K, int dtype, const beam_tile_cfg* cfg, int mode,
                       void* ws, size_t ws_bytes, void* stream);
-/* The fused path keeps state in its workspace between launches (each launch prepares the statistics
- * slots of the next one), described by a 256-byte header in the workspace itself: magic word,
- * geometry, launch count and how many workgroups of the latest launch finished.  A small kernel in
- * front of every fused launch checks the header on the device and re-initialises the workspace if
- * anything is off, so a fresh buffer, a buffer the allocator hands out again, a different problem
- * shape or an interrupted launch need nothing from the caller; the library keeps no host-side record
- * of workspaces.  What the check cannot see is a foreign write into the statistics that leaves the
- * header intact: after such a write call this (it clears the header, synchronously).  Launches
- * sharing one workspace must be ordered on one stream. */
+/* The fused path's workspace needs no preparation and carries no state from call to call: every
+ * fused launch has a tag that no earlier launch had, and a statistics word counts only if it carries
+ * that tag (a stray word passes with probability 2^-32, and both words of a row have to).  So a fresh
+ * buffer, one the allocator hands out again, one used for another shape or written over by somebody
+ * else all work as they are, and the library keeps no host-side record of workspaces.  Launches that
+ * share one workspace must be ordered on one stream.  This call only zeroes the 256-byte header
+ * (synchronously), which forgets a recorded time-out; nothing requires it. */
 int beam_gemmrc_ln_workspace_reset(const void* ws);
 /* Waits for `stream`, then *timed_out = 1 if the latest fused call on this workspace gave up
  * waiting for a band: the rows concerned are then NaN in Y.  Only possible if the device could not
  * hold a whole band of workgroups at once, e.g. because another process occupied most of it.  The
- * flag is cleared at the start of every fused call. */
+ * record names the launch it is about, so every fused call starts with a clean slate. */
 int beam_gemmrc_ln_timed_out(const void* ws, void* stream, int* timed_out);
 /* Bound of that wait: polls of statistics slots per thread (roughly a microsecond each; default
  * 4 Mi).  0 makes every thread that finds a slot unpublished give up at once; -1 makes every wait give
@@ -262,7 +260,7 @@ int beam_event_destroy(void* event);
  * has no counterpart (it launches on the legacy default stream, cuda/cute_kernels/cute_gemm_128x128.cu:
  * 203).  Rules: call every operator once eagerly before capturing it (the first launch of a kernel
  * configures its LDS size); BEAM_LN_AUTO takes the two-pass path under capture (BEAM_LN_FUSED is honoured:
- * the workspace's epoch moves on inside the captured launches); K = 0 clears C with a kernel, not a
+ * a one-thread kernel recorded in front of it makes every replay's tag new); K = 0 clears C with a kernel, not a
  * memset node.  Streams are created at the default priority. */
 int beam_stream_create(void** stream);
 int beam_stream_destroy(void* stream);

@@ -85,6 +85,18 @@ def test_graph_replay_matches_eager(gpu, beamc):
             timed_out = ctypes.c_int(1)
             chk(L.beam_gemmrc_ln_timed_out(ws_lnf.ptr, stream, ctypes.byref(timed_out)))
             assert timed_out.value == 0
+            # a second replay right behind the first, on new data: what the first replay left in the workspaces
+            # (the fused LayerNorm's statistics among it) must not pass for the second one's
+            upload()
+            poison()
+            chk(L.beam_graph_launch(graph, stream))
+            chk(L.beam_sync(stream))
+            got = snapshot()
+            poison()
+            sequence(None)
+            want = snapshot()
+            for k in want:
+                assert (got[k] == want[k]).all(), f"replay {replay}, second in a row: {k} differs from the eager result"
     finally:
         chk(L.beam_graph_destroy(graph))
         chk(L.beam_stream_destroy(stream))

@@ -165,9 +165,10 @@ def _ln_ex(beamc, da, db, dg, dbt, y, M, N, K, dtype, ws, mode):
 
 
 def test_ln_fused_workspace_describes_itself(gpu, beamc, oracle):
-    """The fused kernel's workspace carries its own state: a buffer freed and handed out again, overwritten
-    with bytes that read as published statistics (0x3f...: sign bit clear), or used for another shape before,
-    needs no reset call -- the launch notices on the device and starts over."""
+    """The fused kernel's workspace needs no preparation and no reset: statistics words count only if they carry
+    the tag of the launch that reads them.  A fresh buffer, one freed and handed out again, one overwritten
+    with bytes that look like plausible statistics (0x3f...), one that holds the statistics of the previous
+    launch on other data of the same shape, one used for another shape in between: all give the oracle's result."""
     M, N, K = 768, 2048, 256
     a, b, g_, bt = make_ln_inputs(beamc, M, N, K, F16, 31)
     ref = oracle.gemmrc_ln(a, b, g_, bt, 1e-5, F16)
@@ -191,6 +192,19 @@ def test_ln_fused_workspace_describes_itself(gpu, beamc, oracle):
     ws.fill_bytes(0x3F)
     launch_and_check(ws, "re-allocated workspace full of 0x3f")
     launch_and_check(ws, "launch after that")
+    # the same shape with other data: what the previous launch published must not pass for this launch's
+    a3, b3, g3, bt3 = make_ln_inputs(beamc, M, N, K, F16, 33)
+    ref3 = oracle.gemmrc_ln(a3, b3, g3, bt3, 1e-5, F16)
+    da3, db3 = beamc.DeviceArray.from_numpy(a3), beamc.DeviceArray.from_numpy(b3)
+    dg3, dbt3 = beamc.DeviceArray.from_numpy(g3), beamc.DeviceArray.from_numpy(bt3)
+    for rep in range(3):
+        y.fill_bytes(0xEE)
+        _ln_ex(beamc, da3, db3, dg3, dbt3, y, M, N, K, F16, ws, beamc.LN_FUSED)
+        beamc.sync()
+        check_ln(oracle, y.to_numpy(), ref3, F16, f"other data, same shape, same workspace ({rep})")
+        launch_and_check(ws, f"and the first data again ({rep})")
+    for x in (da3, db3, dg3, dbt3):
+        x.free()
     # another shape on the same buffer in between (same bytes needed or fewer), then the first one again
     M2, N2 = 512, 1024
     a2, b2, g2, bt2 = make_ln_inputs(beamc, M2, N2, K, F16, 32)
