@@ -80,6 +80,8 @@ def _load() -> ctypes.CDLL:
     L.beam_splitk_workspace_bytes.restype = sz
     L.beam_gemmrc_splitk.argtypes = [vp, vp, vp, i, i, i, i, cfgp, i, vp, sz, vp]
     L.beam_splitk_effective.argtypes = [i, i, i, cfgp, i]
+    L.beam_set_splitk_two_launches.argtypes = [i]
+    L.beam_gemmrc_splitk_timed_out.argtypes = [vp, i, i, i, vp, ctypes.POINTER(i)]
     L.beam_splitk_noalloc_max_bytes.argtypes = []
     L.beam_splitk_noalloc_max_bytes.restype = sz
     L.beam_gemmrc_splitk_noalloc.argtypes = [vp, vp, vp, i, i, i, i, cfgp, i, vp]
@@ -339,7 +341,7 @@ def gemmrc_spec(a, b, c, shape_threadblock=(128, 128), shape_warp=(64, 64), pipe
     _check(lib.beam_gemmrc(pa, pb, pc, M, N, K, d, ctypes.byref(cfg), st))
 
 
-def _splitk(a, b, c, cfgp, split_k_slices: int) -> None:
+def _splitk(a, b, c, cfgp, split_k_slices: int, check: bool = False) -> None:
     pa, pb, pc, M, N, K, d, st = _problem(a, b, c)
     s = lib.beam_splitk_effective(M, N, K, cfgp, split_k_slices)
     if s < 0:
@@ -348,20 +350,32 @@ def _splitk(a, b, c, cfgp, split_k_slices: int) -> None:
     ws = _get_workspace(need) if need else None
     _check(lib.beam_gemmrc_splitk(pa, pb, pc, M, N, K, d, cfgp, split_k_slices,
                                   ws.ptr if ws else None, ws.nbytes if ws else 0, st))
+    if check and ws is not None:
+        flag = ctypes.c_int(0)
+        _check(lib.beam_gemmrc_splitk_timed_out(ws.ptr, M, N, s, st, ctypes.byref(flag)))
+        if flag.value:
+            raise BeamError(4, "split-K: a reducing workgroup gave up waiting for the slices of its tile; "
+                               "the outputs concerned are NaN")
 
 
-def gemmrc_splitk(a, b, c, split_k_slices: int = 0) -> None:
+def set_splitk_two_launches(on: bool) -> None:
+    """True: split-K always runs as partial kernel + reduce kernel; False (default): one launch where it applies."""
+    _check(lib.beam_set_splitk_two_launches(1 if on else 0))
+
+
+def gemmrc_splitk(a, b, c, split_k_slices: int = 0, check: bool = False) -> None:
     """Split-K with the library's default tile for the problem; split_k_slices <= 0: the library
     picks the slice count as well (one full round of workgroups)
-    (reference: cutlass_gemmrc_splitk, python/beam/_C/beam_C.pyi:18)."""
-    _splitk(a, b, c, None, split_k_slices)
+    (reference: cutlass_gemmrc_splitk, python/beam/_C/beam_C.pyi:18).  check=True waits for the
+    result and raises if the one-launch form's bounded wait ran out."""
+    _splitk(a, b, c, None, split_k_slices, check)
 
 
 def gemmrc_splitk_spec(a, b, c, shape_threadblock=(128, 128), shape_warp=(64, 64), split_k_slices: int = 0,
-                       pipeline: int = 0, group_m: int = 0) -> None:
+                       pipeline: int = 0, group_m: int = 0, check: bool = False) -> None:
     """Split-K with explicit tiles (reference: cutlass_gemmrc_splitk_spec, beam_C.pyi:20)."""
     cfg = _cfg_from_shapes(shape_threadblock, shape_warp, pipeline, group_m)
-    _splitk(a, b, c, ctypes.byref(cfg), split_k_slices)
+    _splitk(a, b, c, ctypes.byref(cfg), split_k_slices, check)
 
 
 LN_AUTO, LN_TWOPASS, LN_FUSED = 0, 1, 2

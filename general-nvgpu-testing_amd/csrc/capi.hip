@@ -65,7 +65,8 @@ std::atomic<unsigned> g_ln_nonce{(unsigned)std::chrono::steady_clock::now().time
 // code is loaded on a GPU until the process ends, so the entry point never allocates.  In host code the
 // array's name is only a handle for hipGetSymbolAddress; what kernels and copies get is the per-device
 // address looked up below (every GPU has its own copy at its own address).
-constexpr size_t kScratchBytes = (size_t)16 << 20;
+constexpr size_t kScratchPartialBytes = (size_t)16 << 20;                      // the partial sums a call may need
+constexpr size_t kScratchBytes = kScratchPartialBytes + ((size_t)256 << 10);  // ... + synchronisation words of the one-launch form
 constexpr int kMaxDevices = 64;
 void* g_scratch_ptr[kMaxDevices] = {};
 std::mutex g_scratch_mu;
@@ -576,9 +577,25 @@ int beam_custom_gemmrc_256x128(const void* A, const void* B, void* C, int M, int
   return custom_fixed(256, 128, 64, 64, A, B, C, M, N, K, stream);
 }
 
+// Workspace of a split-K call: fp32 partial sums [split_k][M][N], then (256-byte aligned) the synchronisation
+// words of the one-launch form.  A workspace that only holds the partial sums still works: two launches.
+static size_t splitk_partial_bytes(int M, int N, int split_k) {
+  return (size_t)split_k * (size_t)M * (size_t)N * sizeof(float);
+}
 size_t beam_splitk_workspace_bytes(int M, int N, int split_k) {
   if (M <= 0 || N <= 0 || split_k <= 0) return 0;
-  return (size_t)split_k * (size_t)M * (size_t)N * sizeof(float);
+  return align_up(splitk_partial_bytes(M, N, split_k), 256) + (size_t)sk_sync_bytes(M, N, split_k);
+}
+
+// 0: one launch where it applies, 1: always the partial kernel followed by the reduce kernel
+static std::atomic<int> g_splitk_two_launches{[] {
+  const char* e = getenv("BEAM_SPLITK_TWO_LAUNCHES");
+  return e && *e && *e != '0' ? 1 : 0;
+}()};
+
+int beam_set_splitk_two_launches(int on) {
+  g_splitk_two_launches.store(on != 0);
+  return BEAM_OK;
 }
 
 static int effective_split(int M, int N, int K, const beam_tile_cfg& c, int split_k) {
@@ -656,7 +673,7 @@ int beam_gemmrc_splitk(const void* A, const void* B, void* C, int M, int N, int 
     BEAM_HIP(ks->launch[dtype][kEpiStore][c.pipeline](p, dim3((unsigned)(p.tiles_m * p.tiles_n), 1, 1), st));
     return BEAM_OK;
   }
-  const size_t need = beam_splitk_workspace_bytes(M, N, s);
+  const size_t need = splitk_partial_bytes(M, N, s);
   if (!ws || ws_bytes < need)
     return fail(BEAM_ERR_WORKSPACE, "split-K with %d slices needs %zu bytes of workspace, got %zu", s, need, ws_bytes);
   if ((uintptr_t)ws & 15) return fail(BEAM_ERR_UNSUPPORTED, "workspace must be 16-byte aligned");
@@ -664,12 +681,42 @@ int beam_gemmrc_splitk(const void* A, const void* B, void* C, int M, int N, int 
   p.ws = (float*)ws;
   p.k_slice = split_k_len(K, s);
   p.splits = s;
+  // One launch: the reducing workgroups ride behind the multiplying ones in the same grid.  Needs a tile the
+  // form is built for, 16-byte rows of partial sums, at most one flag per lane, a slice that fits one buffer
+  // descriptor, and room for the synchronisation words behind the partial sums.
+  const GemmLauncher one_launch = ks->launch_partial_fused[dtype][c.pipeline];
+  const size_t sync_at = align_up(need, 256);
+  if (one_launch && !g_splitk_two_launches.load(std::memory_order_relaxed) && N % 4 == 0 && s <= 64 &&
+      (size_t)M * N <= ((size_t)1 << 28) && ws_bytes >= sync_at + (size_t)sk_sync_bytes(M, N, s)) {
+    p.C = C;
+    p.sk_sync = (int*)((char*)ws + sync_at);
+    p.ln_nonce = g_ln_nonce.fetch_add(1, std::memory_order_relaxed) + 1;
+    p.spin_limit = g_ln_spin_limit.load();
+    const int tiles = p.tiles_m * p.tiles_n;
+    // parts of 4 outputs per thread, smaller ones while the reducing workgroups are fewer than the CUs
+    const int cus = g_dev.cus > 0 ? g_dev.cus : 256;
+    p.sk_out = 4;
+    while (p.sk_out > 1 && tiles * sk_parts_per_tile(c.block_m, c.block_n, ks->threads, p.sk_out) < cus) p.sk_out /= 2;
+    const int parts = sk_parts_per_tile(c.block_m, c.block_n, ks->threads, p.sk_out);
+    BEAM_HIP(one_launch(p, dim3((unsigned)(tiles * s + tiles * parts), 1, 1), st));
+    return BEAM_OK;
+  }
   BEAM_HIP(ks->launch[dtype][kEpiPartial][c.pipeline](p, dim3((unsigned)(p.tiles_m * p.tiles_n * s), 1, 1), st));
   BEAM_HIP(launch_splitk_reduce((const float*)ws, C, (size_t)M * N, s, dtype, st));
   return BEAM_OK;
 }
 
-size_t beam_splitk_noalloc_max_bytes(void) { return kScratchBytes; }
+int beam_gemmrc_splitk_timed_out(const void* ws, int M, int N, int split_k_effective, void* stream, int* timed_out) {
+  if (!ws || !timed_out || M <= 0 || N <= 0 || split_k_effective < 1) return fail(BEAM_ERR_INVALID, "bad argument");
+  BEAM_HIP(hipStreamSynchronize((hipStream_t)stream));
+  int hdr[4] = {0, 0, 0, 0};
+  const size_t sync_at = align_up(splitk_partial_bytes(M, N, split_k_effective), 256);
+  BEAM_HIP(hipMemcpy(hdr, (const char*)ws + sync_at, sizeof hdr, hipMemcpyDeviceToHost));
+  *timed_out = hdr[kSkMagic] == kSkMagicValue && hdr[kSkLaunchTag] != 0 && hdr[kSkTimeout] == hdr[kSkLaunchTag];
+  return BEAM_OK;
+}
+
+size_t beam_splitk_noalloc_max_bytes(void) { return kScratchPartialBytes; }
 
 int beam_gemmrc_splitk_noalloc(const void* A, const void* B, void* C, int M, int N, int K, int dtype,
                                const beam_tile_cfg* cfg, int split_k, void* stream) {
@@ -678,11 +725,11 @@ int beam_gemmrc_splitk_noalloc(const void* A, const void* B, void* C, int M, int
   if (M > 0 && N > 0 && K > 0) {
     const int s = beam_splitk_effective(M, N, K, cfg, split_k);
     if (s < 0) return BEAM_ERR_UNSUPPORTED;  // the message is already set
-    const size_t need = s > 1 ? beam_splitk_workspace_bytes(M, N, s) : 0;
-    if (need > kScratchBytes)
+    const size_t need = s > 1 ? splitk_partial_bytes(M, N, s) : 0;
+    if (need > kScratchPartialBytes)
       return fail(BEAM_ERR_WORKSPACE, "split-K of %d x %d in %d slices needs %zu bytes; the built-in workspace of the "
                   "no-allocation entry point holds %zu (use beam_gemmrc_splitk with a workspace of your own)", M, N, s, need,
-                  kScratchBytes);
+                  kScratchPartialBytes);
   }
   void* ws = nullptr;
   if ((rc = scratch_on_current_device(&ws))) return rc;

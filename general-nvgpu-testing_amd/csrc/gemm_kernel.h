@@ -91,6 +91,10 @@ enum Epilogue : int {
   // kEpiPartial with its global->LDS loads and fragment reads but without MFMAs, and nothing stored.
   // What such a launch costs is the floor that the loads of a split-K launch shape set by themselves.
   kEpiProbeLoads = 6,
+  // Split-K in one launch (own launch table, small tiles only): kEpiPartial with its partial sums written
+  // through to memory, followed in the same grid by reducing workgroups that add the slices of a tile in
+  // slice order as soon as all of them have signalled (splitk_reduce_part_of below).
+  kEpiPartialFused = 7,
 };
 constexpr int kNumEpilogues = 6;  // epilogues of the launch tables
 
@@ -126,6 +130,10 @@ struct GemmParams {
   int side_iters;        // K tiles' worth of units per workgroup
   int side_width;        // bytes per unit
   int c_streaming;       // kEpiStoreLoop: store C non-temporal
+  // kEpiPartialFused: word kSkTimeout, then from word kSkFlags on one flag per (tile, part of the tile, slice);
+  // behind the partial sums in the caller's workspace.  Never has to be initialised (see sk_launch_tag).
+  int* sk_sync;
+  int sk_out;  // kEpiPartialFused: outputs per thread of a reducing workgroup (4, 2 or 1)
 };
 
 // ---- statistics exchange of the fused GEMM+LayerNorm (both K loops: this file's and gemm_w4.h's) ----------
@@ -203,6 +211,27 @@ __device__ __forceinline__ void ln_gather(const GemmParams& p, unsigned tag, siz
     }
   }
 }
+
+// ---- split-K in one launch (kEpiPartialFused) -----------------------------------------------------------
+// The grid holds the tiles x slices workgroups of kEpiPartial and, behind them, one reducing workgroup per
+// (tile, part).  Workgroups are placed in id order, so a reducing workgroup starts only once every multiplying
+// workgroup has been placed (on its own XCD; the other XCDs place theirs whatever a waiting workgroup here does):
+// what it waits for always arrives, with any number of rounds and on a device shared with other work.  The
+// partial sums leave with device-scope (write-through) stores, and the flag that announces them is stored after
+// those have been acknowledged; the reducing workgroup reads flags and sums with device-scope loads, which come
+// from memory, not from an XCD-private L2.  A flag counts only if it equals the launch's tag (a hash of a nonce
+// that no earlier launch of the process had), so the workspace needs no clearing; the reducer clears the flags it
+// has consumed, so a graph replay, whose arguments and therefore tag repeat, starts clean as well.
+__device__ __forceinline__ unsigned sk_launch_tag(unsigned nonce) {
+  unsigned x = nonce;
+  x ^= x >> 16;
+  x *= 0x7feb352du;
+  x ^= x >> 15;
+  x *= 0x846ca68bu;
+  x ^= x >> 16;
+  return x | 1u;  // never 0: a cleared flag is never "set"
+}
+constexpr int kAuxDeviceScope = 16;  // sc1: the access is performed at device scope (through the L2, to memory)
 
 // Buffer descriptor word 3 for gfx9-family raw buffers: 32-bit data format, no swizzle.
 constexpr int kRsrcFlags = 0x00020000;
@@ -303,12 +332,102 @@ struct GemmTile {
     return (unsigned)row * (unsigned)K * 2u + (unsigned)chunk * 16u;
   }
 
+  // kEpiPartialFused: reducing workgroup r = (tile, part).  Waits until the tile's slices have all signalled,
+  // adds their partial sums in slice order 0, 1, 2, ... (the order of splitk_reduce_kernel: same bits) and
+  // rounds once.  A thread owns OUT = p.sk_out (4, 2 or 1) consecutive columns of one row of the part: the host
+  // makes the parts small when there are few tiles, so that the reads spread over many CUs (a CU takes in its
+  // share of the partial sums at well under 100 GB/s; 64 workgroups reading 128 KiB each took 2 us).
+  template <int OUT>
+  static __device__ __forceinline__ void splitk_reduce_part_of(const GemmParams& p, int r) {
+    constexpr int P = sk_parts_per_tile(BM, BN, NT, OUT);
+    constexpr int PART_ROWS = NT * OUT / BN;
+    static_assert(P >= 1 && P <= NT && P * NT * OUT == BM * BN && PART_ROWS * BN == NT * OUT, "parts tile the tile");
+    typedef float acc_t __attribute__((ext_vector_type(OUT)));
+    typedef T out_t __attribute__((ext_vector_type(OUT)));
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int t = r / P, q = r - t * P;
+    const int tm = t / p.tiles_n, tn = t - tm * p.tiles_n;
+    const int M = p.M, N = p.N, S = p.splits;
+    const int tag = (int)sk_launch_tag(p.ln_nonce);
+    int* flags = p.sk_sync + kSkFlags + (size_t)r * S;
+    if (r == 0 && tid == 0) {  // which launch the header speaks of
+      p.sk_sync[kSkMagic] = kSkMagicValue;
+      p.sk_sync[kSkLaunchTag] = tag;
+    }
+    // every wavefront polls for itself (S <= 64: one flag per lane); one bounded budget
+    bool arrived = false;
+    for (int polls = 0; polls <= p.spin_limit; ++polls) {
+      const int v = lane < S ? __hip_atomic_load(flags + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : tag;
+      if (__all(v == tag)) {
+        arrived = true;
+        break;
+      }
+      __builtin_amdgcn_s_sleep(1);
+    }
+    const int m = tm * BM + q * PART_ROWS + tid / (BN / OUT);
+    const int n = tn * BN + (tid % (BN / OUT)) * OUT;
+    const bool valid = m < M && n < N;  // N is a multiple of 4: a thread's columns exist together
+    const unsigned off = valid ? ((unsigned)m * (unsigned)N + (unsigned)n) * 4u : kOobOffset;
+    const unsigned slice_bytes = (unsigned)M * (unsigned)N * 4u;
+    auto load = [&](int z) __attribute__((always_inline)) -> acc_t {
+      const __amdgpu_buffer_rsrc_t rs = make_rsrc(p.ws + (size_t)z * M * N, slice_bytes);
+      if constexpr (OUT == 4) return __builtin_bit_cast(acc_t, __builtin_amdgcn_raw_buffer_load_b128(rs, (int)off, 0, kAuxDeviceScope));
+      else if constexpr (OUT == 2) return __builtin_bit_cast(acc_t, __builtin_amdgcn_raw_buffer_load_b64(rs, (int)off, 0, kAuxDeviceScope));
+      else return __builtin_bit_cast(acc_t, __builtin_amdgcn_raw_buffer_load_b32(rs, (int)off, 0, kAuxDeviceScope));
+    };
+    acc_t s = 0.0f;
+    int z = 0;
+    // batches of 16, 8, 4, 2, 1 slices: the loads of a batch in flight before the first add
+    auto batch = [&](auto n_tag) __attribute__((always_inline)) {
+      constexpr int NB = decltype(n_tag)::value;
+      while (z + NB <= S) {
+        acc_t v[NB];
+#pragma unroll
+        for (int u = 0; u < NB; ++u) v[u] = load(z + u);
+        if (z == 0) s = v[0];
+        else s += v[0];
+#pragma unroll
+        for (int u = 1; u < NB; ++u) s += v[u];
+        z += NB;
+      }
+    };
+    if constexpr (OUT < 4) batch(std::integral_constant<int, 32>{});
+    batch(std::integral_constant<int, 16>{});
+    batch(std::integral_constant<int, 8>{});
+    batch(std::integral_constant<int, 4>{});
+    batch(std::integral_constant<int, 2>{});
+    batch(std::integral_constant<int, 1>{});
+    __syncthreads();  // every wavefront has seen the flags: they can go
+    if (tid < S) __hip_atomic_store(flags + tid, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (!arrived) {  // never on a working device; visible in the data and in the workspace if it happens
+      if (tid == 0) p.sk_sync[kSkTimeout] = tag;
+      s = __builtin_nanf("");
+    }
+    if (valid) {
+      out_t o;
+#pragma unroll
+      for (int e = 0; e < OUT; ++e) o[e] = (T)s[e];
+      *(out_t*)((T*)p.C + (size_t)m * N + n) = o;
+    }
+  }
+
   static __device__ __forceinline__ void run(const GemmParams& p, char* smem) {
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave % WAVES_M;
     const int wn = wave / WAVES_M;
+
+    if constexpr (EPI == kEpiPartialFused) {
+      const int multiplying = p.tiles_m * p.tiles_n * p.splits;
+      if ((int)blockIdx.x >= multiplying) {  // (uniform)
+        const int r = (int)blockIdx.x - multiplying;
+        if (p.sk_out == 4) splitk_reduce_part_of<4>(p, r);
+        else if (p.sk_out == 2) splitk_reduce_part_of<2>(p, r);
+        else splitk_reduce_part_of<1>(p, r);
+        return;
+      }
+    }
 
     // Fused LayerNorm uses the band-block order, which keeps the workgroups that must exchange
     // statistics resident together; its grid is padded and the surplus workgroups leave here.
@@ -1143,6 +1262,29 @@ struct GemmTile {
         }
       }
       if constexpr (EPI == kEpiProbeLoads) return;
+      if constexpr (EPI == kEpiPartialFused) {
+        // The slice's partial sums, written through to memory (N is a multiple of 4 and M * N * 4 fits a
+        // descriptor: the host sees to it), then the flags of the tile's parts.
+        const __amdgpu_buffer_rsrc_t rsrc_w = make_rsrc(p.ws + (size_t)slice * M * N, (unsigned)M * (unsigned)N * 4u);
+#pragma unroll
+        for (int i = 0; i < FM; ++i) {
+          const int m = m_base + i * 16;
+#pragma unroll
+          for (int j = 0; j < FN; ++j) {
+            const int n = n_base + j * 16;
+            const unsigned off = (m < M && n < N) ? ((unsigned)m * (unsigned)N + (unsigned)n) * 4u : kOobOffset;
+            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(i32x4, acc[i][j]), rsrc_w, (int)off, 0, kAuxDeviceScope);
+          }
+        }
+        __builtin_amdgcn_s_waitcnt(0);  // this wavefront's stores have been acknowledged by memory ...
+        __syncthreads();                // ... and so have everyone's
+        const int P = sk_parts_per_tile(BM, BN, NT, p.sk_out);
+        if (tid < P) {
+          const size_t f = ((size_t)(tc.tm * p.tiles_n + tc.tn) * P + tid) * p.splits + slice;
+          __hip_atomic_store(p.sk_sync + kSkFlags + f, (int)sk_launch_tag(p.ln_nonce), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        return;
+      }
       // fp32 tile: split-K partial sums of this slice, or X for the normalisation pass.
       float* W = p.ws + (EPI == kEpiPartial ? (size_t)slice * M * N : (size_t)0);
 #pragma unroll

@@ -21,6 +21,9 @@ struct KernelSet {
   GemmLauncher launch[2][kNumEpilogues][3];
   // B stored [K][N] instead of [N][K], kEpiStore only: [dtype][pipeline 0 or 1]
   GemmLauncher launch_kmajor[2][2];
+  // Split-K in one launch (kEpiPartialFused), tiles up to 128 x 128 only (what split-K problems run on):
+  // [dtype][pipeline]; nullptr otherwise.
+  GemmLauncher launch_partial_fused[2][3];
 };
 
 template <typename T, int BM, int BN, int WVM, int WVN, int EPI, int AST, int BST, bool B_KMAJOR = false>
@@ -46,6 +49,12 @@ GemmLauncher loop_launcher() {
     return launch_gemm<T, BM, BN, WVM, WVN, kEpiStoreLoop, 3, 2>;
   else
     return nullptr;
+}
+
+template <typename T, int BM, int BN, int WVM, int WVN, int AST, int BST>
+GemmLauncher partial_fused_launcher() {
+  if constexpr (BM * BN <= 128 * 128) return launch_gemm<T, BM, BN, WVM, WVN, kEpiPartialFused, AST, BST>;
+  else return nullptr;
 }
 
 template <int BM, int BN, int TM, int TN>
@@ -81,7 +90,10 @@ KernelSet make_kernel_set() {
   k.launch_kmajor[D][1] = launch_gemm<T, BM, BN, WVM, WVN, kEpiStore, 2, 2, true>; \
   k.launch[D][kEpiStoreLoop][0] = loop_launcher<T, BM, BN, WVM, WVN>();              \
   k.launch[D][kEpiStoreLoop][1] = nullptr;                                            \
-  k.launch[D][kEpiStoreLoop][2] = nullptr;
+  k.launch[D][kEpiStoreLoop][2] = nullptr;                                            \
+  k.launch_partial_fused[D][0] = partial_fused_launcher<T, BM, BN, WVM, WVN, 3, 2>();  \
+  k.launch_partial_fused[D][1] = partial_fused_launcher<T, BM, BN, WVM, WVN, 2, 2>();  \
+  k.launch_partial_fused[D][2] = partial_fused_launcher<T, BM, BN, WVM, WVN, DA, DA - 1>();
   BEAM_FILL(0, _Float16)
   BEAM_FILL(1, __bf16)
 #undef BEAM_FILL

@@ -60,6 +60,27 @@ constexpr int kLnHdrReplay = 3;     // counter that a one-thread kernel moves on
                                     // kernel arguments repeat from replay to replay; part of the tag
 constexpr int kLnMagic = 0x4c4e3033;
 
+// Split-K in one launch: the synchronisation words behind the partial sums in the workspace.  The first words
+// say which launch ran last and whether one of its reducing workgroups gave up waiting (never initialised: the
+// words name the launch they speak of); from word kSkFlags on there is one
+// flag per (tile, part, slice): the workgroup of (tile, slice) sets the flags of all the tile's parts to the
+// launch's tag once its partial sums are in memory, the workgroup that reduces (tile, part) waits for its
+// `splits` flags and clears them again.  A part is what one reducing workgroup adds up: 4, 2 or 1 outputs per
+// thread (the fewer the tiles, the smaller the parts, so that many CUs share the reading).
+constexpr int kSkTimeout = 0;    // tag of a launch in which a reducing workgroup gave up waiting
+constexpr int kSkMagic = 1;      // kSkMagicValue once a one-launch split-K has run on this workspace
+constexpr int kSkLaunchTag = 2;  // tag of the latest launch
+constexpr int kSkMagicValue = 0x534b3031;
+constexpr int kSkFlags = 64;
+__host__ __device__ constexpr int sk_parts_per_tile(int block_m, int block_n, int threads, int out) {
+  return block_m * block_n / (threads * out);
+}
+// Bytes of synchronisation words that are enough for any tile of the library (every tile is at least 64 x 64
+// and every part at least 256 outputs): ceil(M/64) * ceil(N/64) * 16 parts * splits flags.
+__host__ __device__ constexpr unsigned long long sk_sync_bytes(int M, int N, int splits) {
+  return 4ull * (kSkFlags + (unsigned long long)((M + 63) / 64) * ((N + 63) / 64) * 16ull * (unsigned long long)splits);
+}
+
 struct TileCoord {
   int tm;  // tile index along M
   int tn;  // tile index along N

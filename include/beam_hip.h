@@ -90,19 +90,34 @@ int beam_custom_gemmrc_256x128(const void* A, const void* B, void* C, int M, int
  * beam_gemmrc_splitk with split_k <= 0 uses floor(CUs / tiles) instead (at most 64, at least
  * 4 K tiles of 64 per slice; 1 when the tiles already fill half the CUs). */
 int beam_slice_heuristic(int tiles, int compute_units);
-/* Bytes of fp32 workspace for `split_k` partial results (replaces the hidden grow-only
- * buffer get_the_buffer, cutlass_gemmrc_splitk.cu:31-42: the caller owns the workspace). */
+/* Bytes of workspace for `split_k` slices: the fp32 partial results [split_k][M][N] and, behind them, the
+ * synchronisation words of the one-launch form (a few KiB).  Replaces the hidden grow-only buffer
+ * get_the_buffer, cutlass_gemmrc_splitk.cu:31-42: the caller owns the workspace.  The workspace never has
+ * to be cleared or prepared, and may be shared by calls of any shapes that do not overlap in time. */
 size_t beam_splitk_workspace_bytes(int M, int N, int split_k);
 /* split_k <= 0: the library chooses (see above; with cfg == NULL the tile is chosen together
  * with its slice count).  The effective factor is clamped to [1, ceil(K/64)].
  * Slice s covers K elements [s*len, (s+1)*len), len = ceil(ceil(K/64)/split_k)*64; partial
- * sums are fp32 in ws[split][M][N]; a second kernel adds them in slice order 0,1,2,... and
- * rounds once, so results are bit-identical from run to run.
+ * sums are fp32 in ws[split][M][N]; they are added in slice order 0,1,2,... and rounded once, so results
+ * are bit-identical from run to run.  One launch: the workgroups that add ride in the same grid behind
+ * the ones that multiply and start on a tile as soon as its slices have signalled (they are placed after
+ * every multiplying workgroup, so what they wait for always arrives; the wait is bounded all the same, by
+ * beam_set_ln_spin_limit: a workgroup that gives up writes NaN, see beam_gemmrc_splitk_timed_out).  Two
+ * launches (partial kernel, reduce kernel; the same bits) for tiles above 128 x 128, N not a multiple of
+ * 4, more than 64 slices, M * N above 2^28, or a workspace that only holds the partial sums
+ * (split_k * M * N * 4 bytes; anything smaller is BEAM_ERR_WORKSPACE).
  * Replaces entry_cutlass_gemmrc_splitk / _spec
  * (cuda/cutlass_kernels/main.cc:17-21, cutlass_gemmrc_splitk.cu:59-105,107-195). */
 int beam_gemmrc_splitk(const void* A, const void* B, void* C, int M, int N, int K, int dtype,
                        const beam_tile_cfg* cfg, int split_k, void* ws, size_t ws_bytes,
                        void* stream);
+/* Waits for `stream`; *timed_out = 1 if a reducing workgroup of the latest one-launch split-K call on this
+ * workspace gave up waiting (its outputs are NaN).  split_k_effective: beam_splitk_effective of that call.
+ * Does not happen on a working device; the bound exists so that no kernel of the library can wait for ever. */
+int beam_gemmrc_splitk_timed_out(const void* ws, int M, int N, int split_k_effective, void* stream, int* timed_out);
+/* on != 0: beam_gemmrc_splitk always runs as two launches.  Off by default (environment:
+ * BEAM_SPLITK_TWO_LAUNCHES=1).  Results are the same bits either way. */
+int beam_set_splitk_two_launches(int on);
 /* The effective split factor beam_gemmrc_splitk would use for these arguments. */
 int beam_splitk_effective(int M, int N, int K, const beam_tile_cfg* cfg, int split_k);
 /* verbose != 0: when the library chooses the slice count itself, beam_gemmrc_splitk writes one line to
@@ -113,7 +128,8 @@ int beam_splitk_effective(int M, int N, int K, const beam_tile_cfg* cfg, int spl
 int beam_set_verbose(int verbose);
 /* beam_gemmrc_splitk without a workspace argument and without any allocation: the fp32 partial sums go
  * into device memory built into the library (a fixed array of beam_splitk_noalloc_max_bytes() = 16 MiB
- * per GPU, present from the first call into the library until the process ends).  No counterpart in
+ * for them, plus 256 KiB for the synchronisation words of the one-launch form, per GPU, present from the
+ * first call into the library until the process ends).  No counterpart in
  * the reference; it is for callers that cannot allocate: code under HIP graph capture, tight serving
  * loops, harnesses that forbid hipMalloc.  Same results as beam_gemmrc_splitk, bit for bit.
  * split_k * M * N * 4 bytes beyond the array's size -> BEAM_ERR_WORKSPACE.  All calls on one GPU share

@@ -1,6 +1,6 @@
 """A captured sequence of operators replays as a HIP graph with the eager results.
 
-The graph holds gemmrc, split-K (two kernels), GEMM+SiLU, the [K][N] matmul, a K = 0 call (its clear is a
+The graph holds gemmrc, split-K (one launch: multiplying and reducing workgroups in one grid), GEMM+SiLU, the [K][N] matmul, a K = 0 call (its clear is a
 kernel, not a memset node), a two-pass GEMM+LayerNorm (what BEAM_LN_AUTO turns into under capture) and an
 explicitly fused one (its workspace keeps its launch count on the device, so replays and the eager calls in
 between simply take turns on it).

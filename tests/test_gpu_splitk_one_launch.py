@@ -1,0 +1,110 @@
+"""Split-K in one launch (reducing workgroups in the same grid as the multiplying ones) against the two-launch
+form (partial kernel, reduce kernel): same bits on every tile the form is built for, on one workspace that is
+never cleared between shapes; the fallbacks; the bounded wait forced to give up from the host."""
+import ctypes
+
+import numpy as np
+import pytest
+
+from test_gpu_gemm import F16, BF16, assert_close
+
+pytestmark = pytest.mark.gpu
+
+SMALL_TILES = [(128, 128, 64, 64), (128, 128, 64, 32), (128, 64, 64, 32), (64, 128, 32, 64), (64, 64, 32, 32)]
+
+
+def _call(beamc, a, b, c, M, N, K, dtype, cfg, split, ws, two_launches):
+    L = beamc.lib
+    assert L.beam_set_splitk_two_launches(1 if two_launches else 0) == 0
+    try:
+        c.fill_bytes(0xEE)
+        cfgp = ctypes.byref(cfg) if cfg is not None else None
+        rc = L.beam_gemmrc_splitk(a.ptr, b.ptr, c.ptr, M, N, K, dtype, cfgp, split, ws.ptr, ws.nbytes, None)
+        assert rc == 0, L.beam_last_error().decode()
+        beamc.sync()
+        return c.to_numpy().copy()
+    finally:
+        L.beam_set_splitk_two_launches(0)
+
+
+def test_one_launch_equals_two_launches(gpu, beamc):
+    """Every small tile x LDS depth on shapes with one and with several rounds of workgroups, ragged M and N,
+    a K tail, both dtypes; the workspace starts as 0x3F bytes and is shared by all cases without clearing."""
+    L = beamc.lib
+    ws = beamc.DeviceArray((64 << 20,), itemsize=1)
+    ws.fill_bytes(0x3F)
+    cases = [(256, 256, 32768, F16, 32), (256, 256, 32768, F16, 16), (64, 128, 65536, F16, 64), (512, 512, 8192, F16, 16),
+             (200, 136, 4104, BF16, 7), (100, 260, 2048, F16, 5), (33, 68, 4096, BF16, 3), (1024, 256, 4096, F16, 4)]
+    seed = 50
+    for (M, N, K, dtype, split) in cases:
+        seed += 1
+        a = beamc.DeviceArray.from_numpy(beamc.host_uniform((M, K), dtype, seed, 0), dtype)
+        b = beamc.DeviceArray.from_numpy(beamc.host_uniform((N, K), dtype, seed, 1), dtype)
+        c = beamc.DeviceArray((M, N), dtype)
+        for (bm, bn, tm, tn) in SMALL_TILES:
+            for pipe in (0, 2):
+                cfg = beamc.TileConfig(bm, bn, tm, tn, pipe, 0).to_c()
+                s = L.beam_splitk_effective(M, N, K, ctypes.byref(cfg), split)
+                assert s > 1 and L.beam_splitk_workspace_bytes(M, N, s) <= ws.nbytes
+                two = _call(beamc, a, b, c, M, N, K, dtype, cfg, split, ws, True)
+                for _ in range(2):  # twice: the second call finds the first one's flags cleared
+                    one = _call(beamc, a, b, c, M, N, K, dtype, cfg, split, ws, False)
+                    assert (one == two).all(), (M, N, K, dtype, split, bm, bn, tm, tn, pipe)
+                assert not (one == 0xEEEE).any()
+                flag = ctypes.c_int(1)
+                assert L.beam_gemmrc_splitk_timed_out(ws.ptr, M, N, s, None, ctypes.byref(flag)) == 0 and flag.value == 0
+        for t in (a, b, c):
+            t.free()
+    ws.free()
+
+
+def test_fallbacks_to_two_launches(gpu, beamc, oracle):
+    """A workspace that holds the partial sums only, N that is not a multiple of 4, a tile above 128 x 128:
+    two launches, same contract."""
+    L = beamc.lib
+    cfg = beamc.TileConfig(64, 64, 32, 32, 2, 0).to_c()
+    for (M, N, K, tile) in ((256, 256, 8192, cfg), (96, 70, 4096, cfg), (512, 512, 4096, beamc.TileConfig(256, 128, 64, 64, 0, 0).to_c())):
+        a_bits = beamc.host_uniform((M, K), F16, 61, 0)
+        b_bits = beamc.host_uniform((N, K), F16, 61, 1)
+        a, b = beamc.DeviceArray.from_numpy(a_bits), beamc.DeviceArray.from_numpy(b_bits)
+        c = beamc.DeviceArray((M, N))
+        s = L.beam_splitk_effective(M, N, K, ctypes.byref(tile), 8)
+        ws = beamc.DeviceArray((s * M * N * 4,), itemsize=1)  # no room for synchronisation words
+        ws.fill_bytes(0x3F)
+        got = _call(beamc, a, b, c, M, N, K, F16, tile, 8, ws, False)
+        assert_close(oracle, got, oracle.gemmrc(a_bits, b_bits, F16), K, F16, f"{M}x{N}x{K}")
+        for t in (a, b, c, ws):
+            t.free()
+
+
+def test_bounded_wait_gives_up_visibly(gpu, beamc):
+    """The reducing workgroups' wait forced to give up from the host (spin limit -1: no poll is ever made):
+    every kernel still ends, the outputs are NaN, the query says so and the checking Python call raises; the
+    next call on the same workspace is clean."""
+    L = beamc.lib
+    M, N, K = 256, 256, 8192
+    a = beamc.DeviceArray.from_numpy(beamc.host_uniform((M, K), F16, 71, 0))
+    b = beamc.DeviceArray.from_numpy(beamc.host_uniform((N, K), F16, 71, 1))
+    c = beamc.DeviceArray((M, N))
+    cfg = beamc.TileConfig(64, 64, 32, 32, 2, 0).to_c()
+    s = L.beam_splitk_effective(M, N, K, ctypes.byref(cfg), 16)
+    ws = beamc.DeviceArray((L.beam_splitk_workspace_bytes(M, N, s),), itemsize=1)
+    good = _call(beamc, a, b, c, M, N, K, F16, cfg, 16, ws, False)
+    assert L.beam_set_ln_spin_limit(-1) == 0
+    try:
+        bad = _call(beamc, a, b, c, M, N, K, F16, cfg, 16, ws, False)
+        flag = ctypes.c_int(0)
+        assert L.beam_gemmrc_splitk_timed_out(ws.ptr, M, N, s, None, ctypes.byref(flag)) == 0 and flag.value == 1
+        assert np.isnan(bad.view(np.float16)).all()
+        with pytest.raises(beamc.BeamError):
+            beamc.gemmrc_splitk_spec(a, b, c, shape_threadblock=(64, 64), shape_warp=(32, 32), split_k_slices=16,
+                                     pipeline=2, check=True)
+    finally:
+        assert L.beam_set_ln_spin_limit(4 << 20) == 0
+    again = _call(beamc, a, b, c, M, N, K, F16, cfg, 16, ws, False)
+    assert (again == good).all()
+    flag = ctypes.c_int(1)
+    assert L.beam_gemmrc_splitk_timed_out(ws.ptr, M, N, s, None, ctypes.byref(flag)) == 0 and flag.value == 0
+    beamc.gemmrc_splitk_spec(a, b, c, shape_threadblock=(64, 64), shape_warp=(32, 32), split_k_slices=16, pipeline=2, check=True)
+    for t in (a, b, c, ws):
+        t.free()

@@ -165,7 +165,12 @@ def test_split_partition(beamc, oracle):
             assert 1 <= eff <= min(s, ktiles)
             L = oracle.split_k_len(K, eff)
             assert L * eff >= K and L * (eff - 1) < K          # no empty slice
-    assert beamc.lib.beam_splitk_workspace_bytes(256, 256, 8) == 8 * 256 * 256 * 4
+    # the fp32 partial sums, 256-byte aligned, then the synchronisation words of the one-launch form:
+    # 64 header words + one flag per (64 x 64 block of C, one of up to 16 parts, slice)
+    for (M, N, S) in ((256, 256, 8), (100, 260, 5), (64, 128, 64), (1, 1, 2)):
+        partial = (S * M * N * 4 + 255) // 256 * 256
+        sync = 4 * (64 + -(-M // 64) * -(-N // 64) * 16 * S)
+        assert beamc.lib.beam_splitk_workspace_bytes(M, N, S) == partial + sync
     assert beamc.lib.beam_splitk_workspace_bytes(0, 256, 8) == 0
 
 
