@@ -167,6 +167,12 @@ def extra_splitk(_C):
                 ms = _C.bench(1, a, b, c, config=pc, split_k=s, warmup=3, iters=20)
                 if ms < best_split[1]:
                     best_split = (f"{pc.name},S={s}", ms, pc, s)
+    # the same (tile, S) as partial kernel + reduce kernel (what the one-launch form replaced)
+    _C.set_splitk_two_launches(True)
+    try:
+        two_ms = min(_C.bench(1, a, b, c, config=best_split[2], split_k=best_split[3], warmup=20, iters=100) for _ in range(2))
+    finally:
+        _C.set_splitk_two_launches(False)
     graph_us = splitk_graph_us(_C, a, b, c, best_split[2], best_split[3])
     cold_us = splitk_graph_us(_C, a, b, c, best_split[2], best_split[3], calls=48, operand_sets=12)
     # what a call that names neither tile nor slice count gets
@@ -185,7 +191,8 @@ def extra_splitk(_C):
     for x in (a, b, c):
         x.free()
     bytes_alg = 2.0 * (M * K + N * K + M * N)
-    return {"shape": [M, N, K], "splitk_us": round(best_split[1] * 1e3, 2), "splitk_config": best_split[0], "floor": floor,
+    return {"shape": [M, N, K], "splitk_us": round(best_split[1] * 1e3, 2), "splitk_config": best_split[0],
+            "launches": 1, "same_config_as_two_launches_us": round(two_ms * 1e3, 2), "floor": floor,
             "splitk_in_graph_us": round(graph_us, 2), "splitk_cold_operands_us": round(cold_us, 2),
             "cold_hbm_GBs": round(2.0 * (M * K + N * K + M * N) / (cold_us * 1e-6) / 1e9, 1),
             "library_choice_us": round(auto_ms * 1e3, 2), "library_choice": f"{auto_cfg.name},S={auto_s}",
@@ -244,10 +251,26 @@ def extra_nn(_C):
     return {"shape": [M, N, K], "us": round(ms * 1e3, 1), "TFLOPs": round(2.0 * M * N * K / (ms * 1e-3) / 1e12, 1)}
 
 
+def settled_ms(measure, window_s=0.025, agree=0.02, max_rounds=6):
+    """Milliseconds per call once successive measurements agree: measure(warmup, iters) is called with enough
+    launches for about `window_s` seconds each until two in a row differ by at most `agree` (at most max_rounds
+    times); the last one is returned.  A few milliseconds of launches after an idle period are timed on a clock
+    that is still rising (2048^3: 25 us per launch over the first 100 launches, 19 us from the 500th on)."""
+    est = max(measure(3, 5), 1e-4)
+    n = int(min(max(window_s * 1e3 / est, 20), 4000))
+    prev = measure(n // 2, n)
+    for _ in range(max_rounds - 1):
+        cur = measure(0, n)
+        if abs(cur - prev) <= agree * prev:
+            return cur
+        prev = cur
+    return prev
+
+
 def extra_sweep(_C):
     """The shape/dtype sweep of the configuration list with the tile the library picks: squares 512 ... 16384,
     the two LLM shapes and the ragged 3000 x 5000 x 2000, fp16 and bf16 (uniform[-1, 1) values), plus a few
-    squares between the powers of two in fp16."""
+    squares between the powers of two in fp16.  Every figure is a settled one (settled_ms)."""
     shapes = [(512, 512, 512), (1024, 1024, 1024), (2048, 2048, 2048), (4096, 4096, 4096), (16384, 16384, 16384),
               (4096, 11008, 4096), (4096, 4096, 11008), (3000, 5000, 2000)]
     more_fp16 = [(3072, 3072, 3072), (6144, 6144, 6144), (7168, 7168, 7168), (16384, 16384, 2048)]
@@ -258,8 +281,7 @@ def extra_sweep(_C):
             b = _C.DeviceArray.from_numpy(_C.host_uniform((N, K), dtype, 5, 1), dtype)
             c = _C.DeviceArray((M, N), dtype)
             cfg, _ = _C.default_config(M, N, K, split=False)
-            big = 2.0 * M * N * K > 2e12
-            ms = min(_C.bench(_C.OP_GEMM, a, b, c, warmup=10 if big else 50, iters=20 if big else 100) for _ in range(2))
+            ms = settled_ms(lambda w, n: _C.bench(_C.OP_GEMM, a, b, c, warmup=w, iters=n))
             for t in (a, b, c):
                 t.free()
             out.append({"shape": [M, N, K], "dtype": name, "tile": cfg.name, "us": round(ms * 1e3, 1),

@@ -150,6 +150,12 @@ int auto_slices(long tiles, int K, int cus) {
   long s = cus / (tiles < 1 ? 1 : tiles);
   if (s > ktiles / 4) s = ktiles / 4;
   if (s > 64) s = 64;  // the reduction reads every slice: 64 x 64 x 32768 takes 9.1 us with 64 slices, 11.4 with 128
+  // Half a round of workgroups with 16 K tiles each beats a full round of shorter slices (every slice pays its
+  // pipeline fill and adds M x N partial sums): 128 x 128 x 32768 takes 8.5 us in 32 slices, 9.6 in 64;
+  // 128 x 256 x 8192 7.8 us in 16, 7.9 in 32.
+  const long half_round = (cus / 2 + tiles - 1) / (tiles < 1 ? 1 : tiles);
+  const long want = ktiles / 16 > half_round ? ktiles / 16 : half_round;
+  if (s > want) s = want;
   return s < 1 ? 1 : (int)s;
 }
 
@@ -389,7 +395,9 @@ int choose_default(int M, int N, int K, int split_req, beam_tile_cfg* cfg, int* 
     const double rate = k.occ == 1 ? k.alone : k.alone + (k.full - k.alone) * (double)(conc - 1) / (k.occ - 1);
     const double mflop = 2.0e-6 * k.cfg.block_m * k.cfg.block_n * (double)K / s;
     double us = (double)((load + k.occ - 1) / k.occ) * k.fixed + (double)load * mflop / rate;
-    if (s > 1) us += 3.0 + (double)s * M * N * 4.0 / 3.0e6;
+    // the partial sums are written through to memory and read back (about 4 TB/s each way), and the reducing
+    // workgroups start behind the multiplying ones
+    if (s > 1) us += 2.0 + (double)s * M * N * 4.0 / 2.0e6;
     if (us < best_us) {
       best_us = us;
       c = k.cfg;
@@ -407,6 +415,10 @@ int choose_default(int M, int N, int K, int split_req, beam_tile_cfg* cfg, int* 
   }
   if (split_req < 0 && tiles(c.block_m, c.block_n) < cus / 2 && K >= 2048)
     cfg->pipeline = 2;  // few workgroups per CU: a long prefetch queue keeps HBM busy
+  // K slices on at most half the CUs: every workgroup has the memory system of two CUs to itself, the long
+  // queue's prologue costs more than it hides (64 x 128 x 65536 in 64 slices: 8.9 against 9.9 us), and the
+  // reducing workgroups of the one-launch form start on the idle CUs at once.
+  if (c_split > 1 && tiles(c.block_m, c.block_n) * c_split <= cus / 2) cfg->pipeline = 0;
   if (split_k) *split_k = c_split;
   return BEAM_OK;
 }

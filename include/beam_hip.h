@@ -88,7 +88,8 @@ int beam_custom_gemmrc_256x128(const void* A, const void* B, void* C, int M, int
  * last round of workgroups that is at least half full, which on this machine (one workgroup
  * of a split-K tile per CU, launch-latency bound) is slower than exactly one full round, so
  * beam_gemmrc_splitk with split_k <= 0 uses floor(CUs / tiles) instead (at most 64, at least
- * 4 K tiles of 64 per slice; 1 when the tiles already fill half the CUs). */
+ * 4 K tiles of 64 per slice, and no more slices than give 16 K tiles each once half the CUs are busy;
+ * 1 when the tiles already fill half the CUs). */
 int beam_slice_heuristic(int tiles, int compute_units);
 /* Bytes of workspace for `split_k` slices: the fp32 partial results [split_k][M][N] and, behind them, the
  * synchronisation words of the one-launch form (a few KiB).  Replaces the hidden grow-only buffer
@@ -272,7 +273,7 @@ int beam_event_destroy(void* event);
 
 /* Every operator above is one or two kernel launches on the caller's stream and neither allocates nor
  * synchronises, so a sequence of them can be captured once and replayed as a HIP graph: the usual cure
- * for launch-bound loops of small GEMMs (a split-K call is two kernels of 13 and 5 us).  The reference
+ * for launch-bound loops of small GEMMs (a split-K call is one launch of 13 us).  The reference
  * has no counterpart (it launches on the legacy default stream, cuda/cute_kernels/cute_gemm_128x128.cu:
  * 203).  Rules: call every operator once eagerly before capturing it (the first launch of a kernel
  * configures its LDS size); BEAM_LN_AUTO takes the two-pass path under capture (BEAM_LN_FUSED is honoured:
