@@ -58,6 +58,26 @@ def test_one_launch_equals_two_launches(gpu, beamc):
     ws.free()
 
 
+def test_new_data_on_a_used_workspace(gpu, beamc):
+    """Call after call on one workspace with different operands: nothing a reducing workgroup reads (partial sums
+    of the previous call at the same addresses, in whatever cache) may be the previous call's."""
+    L = beamc.lib
+    M, N, K = 256, 256, 32768
+    a, b, c = beamc.DeviceArray((M, K)), beamc.DeviceArray((N, K)), beamc.DeviceArray((M, N))
+    s = L.beam_splitk_effective(M, N, K, None, 0)
+    ws = beamc.DeviceArray((L.beam_splitk_workspace_bytes(M, N, s),), itemsize=1)
+    ws2 = beamc.DeviceArray((L.beam_splitk_workspace_bytes(M, N, s),), itemsize=1)
+    for seed in range(80, 86):
+        ha, hb = beamc.host_uniform((M, K), F16, seed, 0), beamc.host_uniform((N, K), F16, seed, 1)
+        beamc._check(L.beam_memcpy_h2d(a.ptr, ha.ctypes.data, ha.nbytes))
+        beamc._check(L.beam_memcpy_h2d(b.ptr, hb.ctypes.data, hb.nbytes))
+        one = _call(beamc, a, b, c, M, N, K, F16, None, 0, ws, False)
+        two = _call(beamc, a, b, c, M, N, K, F16, None, 0, ws2, True)
+        assert (one == two).all(), seed
+    for t in (a, b, c, ws, ws2):
+        t.free()
+
+
 def test_fallbacks_to_two_launches(gpu, beamc, oracle):
     """A workspace that holds the partial sums only, N that is not a multiple of 4, a tile above 128 x 128:
     two launches, same contract."""
