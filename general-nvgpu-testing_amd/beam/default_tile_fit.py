@@ -12,6 +12,14 @@ of 40 launches each, on one MI355X.  `PARAMS` below are the constants compiled i
     python -m beam.default_tile_fit              model's pick per shape against the table, mean / worst regret
     python -m beam.default_tile_fit --refit      coordinate search from PARAMS (what produced them)
     python -m beam.default_tile_fit --collect F  re-measure the table on the GPU at hand into file F
+    python -m beam.default_tile_fit --split      the same for calls with a workspace (split-K): pick against sweep
+    python -m beam.default_tile_fit --collect-split F   re-measure the split-K sweep into file F
+
+With a workspace (beam_gemmrc_splitk, split_k <= 0, no tile given) the deep-pipeline candidates are priced with
+their K slices (`auto_slices`) and the reduction; `splitk_timings.json` holds, for 25 shapes from 64x64x8192 to
+1024x1024x32768, microseconds per call (one launch) of every tile up to 128x128 x {3+2 slots, deep} x
+S in {4, 8, 16, 32, 64} (uniform operands, best of two rounds of 100 calls, one MI355X): the model's pick is what
+`predict_split` restates, and a test keeps it in step with the library.
 
 This stands where the reference has fixed default shapes (cuda/cutlass_kernels/cutlass_gemmrc.cu:22-24).
 """
@@ -40,6 +48,98 @@ PARAMS = {
     "64x64_w32x32": (1.87, 2.9, 2.7), "64x64_w32x32_deep": (2.4, 2.4, 4.0), "64x128_w32x64": (3.15, 3.4, 3.5),
     "64x128_w32x64_deep": (3.3, 3.3, 4.0),
 }
+
+
+SPLIT_TIMINGS = os.path.join(os.path.dirname(os.path.abspath(__file__)), "splitk_timings.json")
+# deep-pipeline candidates (the ones priced with K slices): name -> wavefront tile
+SPLIT_WAVES = {"128x128_w64x32_deep": (64, 32), "128x64_w64x32_deep": (64, 32), "64x64_w32x32_deep": (32, 32),
+               "64x128_w32x64_deep": (32, 64)}
+SPLIT_FIXED_US = 2.0          # the reducing workgroups start behind the multiplying ones
+SPLIT_BYTES_PER_US = 2.0e6    # partial sums written through to memory and read back, ~4 TB/s each way
+
+
+def auto_slices(tiles, K, cus=CUS):
+    """Slices the library takes for `tiles` output tiles (csrc/capi.hip: auto_slices)."""
+    if tiles * 2 > cus:
+        return 1
+    ktiles = (K + 63) // 64
+    s = min(cus // max(tiles, 1), ktiles // 4, 64)
+    half_round = (cus // 2 + tiles - 1) // max(tiles, 1)
+    s = min(s, max(ktiles // 16, half_round))
+    return max(s, 1)
+
+
+def predict_split(params, M, N, K):
+    """(block_m, block_n, pipeline, slices) of the model's pick for a call with a workspace and no slice count."""
+    best = None
+    for name, (bm, bn, occ) in CANDIDATES.items():
+        alone, full, fixed = params[name]
+        tiles = math.ceil(M / bm) * math.ceil(N / bn)
+        s = auto_slices(tiles, K) if name in SPLIT_WAVES else 1
+        load = math.ceil(tiles * s / CUS)
+        conc = min(occ, load)
+        rate = alone if occ == 1 else alone + (full - alone) * (conc - 1) / (occ - 1)
+        mflop = 2.0e-6 * bm * bn * K / s
+        us = math.ceil(load / occ) * fixed + load * mflop / rate
+        if s > 1:
+            us += SPLIT_FIXED_US + s * M * N * 4.0 / SPLIT_BYTES_PER_US
+        if best is None or us < best[0]:
+            best = (us, name, bm, bn, s, tiles)
+    _, name, bm, bn, s, tiles = best
+    pipeline = 2 if name.endswith("_deep") else 0
+    if s > 1 and tiles * s <= CUS // 2:
+        pipeline = 0   # slices on at most half the CUs: the short queue
+    return bm, bn, pipeline, s
+
+
+def split_regret(params, timings, rows=None):
+    """(geometric-mean, worst) ratio of the pick's measured time to the best of the sweep, over the shapes whose
+    pick is in the sweep (its slice counts are powers of two)."""
+    total, worst, n = 0.0, 0.0, 0
+    for key, row in timings.items():
+        M, N, K = map(int, key.split("x"))
+        bm, bn, pipe, s = predict_split(params, M, N, K)
+        t = row.get(f"{bm}x{bn}_p{pipe}_S{s}")
+        best_name = min(row, key=row.get)
+        if rows is not None:
+            rows.append((key, f"{bm}x{bn}_p{pipe}_S{s}", t, best_name, row[best_name]))
+        if t is None:
+            continue
+        r = t / row[best_name]
+        total += math.log(r)
+        worst = max(worst, r)
+        n += 1
+    return math.exp(total / max(n, 1)), worst, n
+
+
+def collect_split(path):
+    """Times every tile up to 128x128 x {3+2, deep} x S in {4..64} on the sweep's shapes on the GPU at hand."""
+    from . import _C
+    out = {}
+    tiles = [(64, 64, 32, 32), (64, 128, 32, 64), (128, 64, 64, 32), (128, 128, 64, 32)]
+    for key in load_timings(SPLIT_TIMINGS):
+        M, N, K = map(int, key.split("x"))
+        a = _C.DeviceArray.from_numpy(_C.host_uniform((M, K), _C.F16, 11, 0))
+        b = _C.DeviceArray.from_numpy(_C.host_uniform((N, K), _C.F16, 11, 1))
+        c = _C.DeviceArray((M, N))
+        res = {}
+        for (bm, bn, tm, tn) in tiles:
+            for pipe in (0, 2):
+                pc = _C.TileConfig(bm, bn, tm, tn, pipe, 0)
+                for s in (4, 8, 16, 32, 64):
+                    if K // 64 // s < 2:
+                        continue
+                    try:
+                        us = min(_C.bench(1, a, b, c, config=pc, split_k=s, warmup=20, iters=100) for _ in range(2)) * 1e3
+                    except _C.BeamError:
+                        continue
+                    res[f"{bm}x{bn}_p{pipe}_S{s}"] = round(us, 2)
+        for x in (a, b, c):
+            x.free()
+        out[key] = res
+        print(key, min(res, key=res.get), min(res.values()), flush=True)
+    with open(path, "w") as f:
+        f.write("{\n" + ",\n".join(f' "{k}": {json.dumps(v)}' for k, v in out.items()) + "\n}\n")
 
 
 def load_timings(path=TIMINGS):
@@ -132,6 +232,18 @@ def collect(path):
 def main(argv):
     if argv[:1] == ["--collect"]:
         collect(argv[1])
+        return 0
+    if argv[:1] == ["--collect-split"]:
+        collect_split(argv[1])
+        return 0
+    if argv[:1] == ["--split"]:
+        rows = []
+        mean, worst, n = split_regret(PARAMS, load_timings(SPLIT_TIMINGS), rows)
+        print("| shape | model's pick | its us | best of the sweep | its us |")
+        print("|---|---|---|---|---|")
+        for key, pick, t, bname, bt in rows:
+            print(f"| {key} | {pick} | {'-' if t is None else f'{t:.2f}'} | {bname} | {bt:.2f} |")
+        print(f"geometric mean {mean:.4f}, worst {worst:.3f} over {n} shapes whose pick is in the sweep")
         return 0
     timings = load_timings()
     params = PARAMS

@@ -319,3 +319,20 @@ def test_default_tile_model_matches_its_table_and_the_library(beamc):
             assert name.startswith(f"{cfg.block_m}x{cfg.block_n}_w{cfg.wave_m}x{cfg.wave_n}"), (key, name, cfg.name)
     mean, worst = fit.regret(fit.PARAMS, timings)
     assert mean < 1.01 and worst < 1.07, (mean, worst)
+
+
+def test_split_choice_matches_its_sweep_and_the_library(beamc):
+    """With a workspace and no slice count, the library's (tile, LDS depth, slices) is what beam/default_tile_fit.py
+    restates, on every shape of the committed split-K sweep; on that sweep the pick costs 1.3% more than the best
+    (tile, depth, slices) on average and 8% at worst."""
+    from beam import default_tile_fit as fit
+    timings = fit.load_timings(fit.SPLIT_TIMINGS)
+    assert len(timings) == 25
+    for key in timings:
+        M, N, K = map(int, key.split("x"))
+        bm, bn, pipe, s = fit.predict_split(fit.PARAMS, M, N, K)
+        cfg, got_s = beamc.default_config(M, N, K, split=True)
+        assert (cfg.block_m, cfg.block_n, cfg.pipeline, got_s) == (bm, bn, pipe, s), (key, cfg.name, got_s, (bm, bn, pipe, s))
+        assert beamc.lib.beam_splitk_effective(M, N, K, None, 0) == s
+    mean, worst, n = fit.split_regret(fit.PARAMS, timings)
+    assert n >= 24 and mean < 1.02 and worst < 1.09, (mean, worst, n)
