@@ -697,21 +697,24 @@ int beam_gemmrc_splitk(const void* A, const void* B, void* C, int M, int N, int 
   // form is built for, 16-byte rows of partial sums, at most one flag per lane, a slice that fits one buffer
   // descriptor, and room for the synchronisation words behind the partial sums.
   const GemmLauncher one_launch = ks->launch_partial_fused[dtype][c.pipeline];
-  const size_t sync_at = align_up(need, 256);
   if (one_launch && !g_splitk_two_launches.load(std::memory_order_relaxed) && N % 4 == 0 && s <= 64 &&
-      (size_t)M * N <= ((size_t)1 << 28) && ws_bytes >= sync_at + (size_t)sk_sync_bytes(M, N, s)) {
-    p.C = C;
-    p.sk_sync = (int*)((char*)ws + sync_at);
-    p.ln_nonce = g_ln_nonce.fetch_add(1, std::memory_order_relaxed) + 1;
-    p.spin_limit = g_ln_spin_limit.load();
-    const int tiles = p.tiles_m * p.tiles_n;
+      (size_t)M * N <= ((size_t)1 << 28)) {
     // parts of 4 outputs per thread, smaller ones while the reducing workgroups are fewer than the CUs
     const int cus = g_dev.cus > 0 ? g_dev.cus : 256;
+    const long tiles = (long)p.tiles_m * p.tiles_n;
     p.sk_out = 4;
     while (p.sk_out > 1 && tiles * sk_parts_per_tile(c.block_m, c.block_n, ks->threads, p.sk_out) < cus) p.sk_out /= 2;
-    const int parts = sk_parts_per_tile(c.block_m, c.block_n, ks->threads, p.sk_out);
-    BEAM_HIP(one_launch(p, dim3((unsigned)(tiles * s + tiles * parts), 1, 1), st));
-    return BEAM_OK;
+    const long parts = sk_parts_per_tile(c.block_m, c.block_n, ks->threads, p.sk_out);
+    const size_t sync_at = align_up(need, 256);
+    const size_t sync_bytes = 4 * ((size_t)kSkFlags + (size_t)(tiles * parts) * (size_t)s);
+    if (ws_bytes >= sync_at + sync_bytes && tiles * (s + parts) < (1l << 30)) {
+      p.C = C;
+      p.sk_sync = (int*)((char*)ws + sync_at);
+      p.ln_nonce = g_ln_nonce.fetch_add(1, std::memory_order_relaxed) + 1;
+      p.spin_limit = g_ln_spin_limit.load();
+      BEAM_HIP(one_launch(p, dim3((unsigned)(tiles * s + tiles * parts), 1, 1), st));
+      return BEAM_OK;
+    }
   }
   BEAM_HIP(ks->launch[dtype][kEpiPartial][c.pipeline](p, dim3((unsigned)(p.tiles_m * p.tiles_n * s), 1, 1), st));
   BEAM_HIP(launch_splitk_reduce((const float*)ws, C, (size_t)M * N, s, dtype, st));

@@ -75,10 +75,10 @@ constexpr int kSkFlags = 64;
 __host__ __device__ constexpr int sk_parts_per_tile(int block_m, int block_n, int threads, int out) {
   return block_m * block_n / (threads * out);
 }
-// Bytes of synchronisation words that are enough for any tile of the library (every tile is at least 64 x 64
-// and every part at least 256 outputs): ceil(M/64) * ceil(N/64) * 16 parts * splits flags.
+// Bytes of synchronisation words that are enough for any tile the one-launch form is built for (up to 128 x 128;
+// a part is at least 256 outputs, and the tiles cover at most (M + 127) x (N + 127) outputs).
 __host__ __device__ constexpr unsigned long long sk_sync_bytes(int M, int N, int splits) {
-  return 4ull * (kSkFlags + (unsigned long long)((M + 63) / 64) * ((N + 63) / 64) * 16ull * (unsigned long long)splits);
+  return 4ull * (kSkFlags + ((unsigned long long)(M + 127) * (unsigned long long)(N + 127) / 256ull + 1ull) * (unsigned long long)splits);
 }
 
 struct TileCoord {

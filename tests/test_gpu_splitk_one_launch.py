@@ -34,7 +34,8 @@ def test_one_launch_equals_two_launches(gpu, beamc):
     ws = beamc.DeviceArray((64 << 20,), itemsize=1)
     ws.fill_bytes(0x3F)
     cases = [(256, 256, 32768, F16, 32), (256, 256, 32768, F16, 16), (64, 128, 65536, F16, 64), (512, 512, 8192, F16, 16),
-             (200, 136, 4104, BF16, 7), (100, 260, 2048, F16, 5), (33, 68, 4096, BF16, 3), (1024, 256, 4096, F16, 4)]
+             (200, 136, 4104, BF16, 7), (100, 260, 2048, F16, 5), (33, 68, 4096, BF16, 3), (1024, 256, 4096, F16, 4),
+             (65, 64, 4096, F16, 8)]  # (a sliver of a second 128-row tile: as many flags as a whole one)
     seed = 50
     for (M, N, K, dtype, split) in cases:
         seed += 1

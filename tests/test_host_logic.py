@@ -166,10 +166,11 @@ def test_split_partition(beamc, oracle):
             L = oracle.split_k_len(K, eff)
             assert L * eff >= K and L * (eff - 1) < K          # no empty slice
     # the fp32 partial sums, 256-byte aligned, then the synchronisation words of the one-launch form:
-    # 64 header words + one flag per (64 x 64 block of C, one of up to 16 parts, slice)
+    # 64 header words + one flag per (part of at least 256 outputs of the at most (M + 127) x (N + 127) that
+    # tiles up to 128 x 128 cover, slice)
     for (M, N, S) in ((256, 256, 8), (100, 260, 5), (64, 128, 64), (1, 1, 2)):
         partial = (S * M * N * 4 + 255) // 256 * 256
-        sync = 4 * (64 + -(-M // 64) * -(-N // 64) * 16 * S)
+        sync = 4 * (64 + ((M + 127) * (N + 127) // 256 + 1) * S)
         assert beamc.lib.beam_splitk_workspace_bytes(M, N, S) == partial + sync
     assert beamc.lib.beam_splitk_workspace_bytes(0, 256, 8) == 0
 
@@ -336,3 +337,19 @@ def test_split_choice_matches_its_sweep_and_the_library(beamc):
         assert beamc.lib.beam_splitk_effective(M, N, K, None, 0) == s
     mean, worst, n = fit.split_regret(fit.PARAMS, timings)
     assert n >= 24 and mean < 1.02 and worst < 1.09, (mean, worst, n)
+
+
+def test_splitk_workspace_query_covers_every_small_tile(beamc):
+    """beam_splitk_workspace_bytes leaves room for the flags of the one-launch form whatever tile (up to 128 x 128)
+    and part size the call ends up with: one flag per (tile, part, slice), parts as small as one output per thread."""
+    small = [(cfg.block_m, cfg.block_n, (cfg.block_m // cfg.wave_m) * (cfg.block_n // cfg.wave_n) * 64)
+             for cfg in beamc.list_configs() if cfg.block_m * cfg.block_n <= 128 * 128]
+    assert len(small) >= 5
+    for M in (1, 63, 64, 65, 127, 129, 200, 256, 257, 1000, 4097):
+        for N in (4, 60, 64, 68, 128, 132, 260, 1024, 4100):
+            for S in (2, 7, 64):
+                have = beamc.lib.beam_splitk_workspace_bytes(M, N, S) - (S * M * N * 4 + 255) // 256 * 256
+                for bm, bn, threads in small:
+                    tiles = -(-M // bm) * -(-N // bn)
+                    parts = bm * bn // threads  # one output per thread
+                    assert have >= 4 * (64 + tiles * parts * S), (M, N, S, bm, bn)
