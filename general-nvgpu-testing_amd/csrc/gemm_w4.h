@@ -309,8 +309,13 @@ struct GemmW4 {
       return o;
     };
     OutTile out = out_tile_of(-1, TileCoord{0, 0});  // the tile whose accumulators are being stored
-    auto store_pair = [&](auto i_tag, auto q_tag) __attribute__((always_inline)) {
+    // LAST: the stores after the workgroup's last K loop.  Nothing hides them, and a kernel ends only when its
+    // dirty lines have left the L2: those go through it to memory at once (device-scope stores; 4096^3, one tile
+    // per workgroup: 98.9 -> 96.5 us, fused LayerNorm 105.7 -> 103.7 us).  The stores of earlier tiles lie under
+    // the next tile's MFMAs and stay plain (written through, 8192^3 loses 0.2%).
+    auto store_pair = [&](auto i_tag, auto q_tag, auto last_tag) __attribute__((always_inline)) {
       constexpr int i = decltype(i_tag)::value, q = decltype(q_tag)::value;
+      constexpr int AUX = C_NT ? 2 : (decltype(last_tag)::value ? kAuxDeviceScope : 0);
       constexpr int R0 = 4 * (8 * i + 2 * q);  // first register of block (i, 2 q); block (i, 2 q + 1) follows
       vec8 v;
       v[0] = (T)w4_acc_read<R0 + 0>();
@@ -324,7 +329,7 @@ struct GemmW4 {
       const int skip = i * 16 * N * 2;  // bytes of the row blocks above this one
       const int left = out.bytes - skip;
       const __amdgpu_buffer_rsrc_t rsrc = make_rsrc(out.base + skip, left > 0 ? (unsigned)left : 0u);
-      __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(i32x4, v), rsrc, (int)out.voff[q], 0, C_NT ? 2 : 0);
+      __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(i32x4, v), rsrc, (int)out.voff[q], 0, AUX);
     };
 
     // ---- one K tile ------------------------------------------------------------------------------
@@ -386,7 +391,7 @@ struct GemmW4 {
         if constexpr (half == 1 && m > LAST_A && m <= LAST_A + 3) advance(ld_a, wrap_a, next_a, 0, B_REGION, m - LAST_A - 1);
         if constexpr (FIRST && !LN && gap >= 10 && gap < 10 + 8 * FM && ((gap - 10) & 1) == 0) {
           // pair q of row block i goes into gap 10 + 8 i + 2 q
-          store_pair(std::integral_constant<int, (gap - 10) / 8>{}, std::integral_constant<int, ((gap - 10) / 2) % 4>{});
+          store_pair(std::integral_constant<int, (gap - 10) / 8>{}, std::integral_constant<int, ((gap - 10) / 2) % 4>{}, std::false_type{});
         }
         __builtin_amdgcn_sched_barrier(0);
       });
@@ -435,7 +440,7 @@ struct GemmW4 {
       if constexpr (!LN) {
         w4_static_for<0, FM * FN / 2>([&](auto o_tag) __attribute__((always_inline)) {
           constexpr int o = decltype(o_tag)::value;
-          store_pair(std::integral_constant<int, o / 4>{}, std::integral_constant<int, o % 4>{});
+          store_pair(std::integral_constant<int, o / 4>{}, std::integral_constant<int, o % 4>{}, std::true_type{});
         });
       } else {
         layer_norm_epilogue(p, smem, ln_tile, out);
@@ -584,7 +589,7 @@ struct GemmW4 {
           constexpr int e = decltype(e_tag)::value;
           v[e] = (T)((w4_acc_read<4 * (8 * i + 2 * q) + e>() - mean) * rstd * (float)gv[q][e] + (float)bv[q][e]);
         });
-        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(i32x4, v), rsrc, (int)out.voff[q], 0, 0);
+        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(i32x4, v), rsrc, (int)out.voff[q], 0, kAuxDeviceScope);
       });
     });
   }
