@@ -186,7 +186,8 @@ int beam_gemmrc_ln_timed_out(const void* ws, void* stream, int* timed_out);
 /* Bound of that wait: polls of statistics slots per thread (roughly a microsecond each; default
  * 4 Mi).  0 makes every thread that finds a slot unpublished give up at once; -1 makes every wait give
  * up whatever it finds: the kernel still ends normally and the flag is set, which is how the failure
- * path is exercised without hanging anything. */
+ * path is exercised without hanging anything.  The same number bounds the wait of the reducing workgroups
+ * of the one-launch split-K (polls of a tile's flags). */
 int beam_set_ln_spin_limit(int polls);
 
 /* ---- GEMM with an independent elementwise job hidden in its K loop ------------------------ */
