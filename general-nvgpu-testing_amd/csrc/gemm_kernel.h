@@ -376,6 +376,9 @@ struct GemmTile {
       }
       __builtin_amdgcn_s_sleep(1);
     }
+    // The partial sums are read after the flags, in the hardware (the loop's exit waits for the flags' values) and
+    // in the compiler (relaxed atomic loads order nothing by themselves; the loads below must not be hoisted).
+    asm volatile("" ::: "memory");
     const int m = tm * BM + q * PART_ROWS + tid / (BN / OUT);
     const int n = tn * BN + (tid % (BN / OUT)) * OUT;
     const bool valid = m < M && n < N;  // N is a multiple of 4: a thread's columns exist together
