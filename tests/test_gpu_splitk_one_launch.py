@@ -59,6 +59,38 @@ def test_one_launch_equals_two_launches(gpu, beamc):
     ws.free()
 
 
+def test_random_shapes_tiles_and_slice_counts(gpu, beamc):
+    """80 seeded random problems (ragged M, N a multiple of 4, K a multiple of 8 with tails inside slices), random
+    small tile, LDS depth and slice count, both dtypes, one never-cleared workspace: the two forms agree bit for bit."""
+    L = beamc.lib
+    rng = np.random.default_rng(20240607)
+    ws = beamc.DeviceArray((96 << 20,), itemsize=1)
+    ws.fill_bytes(0xA5)
+    done = 0
+    while done < 80:
+        M = int(rng.integers(1, 700))
+        N = 4 * int(rng.integers(1, 176))
+        K = 8 * int(rng.integers(16, 1200))
+        dtype = F16 if rng.random() < 0.6 else BF16
+        bm, bn, tm, tn = SMALL_TILES[int(rng.integers(0, len(SMALL_TILES)))]
+        pipe = int(rng.choice([0, 1, 2]))
+        split = int(rng.choice([0, 2, 3, 5, 8, 13, 16, 32, 64]))
+        cfg = beamc.TileConfig(bm, bn, tm, tn, pipe, 0).to_c()
+        s = L.beam_splitk_effective(M, N, K, ctypes.byref(cfg), split)
+        if s <= 1 or L.beam_splitk_workspace_bytes(M, N, s) > ws.nbytes:
+            continue
+        a = beamc.DeviceArray.from_numpy(beamc.host_uniform((M, K), dtype, 900 + done, 0), dtype)
+        b = beamc.DeviceArray.from_numpy(beamc.host_uniform((N, K), dtype, 900 + done, 1), dtype)
+        c = beamc.DeviceArray((M, N), dtype)
+        two = _call(beamc, a, b, c, M, N, K, dtype, cfg, split, ws, True)
+        one = _call(beamc, a, b, c, M, N, K, dtype, cfg, split, ws, False)
+        assert (one == two).all(), (M, N, K, dtype, (bm, bn, tm, tn), pipe, split, s)
+        for t in (a, b, c):
+            t.free()
+        done += 1
+    ws.free()
+
+
 def test_new_data_on_a_used_workspace(gpu, beamc):
     """Call after call on one workspace with different operands: nothing a reducing workgroup reads (partial sums
     of the previous call at the same addresses, in whatever cache) may be the previous call's."""
