@@ -198,6 +198,7 @@ GemmParams base_params(const void* A, const void* B, int M, int N, int K, const 
   if (p.k_slice == 0) p.k_slice = kBK;
   p.splits = 1;
   p.group_m = c.group_m;
+  p.divs = make_tile_divs(p.tiles_m, p.tiles_n, p.group_m);
   return p;
 }
 
@@ -1178,11 +1179,23 @@ int beam_host_fill_normal(void* dst_host, size_t n, int dtype, uint64_t seed, ui
 int beam_dbg_tile_of_workgroup(int wg, int tiles_m, int tiles_n, int group_m, int* tm, int* tn) {
   if (tiles_m < 1 || tiles_n < 1 || group_m < 1 || wg < 0 || wg >= tiles_m * tiles_n || !tm || !tn)
     return fail(BEAM_ERR_INVALID, "bad rasterisation query");
+  const TileDivs dv = make_tile_divs(tiles_m, tiles_n, group_m);
+  const TileCoord t = tile_of_workgroup(wg, tiles_m, tiles_n, group_m, dv);
+  *tm = t.tm;
+  *tn = t.tn;
+  return BEAM_OK;
+}
+
+int beam_dbg_tile_of_workgroup_by_division(int wg, int tiles_m, int tiles_n, int group_m, int* tm, int* tn) {
+  if (tiles_m < 1 || tiles_n < 1 || group_m < 1 || wg < 0 || wg >= tiles_m * tiles_n || !tm || !tn)
+    return fail(BEAM_ERR_INVALID, "bad rasterisation query");
   const TileCoord t = tile_of_workgroup(wg, tiles_m, tiles_n, group_m);
   *tm = t.tm;
   *tn = t.tn;
   return BEAM_OK;
 }
+
+unsigned beam_dbg_fast_div(unsigned n, unsigned d) { return fast_div(n, make_fast_div(d)); }
 
 int beam_dbg_band_xcd_tile(int wg, int tiles_m, int tiles_n, int bx, int* tm, int* tn) {
   if (tiles_m < 1 || tiles_n < 1 || bx < 1 || wg < 0 || wg >= band_xcd_grid(tiles_m, tiles_n, bx) || !tm || !tn)

@@ -119,6 +119,7 @@ struct GemmParams {
   int splits;    // number of K slices (1 = no split); the grid holds tiles_m * tiles_n * splits workgroups
   int group_m;   // rasterisation group height in tiles (fused LayerNorm: bands per band group)
   int group_n;   // fused LayerNorm: columns of a band group owned by one XCD; 0: whole bands, group_m of them, per XCD
+  TileDivs divs; // the tile maps' divisors as multipliers (tile_map.h), made by the host from tiles_m, tiles_n, group_m
   // Side job (kEpiStoreSide): y[i] = silu(x[i]) over a flat 16-bit array.  The whole 8-element
   // groups of the array are cut into units of side_width bytes (16, 8 or 4), dealt out in
   // contiguous runs of side_iters * threads units per workgroup, `threads` units per K tile; the
@@ -457,10 +458,10 @@ struct GemmTile {
     } else if (p.splits > 1) {
       const int tiles = p.tiles_m * p.tiles_n;
       const int pid = xcd_remap(blockIdx.x, tiles * p.splits);
-      slice = pid / tiles;
-      tc = grouped_tile(pid - slice * tiles, p.tiles_m, p.tiles_n, p.group_m);
+      slice = (int)fast_div((unsigned)pid, p.divs.tiles);
+      tc = grouped_tile(pid - slice * tiles, p.tiles_m, p.tiles_n, p.group_m, p.divs);
     } else {
-      tc = tile_of_workgroup(blockIdx.x, p.tiles_m, p.tiles_n, p.group_m);
+      tc = tile_of_workgroup(blockIdx.x, p.tiles_m, p.tiles_n, p.group_m, p.divs);
     }
     int row0 = tc.tm * BM;
     int col0 = tc.tn * BN;
@@ -490,7 +491,7 @@ struct GemmTile {
     // kEpiStoreLoop: the same for the next tile of this workgroup (neither split-K nor the [K][N]
     // layout nor a short K tile exist in that mode: the host sees to it)
     auto set_tile = [&](int id) __attribute__((always_inline)) {
-      tc = tile_of_workgroup(id, p.tiles_m, p.tiles_n, p.group_m);
+      tc = tile_of_workgroup(id, p.tiles_m, p.tiles_n, p.group_m, p.divs);
       row0 = tc.tm * BM;
       col0 = tc.tn * BN;
       rows_a = (M - row0) < BM ? (M - row0) : BM;
@@ -625,7 +626,6 @@ struct GemmTile {
 #pragma unroll
           for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.0f;
     };
-    zero_acc();
 
     // Fragments: both operands are double-buffered in registers (set 0 / set 1).  While the MFMAs
     // of one step consume one set, the LDS reads of the next step fill the other.  They start as
@@ -647,7 +647,6 @@ struct GemmTile {
           fb1[j][e] = 0;
         }
     };
-    zero_fragments();
 
     // ---- side job: state and pieces ------------------------------------------------------
     // side_buf holds the units loaded during the previous K tile; step 1 pushes them through silu
@@ -888,8 +887,13 @@ struct GemmTile {
           else acc[i][j] = Traits::mfma(fb1[j], fa1[i], acc[i][j]);
         }
     };
+    // The first operand tiles are on their way before anything else is set up: accumulators and fragments are
+    // cleared while they travel (a workgroup lives 3-5 us at 512^3 and 1024^3; every 0.1 us in front of its first
+    // load is 2-3% of it).
+    if (n_tiles > 0) issue_prologue();
+    zero_acc();
+    zero_fragments();
     if (n_tiles > 0) {
-      issue_prologue();
       if (SIDE && loader) {
         side_store(-1, W4{});  // dropped; keeps the number of side operations per tile uniform
         if (p.side_width == 16) side_load(0, W16{});

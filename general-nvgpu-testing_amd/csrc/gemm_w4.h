@@ -203,7 +203,7 @@ struct GemmW4 {
     // past its last tile: such loads are issued and counted like any other and touch no memory.
     auto tile_coord = [&](int j) {
       if constexpr (LN) return ln_tile;
-      else return tile_of_workgroup(first_tile + j * tile_step, p.tiles_m, p.tiles_n, p.group_m);
+      else return tile_of_workgroup(first_tile + j * tile_step, p.tiles_m, p.tiles_n, p.group_m, p.divs);
     };
     auto rows_of_a = [&](int j, TileCoord tc) {
       if (j >= my_tiles) return make_rsrc(p.A, 0u);

@@ -96,6 +96,45 @@ BEAM_HD int xcd_remap(int wg, int total) {
   return xcd * base + (xcd < rem ? xcd : rem) + local;
 }
 
+// Division of a number below 2^31 by a divisor known on the host: one multiply-high and a shift in the kernel
+// instead of the ~25 instructions (and a round trip through the vector unit's reciprocal) of a division by a
+// run-time value.  Three of those in a row stood between a workgroup's start and its first load: 0.15 us of
+// a 1024^3 launch's 5.3.  mul = ceil(2^(31 + ceil(log2 d)) / d), shift = ceil(log2 d) - 1; d = 1: mul = 0.
+struct FastDiv {
+  unsigned mul;
+  unsigned shift;
+};
+BEAM_HD FastDiv make_fast_div(unsigned d) {
+  FastDiv f = {0u, 0u};
+  if (d <= 1u) return f;
+  unsigned lg = 0;
+  while ((1ull << lg) < d) ++lg;  // ceil(log2 d), >= 1
+  const unsigned long long p2 = 1ull << (31 + lg);
+  f.mul = (unsigned)((p2 + d - 1) / d);
+  f.shift = lg - 1;
+  return f;
+}
+BEAM_HD unsigned fast_div(unsigned n, FastDiv f) {
+  return f.mul == 0u ? n : (unsigned)(((unsigned long long)n * f.mul) >> 32) >> f.shift;
+}
+// The divisors of a launch's tile maps (made once on the host, passed with the kernel's arguments).
+struct TileDivs {
+  FastDiv group;      // group_m * tiles_n: tiles per group of tile rows
+  FastDiv rows;       // group_m: tile rows of a full group
+  FastDiv rows_last;  // tile rows of the last, short group (= rows when tiles_m is a multiple of group_m)
+  FastDiv tiles;      // tiles_m * tiles_n (split-K: workgroup -> slice)
+};
+BEAM_HD TileDivs make_tile_divs(int tiles_m, int tiles_n, int group_m) {
+  TileDivs d;
+  const int g = group_m < 1 ? 1 : group_m;
+  d.group = make_fast_div((unsigned)(g * tiles_n));
+  d.rows = make_fast_div((unsigned)g);
+  const int last = tiles_m % g;
+  d.rows_last = make_fast_div((unsigned)(last ? last : g));
+  d.tiles = make_fast_div((unsigned)(tiles_m * tiles_n));
+  return d;
+}
+
 // Linear tile id -> (tm, tn): groups of `group_m` tile rows, M fastest inside a group, so
 // that workgroups with neighbouring ids reuse the same B panel and a small set of A panels
 // out of the XCD-private L2.
@@ -164,6 +203,24 @@ BEAM_HD int band_xcd_grid(int tiles_m, int tiles_n, int bx) {
 
 BEAM_HD TileCoord tile_of_workgroup(int wg, int tiles_m, int tiles_n, int group_m) {
   return grouped_tile(xcd_remap(wg, tiles_m * tiles_n), tiles_m, tiles_n, group_m);
+}
+
+// The same maps with the divisions done by multiplication (what the kernels call; a host test walks both over
+// every workgroup of many grids).
+BEAM_HD TileCoord grouped_tile(int pid, int tiles_m, int tiles_n, int group_m, const TileDivs& dv) {
+  const int gsize = group_m * tiles_n;
+  const int g = (int)fast_div((unsigned)pid, dv.group);
+  const int first_m = g * group_m;
+  const bool short_group = tiles_m - first_m < group_m;
+  const int rows = short_group ? tiles_m - first_m : group_m;
+  const int within = pid - g * gsize;
+  TileCoord t;
+  t.tn = (int)fast_div((unsigned)within, short_group ? dv.rows_last : dv.rows);
+  t.tm = first_m + within - t.tn * rows;
+  return t;
+}
+BEAM_HD TileCoord tile_of_workgroup(int wg, int tiles_m, int tiles_n, int group_m, const TileDivs& dv) {
+  return grouped_tile(xcd_remap(wg, tiles_m * tiles_n), tiles_m, tiles_n, group_m, dv);
 }
 
 // K range [begin, end) of split slice `z` out of `splits`: every slice gets the same whole

@@ -310,8 +310,12 @@ int beam_host_fill_normal(void* dst_host, size_t n, int dtype, uint64_t seed, ui
 
 /* ---- index maps, exported for host-side verification ---------------------------------------- */
 
-/* Workgroup id -> (tile_m, tile_n) as the kernels compute it. */
+/* Workgroup id -> (tile_m, tile_n) as the kernels compute it (divisions done as multiplications by constants the
+ * host prepares), and the same map written with plain divisions, which defines it. */
 int beam_dbg_tile_of_workgroup(int wg, int tiles_m, int tiles_n, int group_m, int* tm, int* tn);
+int beam_dbg_tile_of_workgroup_by_division(int wg, int tiles_m, int tiles_n, int group_m, int* tm, int* tn);
+/* n / d (n < 2^31, d >= 1) through the multiplier the host would prepare for d. */
+unsigned beam_dbg_fast_div(unsigned n, unsigned d);
 /* Byte offset of (row, 16-byte chunk) inside an LDS stage. */
 int beam_dbg_lds_offset(int row, int chunk);
 /* Byte offset of element (k, n), n a multiple of 4, inside a K-major LDS stage of block_n columns

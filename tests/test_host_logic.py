@@ -353,3 +353,40 @@ def test_splitk_workspace_query_covers_every_small_tile(beamc):
                     tiles = -(-M // bm) * -(-N // bn)
                     parts = bm * bn // threads  # one output per thread
                     assert have >= 4 * (64 + tiles * parts * S), (M, N, S, bm, bn)
+
+
+def test_division_by_multiplication(beamc):
+    """The kernels divide by launch constants with a multiply-high and a shift (tile_map.h: FastDiv): exact for
+    every numerator below 2^31, checked on small numbers exhaustively, around every multiple of the divisor that a
+    sample reaches, and at the top of the range."""
+    import ctypes
+    L = beamc.lib
+    L.beam_dbg_fast_div.argtypes = [ctypes.c_uint, ctypes.c_uint]
+    L.beam_dbg_fast_div.restype = ctypes.c_uint
+    rng = np.random.default_rng(5)
+    divisors = list(range(1, 200)) + [255, 256, 257, 1000, 1023, 1024, 1025, 4095, 4096, 4097, 65535, 65536, 65537,
+                                       (1 << 20) + 7, (1 << 30) - 1, 1 << 30, (1 << 31) - 1]
+    for d in divisors:
+        ns = set(range(0, 600)) | {(1 << 31) - 1, (1 << 31) - 2, (1 << 30), (1 << 30) + 1}
+        for k in rng.integers(0, ((1 << 31) - 1) // d + 1, 40):
+            for off in (-1, 0, 1):
+                n = int(k) * d + off
+                if 0 <= n < (1 << 31):
+                    ns.add(n)
+        for n in ns:
+            assert L.beam_dbg_fast_div(n, d) == n // d, (n, d)
+
+
+def test_tile_map_with_multipliers_is_the_map_with_divisions(beamc):
+    """What the kernels compute (multipliers prepared on the host) against the map's definition, for every
+    workgroup of many grids, raster groups that divide the tile rows and ones that leave a short last group."""
+    import ctypes
+    L = beamc.lib
+    tm, tn, um, un = (ctypes.c_int() for _ in range(4))
+    grids = [(1, 1), (1, 7), (7, 1), (2, 3), (4, 4), (5, 9), (16, 16), (12, 20), (13, 11), (32, 32), (43, 16), (16, 43), (64, 3)]
+    for tiles_m, tiles_n in grids:
+        for g in (1, 2, 3, 4, 8, 16):
+            for wg in range(tiles_m * tiles_n):
+                assert L.beam_dbg_tile_of_workgroup(wg, tiles_m, tiles_n, g, ctypes.byref(tm), ctypes.byref(tn)) == 0
+                assert L.beam_dbg_tile_of_workgroup_by_division(wg, tiles_m, tiles_n, g, ctypes.byref(um), ctypes.byref(un)) == 0
+                assert (tm.value, tn.value) == (um.value, un.value), (tiles_m, tiles_n, g, wg)
