@@ -708,7 +708,11 @@ int beam_gemmrc_splitk(const void* A, const void* B, void* C, int M, int N, int 
     const long parts = sk_parts_per_tile(c.block_m, c.block_n, ks->threads, p.sk_out);
     const size_t sync_at = align_up(need, 256);
     const size_t sync_bytes = 4 * ((size_t)kSkFlags + (size_t)(tiles * parts) * (size_t)s);
-    if (ws_bytes >= sync_at + sync_bytes && tiles * (s + parts) < (1l << 30)) {
+    // Many tiles make many reducing workgroups, and those carry the kernel's LDS allocation: one per CU at a time,
+    // round after round behind the last multiplying workgroups.  Beyond two rounds of them the reduce kernel of the
+    // two-launch form, which spreads over the CUs at once, is the faster end (2048 x 1024 x 4096 in 2 slices of
+    // 128 x 128 tiles: 25.7 against 27.2 us; 1024 x 1024 x 8192 in 4: 25.9 against 24.8 the other way).
+    if (ws_bytes >= sync_at + sync_bytes && tiles * parts <= 2l * cus) {
       p.C = C;
       p.sk_sync = (int*)((char*)ws + sync_at);
       p.ln_nonce = g_ln_nonce.fetch_add(1, std::memory_order_relaxed) + 1;

@@ -105,7 +105,8 @@ size_t beam_splitk_workspace_bytes(int M, int N, int split_k);
  * every multiplying workgroup, so what they wait for always arrives; the wait is bounded all the same, by
  * beam_set_ln_spin_limit: a workgroup that gives up writes NaN, see beam_gemmrc_splitk_timed_out).  Two
  * launches (partial kernel, reduce kernel; the same bits) for tiles above 128 x 128, N not a multiple of
- * 4, more than 64 slices, M * N above 2^28, or a workspace that only holds the partial sums
+ * 4, more than 64 slices, M * N above 2^28, outputs so large that the adding workgroups would need more than
+ * two rounds of the CUs, or a workspace that only holds the partial sums
  * (split_k * M * N * 4 bytes; anything smaller is BEAM_ERR_WORKSPACE).
  * Replaces entry_cutlass_gemmrc_splitk / _spec
  * (cuda/cutlass_kernels/main.cc:17-21, cutlass_gemmrc_splitk.cu:59-105,107-195). */
