@@ -18,7 +18,8 @@ of 40 launches each, on one MI355X.  `PARAMS` below are the constants compiled i
 With a workspace (beam_gemmrc_splitk, split_k <= 0, no tile given) the deep-pipeline candidates are priced with
 their K slices (`auto_slices`) and the reduction; `splitk_timings.json` holds, for 25 shapes from 64x64x8192 to
 1024x1024x32768, microseconds per call (one launch) of every tile up to 128x128 x {3+2 slots, deep} x
-S in {4, 8, 16, 32, 64} (uniform operands, best of two rounds of 100 calls, one MI355X): the model's pick is what
+S in {4, 8, 16, 32, 64} (uniform operands, best of two rounds of 100 calls, one MI355X, the library as shipped:
+one launch or two as it decides): the model's pick is what
 `predict_split` restates, and a test keeps it in step with the library.
 
 This stands where the reference has fixed default shapes (cuda/cutlass_kernels/cutlass_gemmrc.cu:22-24).

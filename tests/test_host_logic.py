@@ -324,8 +324,8 @@ def test_default_tile_model_matches_its_table_and_the_library(beamc):
 
 def test_split_choice_matches_its_sweep_and_the_library(beamc):
     """With a workspace and no slice count, the library's (tile, LDS depth, slices) is what beam/default_tile_fit.py
-    restates, on every shape of the committed split-K sweep; on that sweep the pick costs 1.3% more than the best
-    (tile, depth, slices) on average and 8% at worst."""
+    restates, on every shape of the committed split-K sweep; on that sweep the pick costs 2.4% more than the best
+    (tile, depth, slices) on average and 15% at worst (two mid-size shapes where 128 x 128 tiles win)."""
     from beam import default_tile_fit as fit
     timings = fit.load_timings(fit.SPLIT_TIMINGS)
     assert len(timings) == 25
@@ -336,7 +336,7 @@ def test_split_choice_matches_its_sweep_and_the_library(beamc):
         assert (cfg.block_m, cfg.block_n, cfg.pipeline, got_s) == (bm, bn, pipe, s), (key, cfg.name, got_s, (bm, bn, pipe, s))
         assert beamc.lib.beam_splitk_effective(M, N, K, None, 0) == s
     mean, worst, n = fit.split_regret(fit.PARAMS, timings)
-    assert n >= 24 and mean < 1.02 and worst < 1.09, (mean, worst, n)
+    assert n >= 24 and mean < 1.03 and worst < 1.17, (mean, worst, n)
 
 
 def test_splitk_workspace_query_covers_every_small_tile(beamc):
