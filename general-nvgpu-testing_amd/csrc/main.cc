@@ -232,8 +232,8 @@ BEAM_TEST(one_hot_k_tail) {
   return c;
 }
 
-// Split-K: one slice is the plain kernel bit for bit; S slices agree with it to fp32 reorder noise and
-// are bit-identical from run to run.
+// Split-K: one slice is the plain kernel bit for bit; S slices agree with it to fp32 reorder noise, are
+// bit-identical from run to run, and give the same bits in one launch and in two.
 BEAM_TEST(splitk_consistency) {
   Check c;
   const int M = 256, N = 256, K = 8192;
@@ -261,6 +261,19 @@ BEAM_TEST(splitk_consistency) {
         break;
       }
     }
+    // the same slices as partial kernel + reduce kernel, and on a workspace that holds the partial sums only
+    // (no room for the one-launch form's flags): the same bits as the one launch above
+    BEAM_REQUIRE(c, beam_set_splitk_two_launches(1));
+    const int rc_two = beam_gemmrc_splitk(da.p, db.p, dc.p, M, N, K, BEAM_F16, &cfg, s, dw.p, dw.bytes, nullptr);
+    beam_set_splitk_two_launches(0);
+    BEAM_REQUIRE(c, rc_two);
+    if (dc.download16() != first) c.fail("split_k = " + std::to_string(s) + ": two launches differ from one");
+    const int eff = beam_splitk_effective(M, N, K, &cfg, s);
+    BEAM_REQUIRE(c, beam_gemmrc_splitk(da.p, db.p, dc.p, M, N, K, BEAM_F16, &cfg, s, dw.p, (size_t)eff * M * N * 4, nullptr));
+    if (dc.download16() != first) c.fail("split_k = " + std::to_string(s) + ": a workspace without flags gives other bits");
+    int timed_out = 1;
+    BEAM_REQUIRE(c, beam_gemmrc_splitk_timed_out(dw.p, M, N, eff, nullptr, &timed_out));
+    if (timed_out) c.fail("split_k = " + std::to_string(s) + ": time-out reported");
   }
   return c;
 }
