@@ -252,7 +252,7 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, un
 // vector instruction that overwrites them must not follow at once.  The compiler keeps that distance for stores it
 // emits itself; it does not look into assembly text.)
 __device__ __forceinline__ void store_through_16(void* dst, i32x4 v) {
-  asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" ::"v"(dst), "v"(v) : "memory");
+  asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 2" ::"v"(dst), "v"(v) : "memory");
 }
 
 // s_waitcnt vmcnt(N) lgkmcnt(0): at most N of this wavefront's buffer loads still in flight,
