@@ -1,6 +1,7 @@
 """A captured sequence of operators replays as a HIP graph with the eager results.
 
-The graph holds gemmrc, split-K (one launch: multiplying and reducing workgroups in one grid), GEMM+SiLU, the [K][N] matmul, a K = 0 call (its clear is a
+The graph holds gemmrc, split-K (one launch: multiplying and reducing workgroups in one grid; with a caller's
+workspace and with the library's built-in one), GEMM+SiLU, the [K][N] matmul, a K = 0 call (its clear is a
 kernel, not a memset node), a two-pass GEMM+LayerNorm (what BEAM_LN_AUTO turns into under capture) and an
 explicitly fused one (its workspace keeps its launch count on the device, so replays and the eager calls in
 between simply take turns on it).
@@ -29,7 +30,7 @@ def test_graph_replay_matches_eager(gpu, beamc):
     a, b, bkn, x = (beamc.DeviceArray(s, F16) for s in ((M, K), (N, K), (K, N), (n,)))
     g = beamc.DeviceArray.from_numpy(beamc.host_normal((N,), F16, 99, 1000, 1.0, 0.1), F16)
     bt = beamc.DeviceArray.from_numpy(beamc.host_normal((N,), F16, 99, 1001, 0.0, 0.1), F16)
-    outs = {k: beamc.DeviceArray((M, N), F16) for k in ("gemm", "splitk", "pair", "nn", "k0", "ln", "lnf")}
+    outs = {k: beamc.DeviceArray((M, N), F16) for k in ("gemm", "splitk", "splitk_na", "pair", "nn", "k0", "ln", "lnf")}
     y = beamc.DeviceArray((n,), F16)
     cfg = beamc.TileConfig(64, 64, 32, 32, 0, 0).to_c()
     s_eff = L.beam_splitk_effective(M, N, K, ctypes.byref(cfg), 4)
@@ -45,6 +46,8 @@ def test_graph_replay_matches_eager(gpu, beamc):
     def sequence(stream):
         chk(L.beam_gemmrc(a.ptr, b.ptr, outs["gemm"].ptr, M, N, K, F16, None, stream))
         chk(L.beam_gemmrc_splitk(a.ptr, b.ptr, outs["splitk"].ptr, M, N, K, F16, ctypes.byref(cfg), 4, ws_sk.ptr, ws_sk.nbytes, stream))
+        # (the entry point made for code under capture: its workspace is the library's own device array)
+        chk(L.beam_gemmrc_splitk_noalloc(a.ptr, b.ptr, outs["splitk_na"].ptr, M, N, K, F16, ctypes.byref(cfg), 8, stream))
         chk(L.beam_parallel_gemmrc_silu(a.ptr, b.ptr, outs["pair"].ptr, M, N, K, x.ptr, y.ptr, n, F16, None, stream))
         chk(L.beam_matmul_nn(a.ptr, bkn.ptr, outs["nn"].ptr, M, N, K, F16, None, stream))
         chk(L.beam_gemmrc(a.ptr, b.ptr, outs["k0"].ptr, M, N, 0, F16, None, stream))
