@@ -56,7 +56,7 @@ Device g_dev;
 std::mutex g_dev_mu;
 // polls of statistics slots (about a microsecond each) before a thread of a fused LayerNorm workgroup gives up
 std::atomic<int> g_ln_spin_limit{4 << 20};
-// Nonces of fused GEMM+LayerNorm launches: consecutive numbers from a start that differs from process to process
+// Nonces of fused GEMM+LayerNorm and one-launch split-K launches: consecutive numbers from a start that differs from process to process
 // (memory recycled from another process of this library then holds tags of another sequence).
 std::atomic<unsigned> g_ln_nonce{(unsigned)std::chrono::steady_clock::now().time_since_epoch().count() * 2654435761u ^
                                  (unsigned)getpid() * 40503u};

@@ -108,11 +108,11 @@ struct GemmParams {
   float* next_stats;    // kEpiLnFused: 8-byte words [tiles_m][tiles_n][BM] = (M2, ~tag)
   // kEpiLnFused: the workspace header (tile_map.h: kLnHdr*); never has to be initialised
   int* timeout_flag;
-  unsigned ln_nonce;    // kEpiLnFused: a number no earlier launch of this process had (see ln_launch_tag)
+  unsigned ln_nonce;    // kEpiLnFused, kEpiPartialFused: a number no earlier launch of this process had (ln_launch_tag, sk_launch_tag)
   const void* gamma;    // 16-bit [N]                                                   (kEpiLnFused)
   const void* beta;     // 16-bit [N]
   float eps;
-  int spin_limit;       // polls of one statistics slot before giving up
+  int spin_limit;       // polls (of statistics slots / of a tile's flags) before a waiting thread gives up
   int M, N, K;
   int tiles_m, tiles_n;
   int k_slice;   // K elements per split-K slice, a multiple of kBK
