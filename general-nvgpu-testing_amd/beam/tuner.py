@@ -267,7 +267,8 @@ class OperatorTuner:
 def _main(argv: Sequence[str]) -> int:
     import argparse
     ap = argparse.ArgumentParser(prog="python -m beam.tuner", description="tune gemmrc shapes and print winner against default")
-    ap.add_argument("shapes", nargs="+", help="M,N,K")
+    ap.add_argument("shapes", nargs="*", help="M,N,K (default: the headline cube, then the shape sweep: squares 512 ... "
+                    "4096, the two LLM shapes and the ragged 3000,5000,2000; 16384,16384,16384 only when named)")
     ap.add_argument("--dtype", default="fp16", choices=["fp16", "bf16", "both"])
     ap.add_argument("--cache", default=None)
     ap.add_argument("--rep", type=int, default=20)
@@ -278,7 +279,9 @@ def _main(argv: Sequence[str]) -> int:
     print(f"{len(tuner.gemm_ops)} candidates")
     print("| shape | dtype | tuned operator | tuned TFLOP/s | default tile | default TFLOP/s | tuned / default |")
     print("|---|---|---|---|---|---|---|")
-    for text in args.shapes:
+    sweep = ["8192,8192,8192", "512,512,512", "1024,1024,1024", "2048,2048,2048", "4096,4096,4096", "4096,11008,4096",
+             "4096,4096,11008", "3000,5000,2000"]
+    for text in (args.shapes or sweep):
         M, N, K = (int(x) for x in text.split(","))
         for dtype in (("fp16", "bf16") if args.dtype == "both" else (args.dtype,)):
             op, tf = tuner.tune((M, N, K), dtype=dtype, verbose=args.verbose)
