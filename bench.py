@@ -212,9 +212,10 @@ def extra_ln(_C):
     g = _C.DeviceArray.from_numpy(_C.host_normal((N,), _C.F16, 22, 2, 1.0, 0.1))
     bt = _C.DeviceArray.from_numpy(_C.host_normal((N,), _C.F16, 22, 3, 0.0, 0.1))
     c = _C.DeviceArray((M, N))
-    for _ in range(2):  # the second round is past the clock transient of a cold start
-        plain = _C.bench(0, a, b, c, warmup=50, iters=100)
-        fused = _C.bench(2, a, b, c, gamma=g, beta=bt, warmup=50, iters=100)
+    # settled figures, the two in turn, twice: the second pair is what is reported
+    for _ in range(2):
+        plain = settled_ms(lambda w, n: _C.bench(0, a, b, c, warmup=w, iters=n))
+        fused = settled_ms(lambda w, n: _C.bench(2, a, b, c, gamma=g, beta=bt, warmup=w, iters=n))
     for x in (a, b, g, bt, c):
         x.free()
     return {"shape": [M, N, K], "gemm_us": round(plain * 1e3, 1), "gemm_ln_us": round(fused * 1e3, 1),
@@ -231,9 +232,9 @@ def extra_silu(_C):
     x = _C.DeviceArray.from_numpy(_C.host_normal((M * N,), _C.F16, 33, 2, 0.0, 2.0))
     y = _C.DeviceArray((M * N,))
     for _ in range(2):
-        gemm = _C.bench(_C.OP_GEMM, a, b, c, warmup=50, iters=100)
-        silu = _C.bench(_C.OP_SILU, a, b, c, x=x, y=y, warmup=50, iters=100)
-        pair = _C.bench(_C.OP_GEMM_SILU, a, b, c, x=x, y=y, warmup=50, iters=100)
+        gemm = settled_ms(lambda w, n: _C.bench(_C.OP_GEMM, a, b, c, warmup=w, iters=n))
+        silu = settled_ms(lambda w, n: _C.bench(_C.OP_SILU, a, b, c, x=x, y=y, warmup=w, iters=n))
+        pair = settled_ms(lambda w, n: _C.bench(_C.OP_GEMM_SILU, a, b, c, x=x, y=y, warmup=w, iters=n))
     for t in (a, b, c, x, y):
         t.free()
     return {"shape": [M, N, K], "elements": M * N, "gemm_us": round(gemm * 1e3, 1), "silu_us": round(silu * 1e3, 1),
