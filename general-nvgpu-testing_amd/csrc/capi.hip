@@ -507,11 +507,27 @@ int beam_matmul_nn(const void* A, const void* B, void* C, int M, int N, int K, i
   }
   beam_tile_cfg c;
   const KernelSet* ks;
-  if ((rc = resolve_cfg(cfg, M, N, K, &c, &ks))) return rc;
+  if ((rc = resolve_cfg(cfg, M, N, K, &c, &ks, -1, true))) return rc;
   if (!cfg && c.pipeline == 2) c.pipeline = 0;
   if (c.pipeline == 2) return fail(BEAM_ERR_UNSUPPORTED, "the [K][N] layout runs with pipeline 0 or 1");
+  // The 4-wavefront kernel, as in beam_gemmrc; the K tile's offset into B is a 32-bit scalar there.
+  const bool w4_fits = c.pipeline == 0 && K % kBK == 0 && K >= kW4MinK && ((uintptr_t)C & 15) == 0 && N <= (1 << 21) &&
+                       (size_t)K * N * 2 < ((size_t)1 << 31);
+  const bool w4_named = c.block_m == 256 && c.block_n == 256 && c.wave_m == 128 && c.wave_n == 128;
+  if (w4_named && !w4_fits && !cfg) {
+    c.wave_m = 128;
+    c.wave_n = 64;
+    if ((rc = resolve_cfg(&c, M, N, K, &c, &ks))) return rc;
+  }
   GemmParams p = base_params(A, B, M, N, K, c);
   p.C = C;
+  if (w4_fits && w4_named) {
+    const long tiles = (long)p.tiles_m * p.tiles_n;
+    const int cus = g_dev.cus > 0 ? g_dev.cus : 256;
+    p.c_streaming = (size_t)M * N * 2 >= ((size_t)256 << 20) && K >= 1024;
+    BEAM_HIP(launch_gemm_w4_kmajor(p, dtype, dim3((unsigned)(tiles < cus ? tiles : cus), 1, 1), st));
+    return BEAM_OK;
+  }
   BEAM_HIP(ks->launch_kmajor[dtype][c.pipeline](p, dim3((unsigned)(p.tiles_m * p.tiles_n), 1, 1), st));
   return BEAM_OK;
 }
@@ -1215,6 +1231,10 @@ int beam_dbg_band_xcd_grid(int tiles_m, int tiles_n, int bx) { return band_xcd_g
 int beam_dbg_lds_offset(int row, int chunk) { return lds_offset(row, chunk); }
 
 int beam_dbg_kmajor_lds_offset(int k, int n, int block_n) { return kmajor_lds_offset(k, n, block_n); }
+
+int beam_dbg_w4_kmajor_swizzle(int k) { return w4_kmajor_swizzle(k); }
+
+int beam_dbg_w4_kmajor_read_offset(int wn, int b, int g, int e, int q) { return w4_kmajor_read_offset(wn, b, g, e, q); }
 
 int beam_dbg_band_block_tile(int wg, int tiles_m, int tiles_n, int gb, int gc, int* tm, int* tn) {
   if (tiles_m < 1 || tiles_n < 1 || gb < 1 || gc < 1 || wg < 0 || wg >= band_block_grid(tiles_m, gb, gc) || !tm || !tn)

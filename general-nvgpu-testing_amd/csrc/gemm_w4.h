@@ -28,8 +28,16 @@
 //     columns per pair of blocks and stores them as one 16-byte access (64 contiguous bytes per
 //     output row and instruction).  The B slots use a swizzle made for that row pattern.
 //
+//   * B stored [K][N] (B_KMAJOR, the layout of matmul(a, b)): a B tile lies in its slot as it lies in
+//     memory, 64 rows of k by 256 columns, and a fragment is two transposing 8-byte reads
+//     (ds_read_b64_tr_b16) in place of one 16-byte read.  In a transposing read four lanes supply the
+//     addresses of the four columns groups of a 16-column block, so the same permuted column order costs
+//     nothing; to keep those reads free of bank conflicts the two blocks of a pair swap their halves of a
+//     lane's 8 columns in the odd lane groups, which the store undoes with four selects (w4_kmajor_*).
+//
 // Preconditions (the host checks them; anything else takes the kernels of gemm_kernel.h):
-// K a multiple of 64 and at least 192, N a multiple of 8, C 16-byte aligned, grid <= number of tiles.
+// K a multiple of 64 and at least 192, N a multiple of 8, C 16-byte aligned, grid <= number of tiles;
+// B_KMAJOR: K * N * 2 below 2^31 (the K tile's byte offset into B is a 32-bit scalar).
 #pragma once
 
 #include "gemm_kernel.h"
@@ -118,6 +126,8 @@ __host__ __device__ inline int w4_swizzle_b(int row) { return (((row >> 3) & 3) 
 // First B row (inside the wavefront's 128) of MFMA block b, and the row of lane-row r in it.
 __host__ __device__ inline int w4_b_row(int b, int r) { return 32 * (b >> 1) + 4 * (b & 1) + 8 * (r >> 2) + (r & 3); }
 
+// (B as [K][N]: the slot layout and the transposing reads' addresses are w4_kmajor_* in tile_map.h.)
+
 // SB, SA: a wavefront issues its 8 loads of the next B tile in gaps 0, SB, 2 SB, ... of step A and its 8
 // loads of the A tile after next in gaps 0, SA, ... of step B.  The path from the vector-memory unit into
 // LDS moves 64 bytes per cycle and CU, i.e. one 1 KiB load per 64 cycles (4 MFMAs) and wavefront when all
@@ -127,8 +137,10 @@ __host__ __device__ inline int w4_b_row(int b, int r) { return 32 * (b >> 1) + 4
 // LN: the fused GEMM+LayerNorm of gemm_kernel.h (kEpiLnFused) with this K loop: one output tile per
 // workgroup in the band order of tile_map.h, and after the K loop the same exchange of per-row (mean, M2)
 // pairs between the column tiles of a row band, normalisation in registers, Y stored once.
-template <typename T, bool C_NT = false, bool LN = false, int SB = 4, int SA = 8, int G0 = 2>
+// B_KMAJOR: B is stored [K][N].
+template <typename T, bool C_NT = false, bool LN = false, int SB = 4, int SA = 8, int G0 = 2, bool B_KMAJOR = false>
 struct GemmW4 {
+  static_assert(!(LN && B_KMAJOR), "the fused LayerNorm is built for B as [N][K]");
   using Traits = ElemTraits<T>;
   using vec8 = typename Traits::vec8;
   using Mfma = W4Mfma<T>;
@@ -142,8 +154,9 @@ struct GemmW4 {
   static constexpr int LDS_BYTES = (AST + BST) * SLOT;
   static constexpr int LPT = SLOT / (NW * 1024);  // buffer loads per wavefront per operand tile (8)
   static_assert(LDS_BYTES == 160 * 1024 && LPT == 8, "LDS budget");
-  // What goes into gap m (after MFMA m) of a step: load number k, or fragment read number n (B 0..7, then
-  // A 0..7; they take the gaps the loads leave free, in order), or nothing (-1).
+  static constexpr int B_READS = B_KMAJOR ? 2 * FN : FN;  // LDS reads that make the B fragments of a step
+  // What goes into gap m (after MFMA m) of a step: load number k, or fragment read number n (B 0..B_READS-1,
+  // then A 0..7; they take the gaps the loads leave free, in order), or nothing (-1).
   // G0: gaps 0 .. G0 - 1 of step A hold nothing but, in the last of them, the wait and the barrier
   static constexpr int load_at(int half, int m) {
     const int s = half == 0 ? SB : SA;
@@ -153,7 +166,7 @@ struct GemmW4 {
     if (m < G0 || load_at(half, m) >= 0) return -1;
     int n = 0;
     for (int x = G0; x < m; ++x) n += load_at(half, x) < 0;
-    return n < FN + FM ? n : -1;
+    return n < B_READS + FM ? n : -1;
   }
   static constexpr int LAST_B = G0 + (LPT - 1) * SB, LAST_A = G0 + (LPT - 1) * SA;  // gaps of a step's last load
   static constexpr int last_read(int half) {
@@ -188,15 +201,21 @@ struct GemmW4 {
     // Load i of wavefront w fills bytes [(4 i + w) KiB, + 1 KiB) of a slot = rows 32 i + 8 w .. + 8;
     // lane l writes position l % 8 of row 32 i + 8 w + l / 8 and fetches the chunk that belongs there.
     // (Neither swizzle depends on i.)  The row goes into the per-lane offset, the K tile into the scalar
-    // offset: the hardware checks only the former against the descriptor, and that check is what keeps
-    // rows past the end of a matrix from touching memory.
+    // offset: the hardware checks their sum against the descriptor's size, and a row past the end of a
+    // matrix is past it by its per-lane part alone: that check is what keeps such rows from touching memory.
     const int fill_row = 8 * wave + (lane >> 3);
     unsigned voff_a[LPT], voff_b[LPT];
 #pragma unroll
     for (int i = 0; i < LPT; ++i) {
       const unsigned row_bytes = (unsigned)(fill_row + 32 * i) * (unsigned)K * 2u;
       voff_a[i] = row_bytes + (unsigned)(((lane & 7) ^ swizzle_of_row(fill_row)) << 4);
-      voff_b[i] = row_bytes + (unsigned)(((lane & 7) ^ w4_swizzle_b(fill_row)) << 4);
+      if constexpr (B_KMAJOR) {
+        // 1 KiB = rows k, k + 1 of the [K][N] tile, k = 8 i + 2 w; lane l fills position l % 32 of row k + l / 32
+        const int k = 8 * i + 2 * wave + (lane >> 5);
+        voff_b[i] = ((unsigned)k * (unsigned)N + (unsigned)(((lane & 31) ^ w4_kmajor_swizzle(k)) << 3)) * 2u;
+      } else {
+        voff_b[i] = row_bytes + (unsigned)(((lane & 7) ^ w4_swizzle_b(fill_row)) << 4);
+      }
     }
 
     // Operand rows of the workgroup's j-th output tile as (address, bytes) of a buffer descriptor; empty
@@ -215,6 +234,10 @@ struct GemmW4 {
       if (j >= my_tiles) return make_rsrc(p.B, 0u);
       const int col0 = tc.tn * BN;
       const int rows = (N - col0) < BN ? (N - col0) : BN;
+      // [K][N]: the tile's columns of all K rows (the range check counts the scalar offset, which holds the K
+      // tile here, together with the per-lane one).  Columns past the tile's last one read the next row's data,
+      // past the last row's end nothing: they only feed output columns that do not exist.
+      if constexpr (B_KMAJOR) return make_rsrc((const T*)p.B + col0, ((unsigned)(K - 1) * (unsigned)N + (unsigned)rows) * 2u);
       return make_rsrc((const T*)p.B + (size_t)col0 * K, (unsigned)rows * (unsigned)K * 2u);
     };
     // A load stream: the operand rows of the output tile it is at (a finished buffer descriptor), the K
@@ -227,7 +250,9 @@ struct GemmW4 {
       int koff;
       int lds;
     };
-    const int k_bytes = K * 2;
+    // bytes from one K tile to the next and to the end of K, per operand
+    const int a_step = kBK * 2, a_end = K * 2;
+    const int b_step = B_KMAJOR ? kBK * N * 2 : kBK * 2, b_end = B_KMAJOR ? K * N * 2 : K * 2;
     // The LDS address of an LDS-direct load comes from M0.  The compiler's own sequence for the builtin
     // is "write M0, one wait state, load" in one place; here M0 is written one gap ahead of the load, so
     // the MFMA between them is the wait state and no gap holds more than one scalar and one memory
@@ -241,14 +266,14 @@ struct GemmW4 {
     };
     // (in `part`s of two or three scalar instructions, one part per gap; part < 0: all of them)
     bool wrap_a = false, wrap_b = false;
-    auto advance = [&](Stream& st, bool& wrap, __amdgpu_buffer_rsrc_t next, int ring_begin, int ring_end, int part) __attribute__((always_inline)) {
+    auto advance = [&](Stream& st, bool& wrap, __amdgpu_buffer_rsrc_t next, int ring_begin, int ring_end, int k_step, int k_end, int part) __attribute__((always_inline)) {
       if (part == 0 || part < 0) {
         const int lds = st.lds + SLOT;
         st.lds = lds == ring_end + wave * 1024 ? ring_begin + wave * 1024 : lds;
       }
       if (part == 1 || part < 0) {
-        const int k = st.koff + kBK * 2;
-        wrap = k == k_bytes;
+        const int k = st.koff + k_step;
+        wrap = k == k_end;
         st.koff = wrap ? 0 : k;
       }
       if (part == 2 || part < 0) st.rows = wrap ? next : st.rows;
@@ -263,6 +288,20 @@ struct GemmW4 {
       const int brow = wn * 128 + w4_b_row(0, r);
       b_off[kk] = brow * kRowBytes + (((4 * kk + g) ^ w4_swizzle_b(brow)) << 4);
     }
+    // [K][N]: where this lane points in a transposing read of block b = 2 pair + parity (first read, first half)
+    int bt_off[2][FN / 2];
+    if constexpr (B_KMAJOR) {
+#pragma unroll
+      for (int par = 0; par < 2; ++par)
+#pragma unroll
+        for (int pair = 0; pair < FN / 2; ++pair) bt_off[par][pair] = w4_kmajor_read_offset(wn, 2 * pair + par, g, (lane >> 2) & 3, lane & 3);
+    }
+    auto read_b_transposed = [&](const char* sb, int half, int n) __attribute__((always_inline)) {
+      // read n of a step: rows +0 (n even) or +4 (n odd) of block n / 2, in the K tile's half `half`
+      typedef short i16x4 __attribute__((ext_vector_type(4)));
+      const char* at = sb + bt_off[(n >> 1) & 1][n >> 2] + half * (32 * 512) + (n & 1) * (4 * 512);
+      return __builtin_bit_cast(i32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) i16x4*)at));
+    };
 
     w4_claim_acc_registers();  // block (i, b) of the wavefront tile is accumulator block 8 i + b
     // Fragments, double buffered: set 0 holds the first 32 K elements of a tile, set 1 the second.
@@ -326,10 +365,15 @@ struct GemmW4 {
       v[5] = (T)w4_acc_read<R0 + 5>();
       v[6] = (T)w4_acc_read<R0 + 6>();
       v[7] = (T)w4_acc_read<R0 + 7>();
+      i32x4 w = __builtin_bit_cast(i32x4, v);
+      if constexpr (B_KMAJOR) {  // odd lane groups hold the two blocks' columns the other way round
+        const i32x4 s = {w[2], w[3], w[0], w[1]};
+        w = (g & 1) ? s : w;
+      }
       const int skip = i * 16 * N * 2;  // bytes of the row blocks above this one
       const int left = out.bytes - skip;
       const __amdgpu_buffer_rsrc_t rsrc = make_rsrc(out.base + skip, left > 0 ? (unsigned)left : 0u);
-      __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(i32x4, v), rsrc, (int)out.voff[q], 0, AUX);
+      __builtin_amdgcn_raw_buffer_store_b128(w, rsrc, (int)out.voff[q], 0, AUX);
     };
 
     // ---- one K tile ------------------------------------------------------------------------------
@@ -374,21 +418,30 @@ struct GemmW4 {
         if constexpr (ld >= 0) {
           if constexpr (half == 0) load_tile_part(ld_b, voff_b[ld]);
           else load_tile_part(ld_a, voff_a[ld]);
-        } else if constexpr (rd >= 0 && rd < FN) {
-          const vec8 v = *(const vec8*)(sb + b_off[half] + (rd >> 1) * 4096 + (rd & 1) * 512);
-          if constexpr (half == 0) fb0[rd] = v;
-          else fb1[rd] = v;
-        } else if constexpr (rd >= FN) {
-          const vec8 v = *(const vec8*)(sa + a_off[half] + (rd - FN) * 2048);
-          if constexpr (half == 0) fa0[rd - FN] = v;
-          else fa1[rd - FN] = v;
+        } else if constexpr (rd >= 0 && rd < B_READS) {
+          if constexpr (B_KMAJOR) {
+            const i32x2 v = read_b_transposed(sb, half, rd);  // K elements 0..3 (even read) or 4..7 of the lane's 8
+            vec8& f = half == 0 ? fb0[rd >> 1] : fb1[rd >> 1];
+            i32x4 w = __builtin_bit_cast(i32x4, f);
+            w[2 * (rd & 1)] = v[0];
+            w[2 * (rd & 1) + 1] = v[1];
+            f = __builtin_bit_cast(vec8, w);
+          } else {
+            const vec8 v = *(const vec8*)(sb + b_off[half] + (rd >> 1) * 4096 + (rd & 1) * 512);
+            if constexpr (half == 0) fb0[rd] = v;
+            else fb1[rd] = v;
+          }
+        } else if constexpr (rd >= B_READS) {
+          const vec8 v = *(const vec8*)(sa + a_off[half] + (rd - B_READS) * 2048);
+          if constexpr (half == 0) fa0[rd - B_READS] = v;
+          else fa1[rd - B_READS] = v;
         }
         // scalar bookkeeping, a few instructions per gap: the B stream moves on after its last load, ...
-        if constexpr (half == 0 && m > LAST_B && m <= LAST_B + 3) advance(ld_b, wrap_b, next_b, B_REGION, LDS_BYTES, m - LAST_B - 1);
+        if constexpr (half == 0 && m > LAST_B && m <= LAST_B + 3) advance(ld_b, wrap_b, next_b, B_REGION, LDS_BYTES, b_step, b_end, m - LAST_B - 1);
         // ... the read slots once the last fragment read of the K tile is out, the A stream after its last load
         if constexpr (half == 1 && m == LAST_READ + 1) rd_a = rd_a + SLOT == B_REGION ? 0 : rd_a + SLOT;
         if constexpr (half == 1 && m == LAST_READ + 2) rd_b = rd_b + SLOT == LDS_BYTES ? B_REGION : rd_b + SLOT;
-        if constexpr (half == 1 && m > LAST_A && m <= LAST_A + 3) advance(ld_a, wrap_a, next_a, 0, B_REGION, m - LAST_A - 1);
+        if constexpr (half == 1 && m > LAST_A && m <= LAST_A + 3) advance(ld_a, wrap_a, next_a, 0, B_REGION, a_step, a_end, m - LAST_A - 1);
         if constexpr (FIRST && !LN && gap >= 10 && gap < 10 + 8 * FM && ((gap - 10) & 1) == 0) {
           // pair q of row block i goes into gap 10 + 8 i + 2 q
           store_pair(std::integral_constant<int, (gap - 10) / 8>{}, std::integral_constant<int, ((gap - 10) / 2) % 4>{}, std::false_type{});
@@ -414,10 +467,10 @@ struct GemmW4 {
       };
       load_whole_tile(ld_a, voff_a);
       load_whole_tile(ld_b, voff_b);
-      advance(ld_a, wrap_a, next_a, 0, B_REGION, -1);
-      advance(ld_b, wrap_b, next_b, B_REGION, LDS_BYTES, -1);
+      advance(ld_a, wrap_a, next_a, 0, B_REGION, a_step, a_end, -1);
+      advance(ld_b, wrap_b, next_b, B_REGION, LDS_BYTES, b_step, b_end, -1);
       load_whole_tile(ld_a, voff_a);
-      advance(ld_a, wrap_a, next_a, 0, B_REGION, -1);
+      advance(ld_a, wrap_a, next_a, 0, B_REGION, a_step, a_end, -1);
 
       for (int j = 0; j < my_tiles; ++j) {
         // The streams move on to tile j + 1 while tile j is multiplied: A in its last but one K tile,
@@ -595,10 +648,10 @@ struct GemmW4 {
   }
 };
 
-template <typename T, bool C_NT = false, bool LN = false, int SB = 4, int SA = 8, int G0 = 2>
+template <typename T, bool C_NT = false, bool LN = false, int SB = 4, int SA = 8, int G0 = 2, bool B_KMAJOR = false>
 __global__ void __launch_bounds__(256) gemmrc_w4_kernel(const GemmParams p) {
   extern __shared__ __attribute__((aligned(1024))) char smem[];
-  GemmW4<T, C_NT, LN, SB, SA, G0>::run(p, smem);
+  GemmW4<T, C_NT, LN, SB, SA, G0, B_KMAJOR>::run(p, smem);
 }
 
 }  // namespace beam

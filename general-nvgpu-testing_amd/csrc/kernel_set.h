@@ -131,6 +131,8 @@ BEAM_FOR_EACH_SET(BEAM_DECLARE_SET)
 // grid <= tiles_m * tiles_n; kW4MinK names the K bound.
 constexpr int kW4MinK = 192;
 hipError_t launch_gemm_w4(const GemmParams& p, int dtype, dim3 grid, hipStream_t stream);
+// The same with B stored [K][N]; additionally K * N * 2 < 2^31.
+hipError_t launch_gemm_w4_kmajor(const GemmParams& p, int dtype, dim3 grid, hipStream_t stream);
 // Its fused GEMM+LayerNorm form: one workgroup per tile, grid and parameters as for the kEpiLnFused kernels;
 // gamma and beta 16-byte aligned as well.
 hipError_t launch_gemm_w4_ln(const GemmParams& p, int dtype, dim3 grid, hipStream_t stream);

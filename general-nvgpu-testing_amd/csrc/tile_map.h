@@ -49,6 +49,19 @@ BEAM_HD int kmajor_lds_offset(int k, int n, int block_n) {
   return k * block_n * 2 + ((((n >> 3) ^ kmajor_swizzle(k, block_n))) << 4) + ((n & 7) << 1);
 }
 
+// The 4-wavefront kernel (gemm_w4.h) with B as [K][N]: XOR pattern of the 16-byte chunks of a k row (512 bytes)
+// in LDS.  A transposing read of block b has, per 32 lanes, lane 4 e + q of group g (g = 0, 1) at row 8 g + e, chunk 4 (b / 2) + q, 8-byte half
+// (b ^ q) % 2: bits 0, 2 and 3 of the code spread the 8 rows, q's bit 1 and the half do the rest, 32 distinct
+// 8-byte bank pairs.  (Bits 2 and 5 of k stay out of it: the second read of a fragment, 4 rows on, and the
+// second half of a K tile, 32 rows on, are constant offsets from the first.)
+BEAM_HD int w4_kmajor_swizzle(int k) { return (k & 1) | (((k >> 1) & 1) << 2) | (((k >> 3) & 1) << 3); }
+// Byte offset in a [K][N] slot of the 8 bytes that lane (g, e, q) of a transposing read of block b supplies
+// (wn: the wavefront's half of the tile's columns; first read of the first half of the K tile).
+BEAM_HD int w4_kmajor_read_offset(int wn, int b, int g, int e, int q) {
+  const int k = 8 * g + e;
+  return k * 512 + (((16 * wn + 4 * (b >> 1) + q) ^ w4_kmajor_swizzle(k)) << 4) + (((b ^ q) & 1) << 3);
+}
+
 // Words of the fused GEMM+LayerNorm workspace header (256 bytes in front of the two arrays of statistics
 // words).  Nothing in it has to be initialised: every fused launch carries a tag that no earlier launch had,
 // a statistics word counts as published only if it carries that tag, and the header words say which launch

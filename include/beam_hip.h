@@ -322,6 +322,11 @@ int beam_dbg_lds_offset(int row, int chunk);
 /* Byte offset of element (k, n), n a multiple of 4, inside a K-major LDS stage of block_n columns
  * (B stored [K][N], beam_matmul_nn). */
 int beam_dbg_kmajor_lds_offset(int k, int n, int block_n);
+/* The 4-wavefront kernel with B stored [K][N] (256 columns, 512 bytes per row of k in an LDS slot): the XOR code of
+ * the 16-byte chunks of row k, and the byte offset of the 8 bytes that lane 16 g + 4 e + q supplies to the first
+ * transposing read of 16-column block b (0..7) of the wavefront's column half wn (0, 1). */
+int beam_dbg_w4_kmajor_swizzle(int k);
+int beam_dbg_w4_kmajor_read_offset(int wn, int b, int g, int e, int q);
 /* Workgroup id -> tile of the padded band-block grid used by the fused GEMM+LayerNorm (tm = -1:
  * the id is padding), and the size of that grid. */
 int beam_dbg_band_block_tile(int wg, int tiles_m, int tiles_n, int gb, int gc, int* tm, int* tn);

@@ -101,6 +101,34 @@ def test_full_size_equals_gemmrc_on_transpose(gpu, beamc, oracle):
     check(oracle, got[rows], ref, K, F16, "sampled rows")
 
 
+@pytest.mark.parametrize("dtype", [F16, BF16])
+@pytest.mark.parametrize("shape", [(4352, 4360, 192), (3000, 5000, 2048), (257, 264, 448), (8192, 520, 1024), (512, 256, 4096)])
+def test_four_wavefront_kernel(gpu, beamc, oracle, shape, dtype):
+    """The 256 x 256 tile of four 128 x 128 wavefronts with B as [K][N]: more tiles than CUs (a workgroup walks
+    several, its operand ring running through the tile boundaries), edge tiles in M and N, the shortest K the
+    kernel takes and a long one.  Bit-identical to gemmrc on B^T with the same tile, and sampled rows against the
+    oracle."""
+    M, N, K = shape
+    cfg = beamc.TileConfig(256, 256, 128, 128, 0, 0)
+    a = beamc.host_uniform((M, K), dtype, 11, 0)
+    b = beamc.host_uniform((K, N), dtype, 11, 1)
+    got = run_nn(beamc, a, b, dtype, cfg)
+    assert (got == run_rc(beamc, a, np.ascontiguousarray(b.T), dtype, cfg)).all()
+    rows = np.unique(np.concatenate([np.arange(0, M, 37), np.arange(max(0, M - 3), M)]))[:160]
+    check(oracle, got[rows], oracle.matmul_nn(a[rows], b, dtype), K, dtype, f"{cfg.name} {shape}")
+
+
+def test_four_wavefront_kernel_streaming_stores(gpu, beamc, oracle):
+    """An output beyond the last-level cache (12288 x 12288: 302 MB) takes the form with non-temporal stores."""
+    M, N, K = 12288, 12288, 1024
+    a = beamc.host_normal((M, K), F16, 13, 0, 0.0, K ** -0.5)
+    b = beamc.host_normal((K, N), F16, 13, 1, 0.0, K ** -0.5)
+    got = run_nn(beamc, a, b, F16)
+    assert (got == run_rc(beamc, a, np.ascontiguousarray(b.T), F16)).all()
+    rows = np.arange(0, M, 131)[:96]
+    check(oracle, got[rows], oracle.matmul_nn(a[rows], b, F16), K, F16, "sampled rows")
+
+
 def test_error_paths(gpu, beamc):
     a = beamc.DeviceArray((64, 64), F16)
     b = beamc.DeviceArray((64, 36), F16)

@@ -127,6 +127,57 @@ def test_kmajor_lds_layout_is_bijective_and_conflict_free(beamc):
                     assert sorted(banks) == list(range(64)), (bn, n0, kbase, half)
 
 
+def test_w4_kmajor_fragments_and_banks(beamc):
+    """The 4-wavefront kernel with B stored [K][N].  Fill: load i of wavefront w puts 1 KiB at byte (4 i + w) KiB of
+    the slot, lane l at 16 l inside it, and fetches the chunk (l % 32) ^ code(k) of row k = 8 i + 2 w + l / 32.  Read:
+    in a group of 16 lanes, lane 4 e + q supplies the address of 8 bytes, and lane i of the group receives element
+    i % 4 of the data of lanes i / 4, 4 + i / 4, 8 + i / 4, 12 + i / 4.  Together: lane (r, g) of block b must end up
+    with K elements 8 g .. 8 g + 7 of the K step at the column the store assumes for it, every pass of 32 lanes
+    must touch each bank once, and the k + 4 / k + 32 reads must be the constant offsets the kernel adds."""
+    L = beamc.lib
+    lds = {}                                    # byte offset of a 16-byte position -> (k, first column)
+    for i in range(8):
+        for w in range(4):
+            for l in range(64):
+                k = 8 * i + 2 * w + l // 32
+                lds[(4 * i + w) * 1024 + 16 * l] = (k, 8 * ((l % 32) ^ L.beam_dbg_w4_kmajor_swizzle(k)))
+    assert sorted(lds) == list(range(0, 32768, 16))
+    for k in range(64):
+        assert sorted(c for (kk, c) in (lds[k * 512 + 16 * pos] for pos in range(32))) == list(range(0, 256, 8))
+        assert all(lds[k * 512 + 16 * pos][0] == k for pos in range(32))
+
+    def element(off):                            # (k, n) of the 2-byte element at byte offset off
+        k, c = lds[off & ~15]
+        return k, c + (off & 15) // 2
+
+    for wn in range(2):
+        for b in range(8):
+            for kstep in (0, 32 * 512):
+                for second in (0, 4 * 512):
+                    for g in range(4):
+                        src = [L.beam_dbg_w4_kmajor_read_offset(wn, b, g, j >> 2, j & 3) + kstep + second for j in range(16)]
+                        for i in range(16):
+                            got = [element(src[4 * t + (i >> 2)] + 2 * (i & 3)) for t in range(4)]
+                            n = 128 * wn + 32 * (b >> 1) + 8 * (i >> 2) + 4 * ((b ^ (i >> 2)) & 1) + (i & 3)
+                            k0 = 8 * g + kstep // 512 + second // 512
+                            assert got == [(k0 + t, n) for t in range(4)], (wn, b, g, i)
+                    for half in (0, 2):
+                        banks = []
+                        for g in (half, half + 1):
+                            for j in range(16):
+                                o = L.beam_dbg_w4_kmajor_read_offset(wn, b, g, j >> 2, j & 3) + kstep + second
+                                banks += [(o // 4) % 64, (o // 4 + 1) % 64]
+                        assert sorted(banks) == list(range(64)), (wn, b, half)
+    # the store: lane group g holds, for the pair of blocks (2 p, 2 p + 1), columns 32 p + 8 g + 0..7 of the
+    # wavefront's half -- the first four in the even block when g is even, in the odd block when g is odd
+    for p in range(4):
+        for g in range(4):
+            even = [32 * p + 8 * g + 4 * ((2 * p ^ g) & 1) + e for e in range(4)]
+            odd = [32 * p + 8 * g + 4 * (((2 * p + 1) ^ g) & 1) + e for e in range(4)]
+            lo, hi = (odd, even) if g & 1 else (even, odd)
+            assert lo + hi == list(range(32 * p + 8 * g, 32 * p + 8 * g + 8))
+
+
 def test_slice_heuristic_matches_reference_rule(beamc, oracle):
     for units in (108, 256):
         for tiles in range(1, units + 2):

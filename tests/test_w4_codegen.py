@@ -12,14 +12,19 @@ CSRC = os.path.join(ROOT, "general-nvgpu-testing_amd", "csrc")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
 
-def test_compiler_never_touches_the_accumulators(tmp_path):
+import pytest
+
+
+# fp16 and bf16: plain, streaming stores, fused LayerNorm; B as [K][N]: plain, streaming stores
+@pytest.mark.parametrize("source,count", [("gemm_inst_w4.hip", 6), ("gemm_inst_w4_kmajor.hip", 4)])
+def test_compiler_never_touches_the_accumulators(tmp_path, source, count):
     out = tmp_path / "w4.s"
     subprocess.run([HIPCC, "--offload-arch=gfx950", "-O3", "-std=c++17", "-Wno-unused-command-line-argument",
                     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-S", "--cuda-device-only",
-                    "-o", str(out), os.path.join(CSRC, "gemm_inst_w4.hip")], check=True, capture_output=True, timeout=600)
+                    "-o", str(out), os.path.join(CSRC, source)], check=True, capture_output=True, timeout=600)
     text = out.read_text()
     kernels = re.findall(r"^(_ZN4beam16gemmrc_w4_kernel\w+):", text, flags=re.M)
-    assert len(kernels) >= 6, kernels          # fp16 and bf16: plain, streaming stores, fused LayerNorm
+    assert len(kernels) >= count, kernels
     assert "v_mfma_f32_16x16x32" in text
     for bad in ("v_accvgpr_write", "v_accvgpr_mov", "scratch_load", "scratch_store"):
         assert bad not in text, f"the compiler emitted {bad} in a 4-wavefront kernel"
