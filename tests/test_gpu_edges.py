@@ -2,9 +2,7 @@
 multiple of 8, operands at addresses that are not 16-byte aligned -- are computed (by a plain kernel), never
 refused: every entry point against the oracle, to the same tolerances as everywhere else.  The reference's
 NN path masks any edge (python/beam/triton_kernels/gemm.py:62-63,75)."""
-import ctypes
 
-import numpy as np
 import pytest
 
 from test_gpu_gemm import F16, BF16, assert_close

@@ -6,7 +6,7 @@ import os
 import numpy as np
 import pytest
 
-from test_gpu_gemm import F16, BF16, run_gemm
+from test_gpu_gemm import BF16, run_gemm
 from test_gpu_ln import run_ln
 
 pytestmark = pytest.mark.gpu

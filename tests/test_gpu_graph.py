@@ -10,7 +10,6 @@ replay must reproduce, bit for bit, what the same calls give eagerly on the same
 """
 import ctypes
 
-import numpy as np
 import pytest
 
 pytestmark = pytest.mark.gpu

@@ -8,7 +8,6 @@ gives on a quiet device, bit for bit.
 import ctypes
 import threading
 
-import numpy as np
 import pytest
 
 pytestmark = pytest.mark.gpu

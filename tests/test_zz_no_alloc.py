@@ -3,7 +3,6 @@ against beam_gemmrc_splitk with a caller-owned workspace: same bits, on two call
 smaller problem (the built-in array keeps the first call's contents), and a clear error beyond its size."""
 import ctypes
 
-import numpy as np
 import pytest
 
 pytestmark = pytest.mark.gpu
