@@ -508,8 +508,21 @@ int beam_matmul_nn(const void* A, const void* B, void* C, int M, int N, int K, i
   beam_tile_cfg c;
   const KernelSet* ks;
   if ((rc = resolve_cfg(cfg, M, N, K, &c, &ks, -1, true))) return rc;
-  if (!cfg && c.pipeline == 2) c.pipeline = 0;
-  if (c.pipeline == 2) return fail(BEAM_ERR_UNSUPPORTED, "the [K][N] layout runs with pipeline 0 or 1");
+  if (!cfg) {
+    // The library's choice is priced for B as [N][K].  In this layout a B fragment is two LDS reads, and the tiles
+    // whose wavefronts are 64 columns wide pay for it: eight wavefronts of 64 x 32 instead of four of 64 x 64
+    // (768 x 3072 x 768: 8.3 against 12.7 us; 2048 x 2048 x 512: 7.9 against 10.0), and 128 x 64 tiles of 64 x 32
+    // instead of 64 x 128 tiles of 32 x 64 where that does not make more tiles (256 x 8192 x 8192: 57 against 71).
+    auto tiles_of = [&](int bm, int bn) { return (long)((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
+    beam_tile_cfg alt = c;
+    if (c.block_m == 128 && c.block_n == 128 && c.wave_m == 64 && c.wave_n == 64) {
+      alt.wave_n = 32;
+    } else if (c.block_m == 64 && c.block_n == 128 && c.wave_m == 32 && c.wave_n == 64 && tiles_of(128, 64) <= tiles_of(64, 128)) {
+      alt.block_m = 128, alt.block_n = 64, alt.wave_m = 64, alt.wave_n = 32;
+    }
+    const KernelSet* alt_ks = nullptr;
+    if ((alt.wave_n != c.wave_n) && resolve_cfg(&alt, M, N, K, &alt, &alt_ks) == BEAM_OK) c = alt, ks = alt_ks;
+  }
   // The 4-wavefront kernel, as in beam_gemmrc; the K tile's offset into B is a 32-bit scalar there.
   const bool w4_fits = c.pipeline == 0 && K % kBK == 0 && K >= kW4MinK && ((uintptr_t)C & 15) == 0 && N <= (1 << 21) &&
                        (size_t)K * N * 2 < ((size_t)1 << 31);

@@ -19,8 +19,8 @@ struct KernelSet {
   int lds_bytes_deep;
   // [dtype][epilogue][pipeline: 0 = 3 A + 2 B slots, 1 = 2 + 2, 2 = deep (store / partial only)]
   GemmLauncher launch[2][kNumEpilogues][3];
-  // B stored [K][N] instead of [N][K], kEpiStore only: [dtype][pipeline 0 or 1]
-  GemmLauncher launch_kmajor[2][2];
+  // B stored [K][N] instead of [N][K], kEpiStore only: [dtype][pipeline]
+  GemmLauncher launch_kmajor[2][3];
   // Split-K in one launch (kEpiPartialFused), tiles up to 128 x 128 only (what split-K problems run on):
   // [dtype][pipeline]; nullptr otherwise.
   GemmLauncher launch_partial_fused[2][3];
@@ -88,6 +88,7 @@ KernelSet make_kernel_set() {
   k.launch[D][kEpiStoreSide][2] = nullptr; \
   k.launch_kmajor[D][0] = launch_gemm<T, BM, BN, WVM, WVN, kEpiStore, 3, 2, true>; \
   k.launch_kmajor[D][1] = launch_gemm<T, BM, BN, WVM, WVN, kEpiStore, 2, 2, true>; \
+  k.launch_kmajor[D][2] = launch_gemm<T, BM, BN, WVM, WVN, kEpiStore, DA, DA - 1, true>; \
   k.launch[D][kEpiStoreLoop][0] = loop_launcher<T, BM, BN, WVM, WVN>();              \
   k.launch[D][kEpiStoreLoop][1] = nullptr;                                            \
   k.launch[D][kEpiStoreLoop][2] = nullptr;                                            \

@@ -218,8 +218,10 @@ int beam_silu(const void* X, void* Y, long long count, int dtype, void* stream);
  * (python/beam/triton_kernels/gemm.py:78-99, kernel :10-76), which torch.matmul callers use.  Same
  * arithmetic as beam_gemmrc (fp32 accumulation, one rounding to 16 bits); same tile space.  B tiles
  * are staged in LDS as they lie in memory and transposed on their way into registers
- * (ds_read_b64_tr_b16), so no transposed copy of B is made.  Requirements beyond beam_gemmrc's:
- * N % 8 == 0; cfg->pipeline 0 or 1. */
+ * (ds_read_b64_tr_b16), so no transposed copy of B is made.  N % 8 != 0 (rows of B that are not multiples of
+ * 16 bytes) runs on the plain kernel, like K % 8 != 0.  With cfg NULL the library starts from the tile it would
+ * take for beam_gemmrc and prefers wavefront tiles of 32 columns to those of 64 (a B fragment is two LDS reads
+ * in this layout). */
 int beam_matmul_nn(const void* A, const void* B, void* C, int M, int N, int K, int dtype, const beam_tile_cfg* cfg,
                    void* stream);
 

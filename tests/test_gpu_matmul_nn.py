@@ -57,7 +57,7 @@ def test_every_config_1024_cube(gpu, beamc, oracle):
     ref = oracle.matmul_nn(a, b, F16)
     bt = np.ascontiguousarray(b.T)
     for cfg in beamc.list_configs():
-        for pipe in (0, 1):
+        for pipe in (0, 1, 2):
             c = beamc.TileConfig(cfg.block_m, cfg.block_n, cfg.wave_m, cfg.wave_n, pipe, 0)
             got = run_nn(beamc, a, b, F16, c)
             check(oracle, got, ref, K, F16, c.name)
@@ -74,6 +74,18 @@ def test_ragged_shapes_every_config(gpu, beamc, oracle, shape, dtype):
     ref = oracle.matmul_nn(a, b, dtype)
     for cfg in beamc.list_configs():
         check(oracle, run_nn(beamc, a, b, dtype, cfg), ref, K, dtype, f"{cfg.name} {shape}")
+        deep = beamc.TileConfig(cfg.block_m, cfg.block_n, cfg.wave_m, cfg.wave_n, 2, 0)
+        check(oracle, run_nn(beamc, a, b, dtype, deep), ref, K, dtype, f"{deep.name} {shape}")
+
+
+@pytest.mark.parametrize("shape", [(768, 3072, 768), (256, 8192, 1024), (64, 4096, 512), (1280, 1280, 1280), (2048, 2048, 512)])
+def test_library_chosen_tile(gpu, beamc, oracle, shape):
+    """No tile named: the library takes the tile it would for gemmrc, except that tiles with 64-column wavefronts
+    give way to their 32-column relatives in this layout (and not where that would make more tiles)."""
+    M, N, K = shape
+    a = beamc.host_uniform((M, K), F16, 5, 0)
+    b = beamc.host_uniform((K, N), F16, 5, 1)
+    check(oracle, run_nn(beamc, a, b, F16), oracle.matmul_nn(a, b, F16), K, F16, f"default {shape}")
 
 
 def test_closed_forms(gpu, beamc):
@@ -137,7 +149,7 @@ def test_error_paths(gpu, beamc):
         beamc.matmul(a, b2)  # inner dimensions differ
     b3 = beamc.DeviceArray((64, 64), F16)
     with pytest.raises(beamc.BeamError) as e:
-        beamc.matmul(a, b3, config=beamc.TileConfig(128, 128, 64, 64, 2, 0))
+        beamc.matmul(a, b3, config=beamc.TileConfig(128, 128, 64, 64, 3, 0))  # no such LDS depth
     assert e.value.status == 2
     for t in (a, b, b2, b3):
         t.free()
