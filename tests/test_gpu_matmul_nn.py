@@ -130,6 +130,27 @@ def test_four_wavefront_kernel(gpu, beamc, oracle, shape, dtype):
     check(oracle, got[rows], oracle.matmul_nn(a[rows], b, dtype), K, dtype, f"{cfg.name} {shape}")
 
 
+def test_four_wavefront_kernel_random_shapes(gpu, beamc, oracle):
+    """Seeded odd shapes on the 4-wavefront kernel: any M, N a multiple of 8, K a multiple of 64 from 192 up,
+    every raster group; one to a few dozen tiles, so single-tile workgroups, edge tiles and empty columns of
+    tiles all occur."""
+    rng = np.random.default_rng(77)
+    for _ in range(24):
+        M = int(rng.integers(1, 1500))
+        N = 8 * int(rng.integers(1, 190))
+        K = int(rng.choice([192, 256, 320, 448, 1024]))
+        dtype = int(rng.integers(0, 2))
+        cfg = beamc.TileConfig(256, 256, 128, 128, 0, int(rng.choice([0, 1, 3, 4, 8])))
+        seed = int(rng.integers(0, 1 << 30))
+        a = beamc.host_uniform((M, K), dtype, seed, 0)
+        b = beamc.host_uniform((K, N), dtype, seed, 1)
+        got = run_nn(beamc, a, b, dtype, cfg)
+        what = f"M={M} N={N} K={K} dtype={dtype} group={cfg.group_m}"
+        assert (got == run_rc(beamc, a, np.ascontiguousarray(b.T), dtype, cfg)).all(), what
+        rows = np.unique(rng.integers(0, M, 48))
+        check(oracle, got[rows], oracle.matmul_nn(a[rows], b, dtype), K, dtype, what)
+
+
 def test_four_wavefront_kernel_streaming_stores(gpu, beamc, oracle):
     """An output beyond the last-level cache (12288 x 12288: 302 MB) takes the form with non-temporal stores."""
     M, N, K = 12288, 12288, 1024

@@ -91,7 +91,7 @@ def test_random_shapes(gpu, beamc, oracle):
         bkn = beamc.host_uniform((K, N8), dtype, seed, 3)
         dbk = beamc.DeviceArray.from_numpy(bkn, dtype)
         dc8 = beamc.DeviceArray((M, N8), dtype)
-        cfg = _tile(beamc, rng, [0, 1])
+        cfg = _tile(beamc, rng, [0, 1, 2])
         dc8.fill_bytes(0xEE)
         beamc.matmul(da, dbk, dc8, config=cfg)
         _close(oracle, dc8.to_numpy(), oracle.matmul_nn(a, bkn, dtype), K, dtype, f"matmul_nn {cfg.name} M={M} N={N8} K={K}")
