@@ -312,6 +312,28 @@ BEAM_TEST(matmul_nn_every_tile) {
   return c;
 }
 
+// The same on the kernel of four 128 x 128 wavefronts, which takes K a multiple of 64 from 192 up: several tiles per
+// column and row of tiles, edge tiles in M and N.
+BEAM_TEST(matmul_nn_four_wavefronts) {
+  Check c;
+  const int M = 700, N = 520, K = 320;
+  beam_tile_cfg cfg = {256, 256, 128, 128, 0, 0};
+  for (int dtype = 0; dtype < 2 && c.ok; ++dtype) {
+    std::vector<uint16_t> a = uniform16((size_t)M * K, dtype, 6, 0), b = uniform16((size_t)K * N, dtype, 6, 1);
+    std::vector<uint16_t> bt((size_t)N * K);
+    for (int k = 0; k < K; ++k)
+      for (int n = 0; n < N; ++n) bt[(size_t)n * K + k] = b[(size_t)k * N + n];
+    DevBuf da(a.size() * 2), db(b.size() * 2), dbt(bt.size() * 2), dc((size_t)M * N * 2), dc2((size_t)M * N * 2);
+    da.upload(a);
+    db.upload(b);
+    dbt.upload(bt);
+    BEAM_REQUIRE(c, beam_matmul_nn(da.p, db.p, dc.p, M, N, K, dtype, &cfg, nullptr));
+    BEAM_REQUIRE(c, beam_gemmrc(da.p, dbt.p, dc2.p, M, N, K, dtype, &cfg, nullptr));
+    if (dc.download16() != dc2.download16()) c.fail(std::string(dtype ? "bf16" : "fp16") + ": differs from gemmrc on B^T");
+  }
+  return c;
+}
+
 // GEMM with the SiLU side job: C equals the plain GEMM bit for bit, Y equals the standalone kernel,
 // silu(0) = 0 and silu(x) = x for x >= 20 (fp16), for an array longer than the K loops can carry.
 BEAM_TEST(gemm_silu_side_job) {
