@@ -31,7 +31,7 @@
 //   * B stored [K][N] (B_KMAJOR, the layout of matmul(a, b)): a B tile lies in its slot as it lies in
 //     memory, 64 rows of k by 256 columns, and a fragment is two transposing 8-byte reads
 //     (ds_read_b64_tr_b16) in place of one 16-byte read.  In a transposing read four lanes supply the
-//     addresses of the four columns groups of a 16-column block, so the same permuted column order costs
+//     addresses of the four column groups of a 16-column block, so the same permuted column order costs
 //     nothing; to keep those reads free of bank conflicts the two blocks of a pair swap their halves of a
 //     lane's 8 columns in the odd lane groups, which the store undoes with four selects (w4_kmajor_*).
 //
@@ -200,7 +200,7 @@ struct GemmW4 {
     // ---- global -> LDS -----------------------------------------------------------------------
     // Load i of wavefront w fills bytes [(4 i + w) KiB, + 1 KiB) of a slot = rows 32 i + 8 w .. + 8;
     // lane l writes position l % 8 of row 32 i + 8 w + l / 8 and fetches the chunk that belongs there.
-    // (Neither swizzle depends on i.)  The row goes into the per-lane offset, the K tile into the scalar
+    // (Neither swizzle depends on i; B as [K][N] has its own map below.)  The row goes into the per-lane offset, the K tile into the scalar
     // offset: the hardware checks their sum against the descriptor's size, and a row past the end of a
     // matrix is past it by its per-lane part alone: that check is what keeps such rows from touching memory.
     const int fill_row = 8 * wave + (lane >> 3);
