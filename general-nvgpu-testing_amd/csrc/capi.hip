@@ -825,10 +825,37 @@ static size_t ln_workspace_need(int M, int N, const beam_tile_cfg& c, int mode) 
 }
 
 // The tile a GEMM+LayerNorm call runs with: the caller's, or the default for (M, N, K); never the deep pipeline.
-static int ln_resolve_cfg(const beam_tile_cfg* cfg, int M, int N, int K, beam_tile_cfg* c, const KernelSet** ks) {
+// The library's choice is priced for the plain GEMM.  With the one-kernel LayerNorm behind it (mode AUTO or FUSED)
+// the tiles of four wavefronts are the better ones -- half the threads in every barrier of the epilogue, and the
+// 8-wavefront forms, with one workgroup per tile and every accumulator live to the end, leave registers in
+// scratch memory: 128 x 128 as 64 x 64 wavefronts (2048^3: 25.4 against 29.1 us), 256 x 128 as 128 x 64, and the
+// 256 x 256 kernel of gemm_w4.h in place of the 192- and 224-row tiles and of anything that takes more than
+// one round of workgroups (3072^3: 61.1 against 66.9 us; 6144 x 6144 x 2048: 167 against 222; 6144 x 3072 x 1024:
+// 62.6 against 83.4).
+static bool ln_fused_applies(const beam_tile_cfg& c, const KernelSet& ks, int N);
+static int ln_resolve_cfg(const beam_tile_cfg* cfg, int M, int N, int K, int mode, beam_tile_cfg* c, const KernelSet** ks) {
   int rc = resolve_cfg(cfg, M, N, K, c, ks, -1, true);
   if (rc) return rc;
   if (c->pipeline == 2) c->pipeline = 0;  // the deep pipeline exists for the store / split-K kernels only
+  if (cfg || mode == BEAM_LN_TWOPASS) return BEAM_OK;
+  const int cus = g_dev.cus > 0 ? g_dev.cus : 256;
+  const long tiles = (long)((M + c->block_m - 1) / c->block_m) * ((N + c->block_n - 1) / c->block_n);
+  const bool w4_shape = K % kBK == 0 && K >= kW4MinK && N % 8 == 0 && N <= (1 << 21);
+  beam_tile_cfg alt = *c;
+  if (w4_shape && (c->block_m >= 192 || tiles > cus)) {
+    alt.block_m = alt.block_n = 256;
+    alt.wave_m = alt.wave_n = 128;
+    alt.group_m = 0;
+  } else if ((c->block_m / c->wave_m) * (c->block_n / c->wave_n) == 8) {
+    alt.wave_m = c->block_m / 2;
+    alt.wave_n = c->block_n / 2;
+  }
+  const KernelSet* alt_ks = nullptr;
+  if ((alt.block_m != c->block_m || alt.wave_m != c->wave_m || alt.wave_n != c->wave_n) && find_set(alt) &&
+      resolve_cfg(&alt, M, N, K, &alt, &alt_ks) == BEAM_OK && ln_fused_applies(alt, *alt_ks, N)) {
+    *c = alt;
+    *ks = alt_ks;
+  }
   return BEAM_OK;
 }
 
@@ -838,7 +865,7 @@ size_t beam_gemmrc_ln_workspace_bytes_for(int M, int N, int K, const beam_tile_c
   (void)beam_init();  // AUTO depends on the device
   beam_tile_cfg c;
   const KernelSet* ks;
-  if (ln_resolve_cfg(cfg, M, N, K, &c, &ks)) return 0;
+  if (ln_resolve_cfg(cfg, M, N, K, mode, &c, &ks)) return 0;
   return ln_workspace_need(M, N, c, ln_resolve_mode(mode, c, *ks, N));
 }
 
@@ -891,18 +918,18 @@ int beam_gemmrc_ln_ex(const void* A, const void* B, const void* gamma, const voi
     BEAM_HIP(launch_ln_rows((const float*)ws, gamma, beta, Y, M, N, eps, dtype, st));
     return BEAM_OK;
   }
-  beam_tile_cfg c;
-  const KernelSet* ks;
-  if ((rc = ln_resolve_cfg(cfg, M, N, K, &c, &ks))) return rc;
-  if (mode == BEAM_LN_FUSED && !ln_fused_applies(c, *ks, N))
-    return fail(BEAM_ERR_UNSUPPORTED, "fused LayerNorm: needs a device of %d CUs and at most 64 column tiles (N=%d, block_n=%d, %d CUs)",
-                kNumXcd * 32, N, c.block_n, g_dev.cus);
   // The fused kernel's workgroups wait for one another; whether a replayed graph meets the residency that
   // wait relies on (other graph branches may share the device) is the caller's business: under stream
   // capture AUTO takes the two-pass path, an explicit FUSED is honoured.
   hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
   if (st != nullptr) (void)hipStreamIsCapturing(st, &capturing);
   if (capturing != hipStreamCaptureStatusNone && mode == BEAM_LN_AUTO) mode = BEAM_LN_TWOPASS;
+  beam_tile_cfg c;
+  const KernelSet* ks;
+  if ((rc = ln_resolve_cfg(cfg, M, N, K, mode, &c, &ks))) return rc;
+  if (mode == BEAM_LN_FUSED && !ln_fused_applies(c, *ks, N))
+    return fail(BEAM_ERR_UNSUPPORTED, "fused LayerNorm: needs a device of %d CUs and at most 64 column tiles (N=%d, block_n=%d, %d CUs)",
+                kNumXcd * 32, N, c.block_n, g_dev.cus);
   mode = ln_resolve_mode(mode, c, *ks, N);
   // The 256 x 256 tile runs on the kernel of gemm_w4.h where that one's preconditions hold (asked for by
   // name, or as the library's own choice); where they do not, the library's own choice falls back to the
@@ -943,13 +970,22 @@ int beam_gemmrc_ln_ex(const void* A, const void* B, const void* gamma, const voi
     //     measured: 16384 x 2048 x 2048, 4 + 8 against 32 + 1 panels, 112 against 120 us;
     //     8192 x 8192 x 4096, 1 + 32 against 8 + 4, 419 against 400 us; 4096^3, 18 either way, 104.1
     //     against 104.8 us)
+    // ... or, when all tiles together are at most one workgroup per CU, the plain kernels' order: the whole
+    //     grid is resident at once whatever the order, and that order is the one that streams the fewest
+    //     operand bytes into the XCDs' L2s (4096^3 in 256 x 256 tiles: a 4 x 8 block of tiles per XCD, 12
+    //     panels, instead of two whole bands, 18)
     unsigned grid;
+    const int raster_group = p.group_m;  // (base_params: the tile's rasterisation group, p.divs made for it)
     p.group_n = (p.tiles_n + kNumXcd - 1) / kNumXcd;
     p.group_m = 32 / p.group_n;
     if (p.group_m > p.tiles_m) p.group_m = p.tiles_m;
     const int bx = p.tiles_n <= 32 ? 32 / p.tiles_n : 0;
     const int rounds_spread = (p.tiles_m + p.group_m - 1) / p.group_m;
-    if (bx > 0 && p.tiles_m >= kNumXcd * bx && (p.tiles_m + kNumXcd * bx - 1) / (kNumXcd * bx) <= rounds_spread &&
+    if ((long)p.tiles_m * p.tiles_n <= (long)g_dev.cus) {
+      p.group_n = -1;
+      p.group_m = raster_group;
+      grid = (unsigned)(p.tiles_m * p.tiles_n);
+    } else if (bx > 0 && p.tiles_m >= kNumXcd * bx && (p.tiles_m + kNumXcd * bx - 1) / (kNumXcd * bx) <= rounds_spread &&
         bx + p.tiles_n <= p.group_m + p.group_n) {
       p.group_n = 0;
       p.group_m = bx;

@@ -118,7 +118,8 @@ struct GemmParams {
   int k_slice;   // K elements per split-K slice, a multiple of kBK
   int splits;    // number of K slices (1 = no split); the grid holds tiles_m * tiles_n * splits workgroups
   int group_m;   // rasterisation group height in tiles (fused LayerNorm: bands per band group)
-  int group_n;   // fused LayerNorm: columns of a band group owned by one XCD; 0: whole bands, group_m of them, per XCD
+  int group_n;   // fused LayerNorm: columns of a band group owned by one XCD; 0: whole bands, group_m of them, per XCD;
+                 // -1: the plain kernels' order (group_m is then the rasterisation group): a grid of one round of workgroups
   TileDivs divs; // the tile maps' divisors as multipliers (tile_map.h), made by the host from tiles_m, tiles_n, group_m
   // Side job (kEpiStoreSide): y[i] = silu(x[i]) over a flat 16-bit array.  The whole 8-element
   // groups of the array are cut into units of side_width bytes (16, 8 or 4), dealt out in
@@ -447,13 +448,15 @@ struct GemmTile {
 
     // Fused LayerNorm uses the band-block order, which keeps the workgroups that must exchange
     // statistics resident together; its grid is padded and the surplus workgroups leave here.
+    // (A grid of at most one workgroup per CU is resident as a whole: it keeps the plain order.)
     // Split-K walks (slice, tile) pairs slice by slice, and the XCD remap gives every XCD one
     // contiguous range of pairs: the tiles that read the same K slice of A and B share an L2.
     TileCoord tc;
     int slice = 0;
     if (EPI == kEpiLnFused) {
-      tc = p.group_n > 0 ? band_block_tile(blockIdx.x, p.tiles_m, p.tiles_n, p.group_m, p.group_n)
-                         : band_xcd_tile(blockIdx.x, p.tiles_m, p.tiles_n, p.group_m);
+      tc = p.group_n > 0    ? band_block_tile(blockIdx.x, p.tiles_m, p.tiles_n, p.group_m, p.group_n)
+           : p.group_n == 0 ? band_xcd_tile(blockIdx.x, p.tiles_m, p.tiles_n, p.group_m)
+                            : tile_of_workgroup(blockIdx.x, p.tiles_m, p.tiles_n, p.group_m, p.divs);
       if (tc.tm < 0) return;
     } else if (p.splits > 1) {
       const int tiles = p.tiles_m * p.tiles_n;

@@ -175,7 +175,9 @@ def test_ln_fused_workspace_describes_itself(gpu, beamc, oracle):
     da, db = beamc.DeviceArray.from_numpy(a), beamc.DeviceArray.from_numpy(b)
     dg, dbt = beamc.DeviceArray.from_numpy(g_), beamc.DeviceArray.from_numpy(bt)
     y = beamc.DeviceArray((M, N))
-    need = beamc.lib.beam_gemmrc_ln_workspace_bytes_for(M, N, K, None, beamc.LN_FUSED)
+    M2, N2 = 512, 1024  # the other shape that shares the buffer below
+    need = max(beamc.lib.beam_gemmrc_ln_workspace_bytes_for(M, N, K, None, beamc.LN_FUSED),
+               beamc.lib.beam_gemmrc_ln_workspace_bytes_for(M2, N2, K, None, beamc.LN_FUSED))
     assert need > 0
 
     def launch_and_check(ws, what):
@@ -205,14 +207,12 @@ def test_ln_fused_workspace_describes_itself(gpu, beamc, oracle):
         launch_and_check(ws, f"and the first data again ({rep})")
     for x in (da3, db3, dg3, dbt3):
         x.free()
-    # another shape on the same buffer in between (same bytes needed or fewer), then the first one again
-    M2, N2 = 512, 1024
+    # another shape on the same buffer in between, then the first one again
     a2, b2, g2, bt2 = make_ln_inputs(beamc, M2, N2, K, F16, 32)
     ref2 = oracle.gemmrc_ln(a2, b2, g2, bt2, 1e-5, F16)
     da2, db2 = beamc.DeviceArray.from_numpy(a2), beamc.DeviceArray.from_numpy(b2)
     dg2, dbt2 = beamc.DeviceArray.from_numpy(g2), beamc.DeviceArray.from_numpy(bt2)
     y2 = beamc.DeviceArray((M2, N2))
-    assert beamc.lib.beam_gemmrc_ln_workspace_bytes_for(M2, N2, K, None, beamc.LN_FUSED) <= need
     _ln_ex(beamc, da2, db2, dg2, dbt2, y2, M2, N2, K, F16, ws, beamc.LN_FUSED)
     beamc.sync()
     check_ln(oracle, y2.to_numpy(), ref2, F16, "other shape on the same workspace")
