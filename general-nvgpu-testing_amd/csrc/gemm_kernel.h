@@ -175,9 +175,10 @@ __device__ __forceinline__ void ln_publish(const GemmParams& p, size_t slot, flo
 }
 
 // Gathers the (mean, M2) pairs of slots [first, first + n_slots) into `gathered` (LDS, 8 bytes per slot):
-// INFLIGHT slots per thread in flight before the first is examined, each polled (one bounded budget per thread)
-// until both its words carry the tag.  A thread that runs out of budget raises the header's flag and poisons
-// the pair, so that the rows concerned come out as NaN instead of as plausible numbers.
+// batches of INFLIGHT slots per thread, a batch fetched again as a whole (one bounded budget of fetches per
+// thread) until both words of each of its slots carry the tag.  A thread that runs out of budget raises the
+// header's flag and poisons the pairs still missing, so that the rows concerned come out as NaN instead of as
+// plausible numbers.
 template <int NT, int INFLIGHT = 8>
 __device__ __forceinline__ void ln_gather(const GemmParams& p, unsigned tag, size_t first, int n_slots, int tid,
                                           unsigned long long* gathered) {
@@ -187,29 +188,36 @@ __device__ __forceinline__ void ln_gather(const GemmParams& p, unsigned tag, siz
   int polls = 0;
   for (int q0 = tid; q0 < n_slots; q0 += INFLIGHT * NT) {
     unsigned long long a[INFLIGHT], b[INFLIGHT];
+    // A batch is fetched as a whole, all its loads in flight at once, until every word of it carries the launch's
+    // tag: a retry then costs one round trip to memory for the batch, not one per word.
+    for (;;) {
 #pragma unroll
-    for (int u = 0; u < INFLIGHT; ++u) {
-      const int q = q0 + u * NT;
-      a[u] = __hip_atomic_load(w0s + (q < n_slots ? q : q0), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      b[u] = __hip_atomic_load(w1s + (q < n_slots ? q : q0), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      for (int u = 0; u < INFLIGHT; ++u) {
+        const int q = q0 + u * NT;
+        a[u] = __hip_atomic_load(w0s + (q < n_slots ? q : q0), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        b[u] = __hip_atomic_load(w1s + (q < n_slots ? q : q0), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+      bool all = true;
+#pragma unroll
+      for (int u = 0; u < INFLIGHT; ++u) all = all && (unsigned)(a[u] >> 32) == tag && (unsigned)(b[u] >> 32) == not_tag;
+      // (a negative limit: treat everything as unpublished -- how the host forces this path in a test)
+      if (all && p.spin_limit >= 0) break;
+      if (++polls > p.spin_limit) {
+        p.timeout_flag[kLnHdrTimeout] = (int)tag;
+#pragma unroll
+        for (int u = 0; u < INFLIGHT; ++u)
+          if ((unsigned)(a[u] >> 32) != tag || (unsigned)(b[u] >> 32) != not_tag || p.spin_limit < 0) {
+            a[u] = 0x7fc00000ull;
+            b[u] = 0x7fc00000ull;
+          }
+        break;
+      }
+      __builtin_amdgcn_s_sleep(4);
     }
 #pragma unroll
     for (int u = 0; u < INFLIGHT; ++u) {
       const int q = q0 + u * NT;
-      if (q >= n_slots) break;
-      // (a negative limit: treat everything as unpublished -- how the host forces this path in a test)
-      while ((unsigned)(a[u] >> 32) != tag || (unsigned)(b[u] >> 32) != not_tag || p.spin_limit < 0) {
-        if (++polls > p.spin_limit) {
-          p.timeout_flag[kLnHdrTimeout] = (int)tag;
-          a[u] = 0x7fc00000ull;
-          b[u] = 0x7fc00000ull;
-          break;
-        }
-        __builtin_amdgcn_s_sleep(4);
-        a[u] = __hip_atomic_load(w0s + q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        b[u] = __hip_atomic_load(w1s + q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      }
-      gathered[q] = (a[u] & 0xffffffffull) | (b[u] << 32);
+      if (q < n_slots) gathered[q] = (a[u] & 0xffffffffull) | (b[u] << 32);
     }
   }
 }
