@@ -175,8 +175,8 @@ __device__ __forceinline__ void ln_publish(const GemmParams& p, size_t slot, flo
 }
 
 // Gathers the (mean, M2) pairs of slots [first, first + n_slots) into `gathered` (LDS, 8 bytes per slot):
-// batches of INFLIGHT slots per thread, a batch fetched again as a whole (one bounded budget of fetches per
-// thread) until both words of each of its slots carry the tag.  A thread that runs out of budget raises the
+// batches of INFLIGHT slots per thread, the missing part of a batch fetched again (one bounded budget of tries
+// per thread) until both words of each of its slots carry the tag.  A thread that runs out of budget raises the
 // header's flag and poisons the pairs still missing, so that the rows concerned come out as NaN instead of as
 // plausible numbers.
 template <int NT, int INFLIGHT = 8>
@@ -188,31 +188,38 @@ __device__ __forceinline__ void ln_gather(const GemmParams& p, unsigned tag, siz
   int polls = 0;
   for (int q0 = tid; q0 < n_slots; q0 += INFLIGHT * NT) {
     unsigned long long a[INFLIGHT], b[INFLIGHT];
-    // A batch is fetched as a whole, all its loads in flight at once, until every word of it carries the launch's
-    // tag: a retry then costs one round trip to memory for the batch, not one per word.
+    // A batch is fetched with all its loads in flight at once; what does not carry the launch's tag yet is fetched
+    // again, again all of it at once and nothing else, after a pause that grows with the number of tries: a try
+    // costs one round trip to memory for the batch, and waiting workgroups do not flood the memory system that
+    // the tiles they wait for still need.
+    unsigned missing = 0;  // bit u: slot u of the batch is still to be fetched
+#pragma unroll
+    for (int u = 0; u < INFLIGHT; ++u) missing |= (q0 + u * NT < n_slots) ? (1u << u) : 0u;
     for (;;) {
 #pragma unroll
       for (int u = 0; u < INFLIGHT; ++u) {
-        const int q = q0 + u * NT;
-        a[u] = __hip_atomic_load(w0s + (q < n_slots ? q : q0), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        b[u] = __hip_atomic_load(w1s + (q < n_slots ? q : q0), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (missing & (1u << u)) {
+          a[u] = __hip_atomic_load(w0s + q0 + u * NT, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          b[u] = __hip_atomic_load(w1s + q0 + u * NT, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
       }
-      bool all = true;
+      // (a negative limit: treat everything as unpublished -- how the host forces the time-out in a test)
 #pragma unroll
-      for (int u = 0; u < INFLIGHT; ++u) all = all && (unsigned)(a[u] >> 32) == tag && (unsigned)(b[u] >> 32) == not_tag;
-      // (a negative limit: treat everything as unpublished -- how the host forces this path in a test)
-      if (all && p.spin_limit >= 0) break;
+      for (int u = 0; u < INFLIGHT; ++u)
+        if ((missing & (1u << u)) && (unsigned)(a[u] >> 32) == tag && (unsigned)(b[u] >> 32) == not_tag && p.spin_limit >= 0)
+          missing &= ~(1u << u);
+      if (missing == 0) break;
       if (++polls > p.spin_limit) {
         p.timeout_flag[kLnHdrTimeout] = (int)tag;
 #pragma unroll
         for (int u = 0; u < INFLIGHT; ++u)
-          if ((unsigned)(a[u] >> 32) != tag || (unsigned)(b[u] >> 32) != not_tag || p.spin_limit < 0) {
+          if (missing & (1u << u)) {
             a[u] = 0x7fc00000ull;
             b[u] = 0x7fc00000ull;
           }
         break;
       }
-      __builtin_amdgcn_s_sleep(4);
+      for (int z = 0; z < (polls < 8 ? polls : 8); ++z) __builtin_amdgcn_s_sleep(8);
     }
 #pragma unroll
     for (int u = 0; u < INFLIGHT; ++u) {

@@ -595,7 +595,7 @@ struct GemmW4 {
       __syncthreads();  // `part` is free again
       // 3. gather the band's pairs into LDS, polling (boundedly) what is not published yet
       float* gathered = part;
-      // (8 slots in flight; 16 measure the same and cost 28 scalar registers parked in vector lanes.  The codegen
+      // (8 slots in flight; 16 measure the same and cost scalar registers parked in vector lanes.  The codegen
       // test watches this kernel: a compiler short of ordinary registers parks values in accumulation registers,
       // i.e. in the accumulators.)
       ln_gather<NT, 8>(p, tag, (size_t)tc.tm * p.tiles_n * BM, p.tiles_n * BM, tid, (unsigned long long*)gathered);
