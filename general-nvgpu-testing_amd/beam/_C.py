@@ -123,6 +123,7 @@ def _load() -> ctypes.CDLL:
     L.beam_dbg_tile_of_workgroup.argtypes = [i, i, i, i, ctypes.POINTER(i), ctypes.POINTER(i)]
     L.beam_dbg_lds_offset.argtypes = [i, i]
     L.beam_dbg_kmajor_lds_offset.argtypes = [i, i, i]
+    L.beam_dbg_ln_default_config.argtypes = [i, i, i, i, ctypes.POINTER(_TileCfg)]
     L.beam_dbg_w4_kmajor_swizzle.argtypes = [i]
     L.beam_dbg_w4_kmajor_read_offset.argtypes = [i, i, i, i, i]
     L.beam_dbg_band_block_tile.argtypes = [i, i, i, i, i, ctypes.POINTER(i), ctypes.POINTER(i)]

@@ -795,15 +795,16 @@ static size_t ln_fused_set_bytes(size_t tiles_m, size_t tiles_n, int block_m) {
   return align_up(tiles_m * tiles_n * (size_t)block_m * 2 * sizeof(float), 256);
 }
 
-static bool ln_fused_applies(const beam_tile_cfg& c, const KernelSet& ks, int N) {
+static bool ln_fused_applies_on(const beam_tile_cfg& c, const KernelSet& ks, int N, int cus) {
   // The residency argument of the fused kernel (tile_map.h: band_block_tile) is made for 8 XCDs of 32 CUs.
-  if (g_dev.cus != kNumXcd * 32) return false;
+  if (cus != kNumXcd * 32) return false;
   // a band's column tiles are spread over the 8 XCDs; each XCD must hold its share (<= 32) at once,
   // and the band's statistics ((tiles_n + 1) * block_m pairs) are gathered into the kernel's LDS
   const int tiles_n = (N + c.block_n - 1) / c.block_n;
   const int lds = c.pipeline ? ks.lds_bytes_shallow : ks.lds_bytes;
   return tiles_n <= 64 && (size_t)(tiles_n + 1) * c.block_m * 8 <= (size_t)lds;
 }
+static bool ln_fused_applies(const beam_tile_cfg& c, const KernelSet& ks, int N) { return ln_fused_applies_on(c, ks, N, g_dev.cus); }
 
 static int ln_resolve_mode(int mode, const beam_tile_cfg& c, const KernelSet& ks, int N) {
   if (mode == BEAM_LN_AUTO) return ln_fused_applies(c, ks, N) ? BEAM_LN_FUSED : BEAM_LN_TWOPASS;
@@ -824,35 +825,55 @@ static size_t ln_workspace_need(int M, int N, const beam_tile_cfg& c, int mode) 
   return align_up((size_t)M * N * sizeof(float), 256) + align_up((size_t)M * tiles_n * 2 * sizeof(float), 256);
 }
 
-// The tile a GEMM+LayerNorm call runs with: the caller's, or the default for (M, N, K); never the deep pipeline.
-// The library's choice is priced for the plain GEMM.  With the one-kernel LayerNorm behind it (mode AUTO or FUSED)
-// the tiles of four wavefronts are the better ones -- half the threads in every barrier of the epilogue, and the
-// 8-wavefront forms, with one workgroup per tile and every accumulator live to the end, leave registers in
-// scratch memory: 128 x 128 as 64 x 64 wavefronts (2048^3: 25.4 against 29.1 us), 256 x 128 as 128 x 64, and the
-// 256 x 256 kernel of gemm_w4.h in place of the 192- and 224-row tiles and of anything that takes more than
-// one round of workgroups (3072^3: 61.1 against 66.9 us; 6144 x 6144 x 2048: 167 against 222; 6144 x 3072 x 1024:
-// 62.6 against 83.4).
-static bool ln_fused_applies(const beam_tile_cfg& c, const KernelSet& ks, int N);
+// The tile a GEMM+LayerNorm call runs with: the caller's, or the library's; never the deep pipeline.
+// For the one-kernel form (mode AUTO or FUSED on a device it runs on) the library does not take the plain GEMM's
+// tile: every workgroup ends with the epilogue's chain of latencies, one tile per workgroup, so a round of
+// workgroups costs a fixed time that grows with the tile, and rounds count in whole numbers.  The model is that
+// sentence: rounds x (fixed + flops of a tile / rate), rates (TFLOP/s per CU) and fixed costs (us) fitted by
+// least squares to the timings of every tile on 34 shapes (beam/ln_tile_timings.json: the pick is within 2.4%
+// of the best tile in the geometric mean, 24% at worst; the plain GEMM's tile is 7% behind in the mean).
+struct LnCandidate {
+  beam_tile_cfg cfg;
+  double rate, fixed;
+};
+static const LnCandidate kLnCandidates[] = {
+    {{256, 256, 128, 128, 0, 0}, 8.01, 12.38},  // (runs as the 8-wavefront 128 x 64 form where gemm_w4.h's conditions fail)
+    {{224, 256, 112, 64, 0, 0}, 7.91, 11.27},
+    {{192, 256, 96, 64, 0, 0}, 7.61, 10.33},
+    {{256, 128, 64, 64, 0, 0}, 6.74, 8.92},
+    {{128, 256, 64, 64, 0, 0}, 6.09, 7.81},
+    {{128, 128, 64, 32, 0, 0}, 4.92, 6.19},
+    {{64, 128, 32, 64, 0, 0}, 3.30, 3.60},
+    {{64, 64, 32, 32, 0, 0}, 3.00, 2.96},
+};
+// The model's pick for a device of `cus` compute units; false if the one-kernel form applies with none of the tiles.
+static bool ln_choose_tile(int M, int N, int K, int cus, beam_tile_cfg* out, const KernelSet** out_ks) {
+  double best_us = 1e300;
+  bool found = false;
+  for (const LnCandidate& k : kLnCandidates) {
+    beam_tile_cfg c = k.cfg;
+    const KernelSet* ks = nullptr;
+    if (resolve_cfg(&c, M, N, K, &c, &ks) != BEAM_OK || !ln_fused_applies_on(c, *ks, N, cus)) continue;
+    const long tiles = (long)((M + c.block_m - 1) / c.block_m) * ((N + c.block_n - 1) / c.block_n);
+    const double rounds = (double)((tiles + cus - 1) / cus);
+    const double us = rounds * (k.fixed + 2.0e-6 * c.block_m * c.block_n * (double)K / k.rate);
+    if (us < best_us) {
+      best_us = us;
+      *out = c;
+      *out_ks = ks;
+      found = true;
+    }
+  }
+  return found;
+}
 static int ln_resolve_cfg(const beam_tile_cfg* cfg, int M, int N, int K, int mode, beam_tile_cfg* c, const KernelSet** ks) {
   int rc = resolve_cfg(cfg, M, N, K, c, ks, -1, true);
   if (rc) return rc;
   if (c->pipeline == 2) c->pipeline = 0;  // the deep pipeline exists for the store / split-K kernels only
-  if (cfg || mode == BEAM_LN_TWOPASS) return BEAM_OK;
-  const int cus = g_dev.cus > 0 ? g_dev.cus : 256;
-  const long tiles = (long)((M + c->block_m - 1) / c->block_m) * ((N + c->block_n - 1) / c->block_n);
-  const bool w4_shape = K % kBK == 0 && K >= kW4MinK && N % 8 == 0 && N <= (1 << 21);
-  beam_tile_cfg alt = *c;
-  if (w4_shape && (c->block_m >= 192 || tiles > cus)) {
-    alt.block_m = alt.block_n = 256;
-    alt.wave_m = alt.wave_n = 128;
-    alt.group_m = 0;
-  } else if ((c->block_m / c->wave_m) * (c->block_n / c->wave_n) == 8) {
-    alt.wave_m = c->block_m / 2;
-    alt.wave_n = c->block_n / 2;
-  }
+  if (cfg || mode == BEAM_LN_TWOPASS || g_dev.cus <= 0) return BEAM_OK;
+  beam_tile_cfg alt;
   const KernelSet* alt_ks = nullptr;
-  if ((alt.block_m != c->block_m || alt.wave_m != c->wave_m || alt.wave_n != c->wave_n) && find_set(alt) &&
-      resolve_cfg(&alt, M, N, K, &alt, &alt_ks) == BEAM_OK && ln_fused_applies(alt, *alt_ks, N)) {
+  if (ln_choose_tile(M, N, K, g_dev.cus, &alt, &alt_ks)) {
     *c = alt;
     *ks = alt_ks;
   }
@@ -1281,6 +1302,12 @@ int beam_dbg_band_xcd_grid(int tiles_m, int tiles_n, int bx) { return band_xcd_g
 int beam_dbg_lds_offset(int row, int chunk) { return lds_offset(row, chunk); }
 
 int beam_dbg_kmajor_lds_offset(int k, int n, int block_n) { return kmajor_lds_offset(k, n, block_n); }
+
+int beam_dbg_ln_default_config(int M, int N, int K, int compute_units, beam_tile_cfg* cfg) {
+  if (!cfg || M <= 0 || N <= 0 || K <= 0) return fail(BEAM_ERR_INVALID, "bad argument");
+  const KernelSet* ks = nullptr;
+  return ln_choose_tile(M, N, K, compute_units, cfg, &ks) ? BEAM_OK : BEAM_ERR_UNSUPPORTED;
+}
 
 int beam_dbg_w4_kmajor_swizzle(int k) { return w4_kmajor_swizzle(k); }
 

@@ -324,6 +324,9 @@ int beam_dbg_lds_offset(int row, int chunk);
 /* Byte offset of element (k, n), n a multiple of 4, inside a K-major LDS stage of block_n columns
  * (B stored [K][N], beam_matmul_nn). */
 int beam_dbg_kmajor_lds_offset(int k, int n, int block_n);
+/* The tile a beam_gemmrc_ln call without a tile takes for its one-kernel form on a device of `compute_units` CUs
+ * (the library's LayerNorm cost model; BEAM_ERR_UNSUPPORTED where that form applies with no tile). */
+int beam_dbg_ln_default_config(int M, int N, int K, int compute_units, beam_tile_cfg* cfg);
 /* The 4-wavefront kernel with B stored [K][N] (256 columns, 512 bytes per row of k in an LDS slot): the XOR code of
  * the 16-byte chunks of row k, and the byte offset of the 8 bytes that lane 16 g + 4 e + q supplies to the first
  * transposing read of 16-column block b (0..7) of the wavefront's column half wn (0, 1). */

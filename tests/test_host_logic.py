@@ -1,6 +1,7 @@
 """Host-side logic of libbeam_hip.so that needs no GPU: index maps shared with the kernels,
 the split heuristic, workspace sizes, the synthetic-data generator and argument validation."""
 import ctypes
+import os
 
 import numpy as np
 import pytest
@@ -125,6 +126,36 @@ def test_kmajor_lds_layout_is_bijective_and_conflict_free(beamc):
                         o = L.beam_dbg_kmajor_lds_offset(kbase + 8 * g + e, n0 + 4 * q, bn)
                         banks += [(o // 4) % 64, (o // 4 + 1) % 64]
                     assert sorted(banks) == list(range(64)), (bn, n0, kbase, half)
+
+
+def test_layernorm_tile_model_against_its_timing_table(beamc):
+    """The tile a GEMM+LayerNorm call without a tile takes (one-kernel form, 256 CUs) against the committed timings
+    of every tile on 34 shapes: within 4% of the best tile in the geometric mean and 25% at worst.  (The table's
+    256x256_w128x128 column is the tile as named; the library's own choice of it runs as the 8-wavefront form
+    where the 4-wavefront kernel's conditions fail, which is never slower.)"""
+    import ctypes
+    import json
+    import math
+    path = os.path.join(os.path.dirname(os.path.abspath(beamc.__file__)), "ln_tile_timings.json")
+    table = json.load(open(path))
+    assert len(table) >= 30
+    logs, worst = [], 1.0
+    for shape, row in table.items():
+        M, N, K = (int(x) for x in shape.split("x"))
+        c = beamc._TileCfg()
+        assert beamc.lib.beam_dbg_ln_default_config(M, N, K, 256, ctypes.byref(c)) == 0
+        name = beamc.TileConfig(c.block_m, c.block_n, c.wave_m, c.wave_n, 0, 0).name
+        tiles = {k: v for k, v in row.items() if k not in ("default", "plain")}
+        picked = tiles[name]
+        if name == "256x256_w128x128" and "256x256_w128x64" in tiles:
+            picked = min(picked, tiles["256x256_w128x64"])
+        r = picked / min(tiles.values())
+        logs.append(math.log(r))
+        worst = max(worst, r)
+    assert math.exp(sum(logs) / len(logs)) < 1.04 and worst < 1.25
+    # no compute units, or not the device the one-kernel form is made for: no pick
+    c = beamc._TileCfg()
+    assert beamc.lib.beam_dbg_ln_default_config(4096, 4096, 4096, 304, ctypes.byref(c)) != 0
 
 
 def test_w4_kmajor_fragments_and_banks(beamc):
