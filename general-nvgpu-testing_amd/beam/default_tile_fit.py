@@ -14,6 +14,9 @@ of 40 launches each, on one MI355X.  `PARAMS` below are the constants compiled i
     python -m beam.default_tile_fit --collect F  re-measure the table on the GPU at hand into file F
     python -m beam.default_tile_fit --split      the same for calls with a workspace (split-K): pick against sweep
     python -m beam.default_tile_fit --collect-split F   re-measure the split-K sweep into file F
+    python -m beam.default_tile_fit --ln         the GEMM+LayerNorm model's pick per shape against its table
+    python -m beam.default_tile_fit --fit-ln     least-squares fit of that model's constants to the table
+    python -m beam.default_tile_fit --collect-ln F      re-measure that table into file F
 
 With a workspace (beam_gemmrc_splitk, split_k <= 0, no tile given) the deep-pipeline candidates are priced with
 their K slices (`auto_slices`) and the reduction; `splitk_timings.json` holds, for 25 shapes from 64x64x8192 to
@@ -21,6 +24,12 @@ their K slices (`auto_slices`) and the reduction; `splitk_timings.json` holds, f
 S in {4, 8, 16, 32, 64} (uniform operands, best of two rounds of 100 calls, one MI355X, the library as shipped:
 one launch or two as it decides): the model's pick is what
 `predict_split` restates, and a test keeps it in step with the library.
+
+A GEMM+LayerNorm call without a tile (one-kernel form) has a model of its own: one tile per workgroup, each ending
+in the epilogue's chain of latencies, so the cost is rounds x (fixed + a tile's flops / rate) with whole rounds.
+`ln_tile_timings.json` holds microseconds per call of the one-kernel form with every compiled tile (3 + 2 slots) on 34
+shapes (fp16, N(0,1)/sqrt(K), best of two rounds, one MI355X; "default": the library's pick at the time, "plain": the
+plain GEMM); `LN_PARAMS` are the least-squares constants compiled into the library (csrc/capi.hip, kLnCandidates).
 
 This stands where the reference has fixed default shapes (cuda/cutlass_kernels/cutlass_gemmrc.cu:22-24).
 """
@@ -201,6 +210,112 @@ def refit(params, timings, steps=4000, seed=1):
     return params, best
 
 
+LN_TIMINGS = os.path.join(os.path.dirname(os.path.abspath(__file__)), "ln_tile_timings.json")
+# name -> (TFLOP/s per CU, fixed microseconds per round of workgroups); order = the library's candidate order
+LN_PARAMS = {
+    "256x256_w128x128": (8.01, 12.38), "224x256_w112x64": (7.91, 11.27), "192x256_w96x64": (7.61, 10.33),
+    "256x128_w64x64": (6.74, 8.92), "128x256_w64x64": (6.09, 7.81), "128x128_w64x32": (4.92, 6.19),
+    "64x128_w32x64": (3.30, 3.60), "64x64_w32x32": (3.00, 2.96),
+}
+# (fitted on the table's column of the 8-wavefront 256x256 tile; the library runs the 4-wavefront kernel where it fits)
+LN_FIT_COLUMN = {"256x256_w128x128": "256x256_w128x64"}
+
+
+def _ln_block(name):
+    bm, bn = name.split("_w")[0].split("x")
+    return int(bm), int(bn)
+
+
+def ln_fused_applies(name, N, cus=CUS):
+    """The one-kernel form's conditions that depend on the tile: 256 CUs, at most 64 column tiles, and the band's
+    statistics fit the kernel's LDS ((3 + 2 slots) x 64 K elements x 2 bytes x (block_m, block_n) rows)."""
+    bm, bn = _ln_block(name)
+    tiles_n = -(-N // bn)
+    lds = (3 * bm + 2 * bn) * 128
+    return cus == 256 and tiles_n <= 64 and (tiles_n + 1) * bm * 8 <= lds
+
+
+def predict_ln(params, M, N, K, cus=CUS):
+    """(name, modelled us) of the tile the library takes for the one-kernel GEMM+LayerNorm, None where none applies."""
+    best = None
+    for name, (rate, fixed) in params.items():
+        if not ln_fused_applies(name, N, cus):
+            continue
+        bm, bn = _ln_block(name)
+        rounds = -(-(-(-M // bm) * -(-N // bn)) // cus)
+        us = rounds * (fixed + 2.0e-6 * bm * bn * K / rate)
+        if best is None or us < best[1]:
+            best = (name, us)
+    return best
+
+
+def ln_regret(params, table, rows=None):
+    logs, worst = [], 1.0
+    for key, row in table.items():
+        M, N, K = map(int, key.split("x"))
+        tiles = {k: v for k, v in row.items() if k not in ("default", "plain")}
+        name, us = predict_ln(params, M, N, K)
+        t = min(tiles[name], tiles.get(LN_FIT_COLUMN.get(name, name), 1e9))
+        bname = min(tiles, key=tiles.get)
+        r = t / tiles[bname]
+        logs.append(math.log(r))
+        worst = max(worst, r)
+        if rows is not None:
+            rows.append((key, name, t, us, bname, tiles[bname], r, row.get("plain")))
+    return math.exp(sum(logs) / len(logs)), worst
+
+
+def fit_ln(table):
+    """Per tile, weighted least squares of measured us on (rounds, rounds x flops of a tile): relative errors."""
+    import numpy as np
+    out = {}
+    for name in LN_PARAMS:
+        col = LN_FIT_COLUMN.get(name, name)
+        X, y = [], []
+        for key, row in table.items():
+            if col not in row:
+                continue
+            M, N, K = map(int, key.split("x"))
+            bm, bn = _ln_block(name)
+            rounds = -(-(-(-M // bm) * -(-N // bn)) // CUS)
+            X.append([rounds, rounds * 2.0e-6 * bm * bn * K])
+            y.append(row[col])
+        X, y = np.array(X), np.array(y)
+        coef = np.linalg.lstsq(X / y[:, None], np.ones(len(y)), rcond=None)[0]
+        out[name] = (round(float(1.0 / coef[1]), 2), round(float(coef[0]), 2))
+    return out
+
+
+def collect_ln(path):
+    """Times the one-kernel GEMM+LayerNorm with every compiled tile on the table's shapes on the GPU at hand."""
+    from . import _C
+    out = {}
+    for key in json.load(open(LN_TIMINGS)):
+        M, N, K = map(int, key.split("x"))
+        a = _C.DeviceArray.from_numpy(_C.host_normal((M, K), _C.F16, 7, 0, 0.0, K ** -0.5))
+        b = _C.DeviceArray.from_numpy(_C.host_normal((N, K), _C.F16, 7, 1, 0.0, K ** -0.5))
+        g = _C.DeviceArray.from_numpy(_C.host_normal((N,), _C.F16, 7, 2, 1.0, 0.1))
+        bt = _C.DeviceArray.from_numpy(_C.host_normal((N,), _C.F16, 7, 3, 0.0, 0.1))
+        c = _C.DeviceArray((M, N))
+        n = max(40, int(6000 / max(1.0, 2.0 * M * N * K / 1.2e9)))
+        row = {}
+        for cfg in _C.list_configs():
+            t = _C.TileConfig(cfg.block_m, cfg.block_n, cfg.wave_m, cfg.wave_n, 0, 0)
+            try:
+                row[t.name] = round(min(_C.bench(_C.OP_GEMM_LN, a, b, c, gamma=g, beta=bt, config=t, warmup=n, iters=n,
+                                                 ln_mode=_C.LN_FUSED) for _ in range(2)) * 1e3, 2)
+            except _C.BeamError:
+                continue
+        row["default"] = round(min(_C.bench(_C.OP_GEMM_LN, a, b, c, gamma=g, beta=bt, warmup=n, iters=n) for _ in range(2)) * 1e3, 2)
+        row["plain"] = round(min(_C.bench(_C.OP_GEMM, a, b, c, warmup=n, iters=n) for _ in range(2)) * 1e3, 2)
+        for x in (a, b, g, bt, c):
+            x.free()
+        out[key] = row
+        print(key, "plain", row["plain"], "default", row["default"], flush=True)
+        with open(path, "w") as f:
+            json.dump(out, f, indent=0)
+
+
 def collect(path):
     """Times every compiled tile (both pipeline depths) on the table's shapes on the GPU at hand."""
     from . import _C
@@ -236,6 +351,24 @@ def main(argv):
         return 0
     if argv[:1] == ["--collect-split"]:
         collect_split(argv[1])
+        return 0
+    if argv[:1] == ["--collect-ln"]:
+        collect_ln(argv[1])
+        return 0
+    if argv[:1] in (["--ln"], ["--fit-ln"]):
+        table = json.load(open(LN_TIMINGS))
+        params = LN_PARAMS
+        if argv[0] == "--fit-ln":
+            params = fit_ln(table)
+            for name, (rate, fixed) in params.items():
+                print(f"{name:22s} {rate:.2f} {fixed:.2f}")
+        rows = []
+        mean, worst = ln_regret(params, table, rows)
+        print("| shape | model's pick | measured us | modelled us | best tile of all | its us | pick / best | plain GEMM us |")
+        print("|---|---|---|---|---|---|---|---|")
+        for key, name, t, us, bname, bt, r, plain in rows:
+            print(f"| {key} | {name} | {t:.1f} | {us:.1f} | {bname} | {bt:.1f} | {r:.3f} | {plain} |")
+        print(f"geometric mean {mean:.4f}, worst {worst:.3f} over {len(rows)} shapes")
         return 0
     if argv[:1] == ["--split"]:
         rows = []

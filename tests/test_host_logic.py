@@ -156,6 +156,18 @@ def test_layernorm_tile_model_against_its_timing_table(beamc):
     # no compute units, or not the device the one-kernel form is made for: no pick
     c = beamc._TileCfg()
     assert beamc.lib.beam_dbg_ln_default_config(4096, 4096, 4096, 304, ctypes.byref(c)) != 0
+    # the Python restatement (what the fit works on) and the compiled model pick the same tile
+    from beam import default_tile_fit as fit
+    rng = np.random.default_rng(5)
+    shapes = [tuple(int(x) for x in s.split("x")) for s in table]
+    shapes += [(int(rng.integers(1, 9000)), 8 * int(rng.integers(1, 2200)), 64 * int(rng.integers(1, 130))) for _ in range(300)]
+    for M, N, K in shapes:
+        want = fit.predict_ln(fit.LN_PARAMS, M, N, K)
+        rc = beamc.lib.beam_dbg_ln_default_config(M, N, K, 256, ctypes.byref(c))
+        if want is None:
+            assert rc != 0, (M, N, K)
+            continue
+        assert rc == 0 and beamc.TileConfig(c.block_m, c.block_n, c.wave_m, c.wave_n, 0, 0).name == want[0], (M, N, K, want)
 
 
 def test_w4_kmajor_fragments_and_banks(beamc):
