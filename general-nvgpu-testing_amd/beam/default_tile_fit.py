@@ -213,9 +213,9 @@ def refit(params, timings, steps=4000, seed=1):
 LN_TIMINGS = os.path.join(os.path.dirname(os.path.abspath(__file__)), "ln_tile_timings.json")
 # name -> (TFLOP/s per CU, fixed microseconds per round of workgroups); order = the library's candidate order
 LN_PARAMS = {
-    "256x256_w128x128": (8.01, 12.38), "224x256_w112x64": (7.91, 11.27), "192x256_w96x64": (7.61, 10.33),
-    "256x128_w64x64": (6.74, 8.92), "128x256_w64x64": (6.09, 7.81), "128x128_w64x32": (4.92, 6.19),
-    "64x128_w32x64": (3.30, 3.60), "64x64_w32x32": (3.00, 2.96),
+    "256x256_w128x128": (7.90, 12.62), "224x256_w112x64": (7.77, 11.56), "192x256_w96x64": (7.49, 10.76),
+    "256x128_w64x64": (6.53, 9.29), "128x256_w64x64": (6.09, 8.77), "128x128_w64x32": (4.85, 6.60),
+    "64x128_w32x64": (3.23, 3.84), "64x64_w32x32": (3.07, 3.19),
 }
 # (fitted on the table's column of the 8-wavefront 256x256 tile; the library runs the 4-wavefront kernel where it fits)
 LN_FIT_COLUMN = {"256x256_w128x128": "256x256_w128x64"}

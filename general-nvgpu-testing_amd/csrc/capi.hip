@@ -830,21 +830,21 @@ static size_t ln_workspace_need(int M, int N, const beam_tile_cfg& c, int mode) 
 // tile: every workgroup ends with the epilogue's chain of latencies, one tile per workgroup, so a round of
 // workgroups costs a fixed time that grows with the tile, and rounds count in whole numbers.  The model is that
 // sentence: rounds x (fixed + flops of a tile / rate), rates (TFLOP/s per CU) and fixed costs (us) fitted by
-// least squares to the timings of every tile on 34 shapes (beam/ln_tile_timings.json: the pick is within 2.4%
-// of the best tile in the geometric mean, 24% at worst; the plain GEMM's tile is 7% behind in the mean).
+// least squares to the timings of every tile on 34 shapes (beam/ln_tile_timings.json: the pick is within 1.5%
+// of the best tile in the geometric mean, 16% at worst; the plain GEMM's tile is 7% behind in the mean).
 struct LnCandidate {
   beam_tile_cfg cfg;
   double rate, fixed;
 };
 static const LnCandidate kLnCandidates[] = {
-    {{256, 256, 128, 128, 0, 0}, 8.01, 12.38},  // (runs as the 8-wavefront 128 x 64 form where gemm_w4.h's conditions fail)
-    {{224, 256, 112, 64, 0, 0}, 7.91, 11.27},
-    {{192, 256, 96, 64, 0, 0}, 7.61, 10.33},
-    {{256, 128, 64, 64, 0, 0}, 6.74, 8.92},
-    {{128, 256, 64, 64, 0, 0}, 6.09, 7.81},
-    {{128, 128, 64, 32, 0, 0}, 4.92, 6.19},
-    {{64, 128, 32, 64, 0, 0}, 3.30, 3.60},
-    {{64, 64, 32, 32, 0, 0}, 3.00, 2.96},
+    {{256, 256, 128, 128, 0, 0}, 7.90, 12.62},  // (runs as the 8-wavefront 128 x 64 form where gemm_w4.h's conditions fail)
+    {{224, 256, 112, 64, 0, 0}, 7.77, 11.56},
+    {{192, 256, 96, 64, 0, 0}, 7.49, 10.76},
+    {{256, 128, 64, 64, 0, 0}, 6.53, 9.29},
+    {{128, 256, 64, 64, 0, 0}, 6.09, 8.77},
+    {{128, 128, 64, 32, 0, 0}, 4.85, 6.60},
+    {{64, 128, 32, 64, 0, 0}, 3.23, 3.84},
+    {{64, 64, 32, 32, 0, 0}, 3.07, 3.19},
 };
 // The model's pick for a device of `cus` compute units; false if the one-kernel form applies with none of the tiles.
 static bool ln_choose_tile(int M, int N, int K, int cus, beam_tile_cfg* out, const KernelSet** out_ks) {
@@ -991,24 +991,27 @@ int beam_gemmrc_ln_ex(const void* A, const void* B, const void* gamma, const voi
     //     measured: 16384 x 2048 x 2048, 4 + 8 against 32 + 1 panels, 112 against 120 us;
     //     8192 x 8192 x 4096, 1 + 32 against 8 + 4, 419 against 400 us; 4096^3, 18 either way, 104.1
     //     against 104.8 us)
-    // ... or, when all tiles together are at most one workgroup per CU, the plain kernels' order: the whole
-    //     grid is resident at once whatever the order, and that order is the one that streams the fewest
-    //     operand bytes into the XCDs' L2s (4096^3 in 256 x 256 tiles: a 4 x 8 block of tiles per XCD, 12
-    //     panels, instead of two whole bands, 18) and needs no padded grid (3072^3 in 256 x 256 tiles: 60.8
-    //     against 66.4 us; 4096^3 and 2048^3 the same either way)
+    // ... or, where those two orders' padding costs rounds of workgroups (20 column tiles are 3 per XCD on
+    //     seven XCDs and none on the eighth: 3000 x 5000 x 2000 in 256 x 256 tiles puts 36 workgroups on six
+    //     XCDs of 32 CUs), band after band with no padding: id = band * tiles_n + column, which the hardware's
+    //     round-robin deals out evenly.
+    // All three keep a band's workgroups together in id order, so a launch that gets only part of the device
+    // still finishes band by band.  (The plain kernels' raster order streams fewer operand bytes into the L2s
+    // when the whole grid is one round -- 4096^3: 204 against 303 MB, in the same time -- but loses exactly that.)
     unsigned grid;
-    const int raster_group = p.group_m;  // (base_params: the tile's rasterisation group, p.divs made for it)
     p.group_n = (p.tiles_n + kNumXcd - 1) / kNumXcd;
     p.group_m = 32 / p.group_n;
     if (p.group_m > p.tiles_m) p.group_m = p.tiles_m;
     const int bx = p.tiles_n <= 32 ? 32 / p.tiles_n : 0;
     const int rounds_spread = (p.tiles_m + p.group_m - 1) / p.group_m;
-    if ((long)p.tiles_m * p.tiles_n <= (long)g_dev.cus) {
+    const bool whole_bands = bx > 0 && p.tiles_m >= kNumXcd * bx && (p.tiles_m + kNumXcd * bx - 1) / (kNumXcd * bx) <= rounds_spread &&
+                             bx + p.tiles_n <= p.group_m + p.group_n;
+    const int rounds_grouped = whole_bands ? (p.tiles_m + kNumXcd * bx - 1) / (kNumXcd * bx) : rounds_spread;
+    const long per_xcd = ((long)p.tiles_m * p.tiles_n + kNumXcd - 1) / kNumXcd;
+    if ((per_xcd + 31) / 32 < rounds_grouped) {
       p.group_n = -1;
-      p.group_m = raster_group;
       grid = (unsigned)(p.tiles_m * p.tiles_n);
-    } else if (bx > 0 && p.tiles_m >= kNumXcd * bx && (p.tiles_m + kNumXcd * bx - 1) / (kNumXcd * bx) <= rounds_spread &&
-        bx + p.tiles_n <= p.group_m + p.group_n) {
+    } else if (whole_bands) {
       p.group_n = 0;
       p.group_m = bx;
       grid = (unsigned)band_xcd_grid(p.tiles_m, p.tiles_n, bx);

@@ -119,7 +119,7 @@ struct GemmParams {
   int splits;    // number of K slices (1 = no split); the grid holds tiles_m * tiles_n * splits workgroups
   int group_m;   // rasterisation group height in tiles (fused LayerNorm: bands per band group)
   int group_n;   // fused LayerNorm: columns of a band group owned by one XCD; 0: whole bands, group_m of them, per XCD;
-                 // -1: the plain kernels' order (group_m is then the rasterisation group): a grid of one round of workgroups
+                 // -1: band after band, workgroup id = band * tiles_n + column (no padding)
   TileDivs divs; // the tile maps' divisors as multipliers (tile_map.h), made by the host from tiles_m, tiles_n, group_m
   // Side job (kEpiStoreSide): y[i] = silu(x[i]) over a flat 16-bit array.  The whole 8-element
   // groups of the array are cut into units of side_width bytes (16, 8 or 4), dealt out in
@@ -462,8 +462,10 @@ struct GemmTile {
     }
 
     // Fused LayerNorm uses the band-block order, which keeps the workgroups that must exchange
-    // statistics resident together; its grid is padded and the surplus workgroups leave here.
-    // (A grid of at most one workgroup per CU is resident as a whole: it keeps the plain order.)
+    // statistics resident together -- and, because a band's workgroups have consecutive ids and workgroups are
+    // placed in id order, lets a launch that gets only part of the device finish band by band.  Its grid is
+    // padded and the surplus workgroups leave here.  (Where the padding would cost a round of workgroups the
+    // host asks for the plain band-after-band order, which has the same property and no padding.)
     // Split-K walks (slice, tile) pairs slice by slice, and the XCD remap gives every XCD one
     // contiguous range of pairs: the tiles that read the same K slice of A and B share an L2.
     TileCoord tc;
@@ -471,7 +473,7 @@ struct GemmTile {
     if (EPI == kEpiLnFused) {
       tc = p.group_n > 0    ? band_block_tile(blockIdx.x, p.tiles_m, p.tiles_n, p.group_m, p.group_n)
            : p.group_n == 0 ? band_xcd_tile(blockIdx.x, p.tiles_m, p.tiles_n, p.group_m)
-                            : tile_of_workgroup(blockIdx.x, p.tiles_m, p.tiles_n, p.group_m, p.divs);
+                            : TileCoord{(int)blockIdx.x / p.tiles_n, (int)blockIdx.x % p.tiles_n};
       if (tc.tm < 0) return;
     } else if (p.splits > 1) {
       const int tiles = p.tiles_m * p.tiles_n;

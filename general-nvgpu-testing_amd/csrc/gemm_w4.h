@@ -192,7 +192,7 @@ struct GemmW4 {
     if constexpr (LN) {
       ln_tile = p.group_n > 0    ? band_block_tile(blockIdx.x, p.tiles_m, p.tiles_n, p.group_m, p.group_n)
                 : p.group_n == 0 ? band_xcd_tile(blockIdx.x, p.tiles_m, p.tiles_n, p.group_m)
-                                 : tile_of_workgroup(blockIdx.x, p.tiles_m, p.tiles_n, p.group_m, p.divs);
+                                 : TileCoord{(int)blockIdx.x / p.tiles_n, (int)blockIdx.x % p.tiles_n};
       if (ln_tile.tm < 0) return;  // the band grids are padded
     }
     const int my_tiles = LN ? 1 : (total_tiles - first_tile + tile_step - 1) / tile_step;
