@@ -221,6 +221,62 @@ def test_ln_fused_workspace_describes_itself(gpu, beamc, oracle):
         x.free()
 
 
+def test_two_fused_launches_share_the_device(gpu, beamc):
+    """Two streams, each with fused launches that fill the device on their own (256 tiles each), issued in turn so
+    that the two are in flight together: a band's workgroups have consecutive ids and are placed in id order, so a
+    launch that holds only part of the device finishes band by band and nobody waits for a workgroup that cannot be
+    placed.  Every result equals the one from a quiet device, and no launch gives up waiting.  (The wait is
+    bounded in any case; the budget is lowered here so that a regression fails in seconds.)"""
+    import ctypes
+    L = beamc.lib
+    M, N, K = 4096, 4096, 256
+    streams = []
+    for _ in range(2):
+        s = ctypes.c_void_p()
+        beamc._check(L.beam_stream_create(ctypes.byref(s)))
+        streams.append(s)
+    sets = []
+    for i in range(2):
+        a, b, g_, bt = make_ln_inputs(beamc, M, N, K, F16, 71 + i)
+        d = [beamc.DeviceArray.from_numpy(x) for x in (a, b, g_, bt)]
+        y = beamc.DeviceArray((M, N))
+        ws = beamc.DeviceArray((L.beam_gemmrc_ln_workspace_bytes_for(M, N, K, None, beamc.LN_FUSED),), itemsize=1)
+        sets.append((d, y, ws))
+
+    def launch(i, stream):
+        (da, db, dg, dbt), y, ws = sets[i]
+        rc = L.beam_gemmrc_ln_ex(da.ptr, db.ptr, dg.ptr, dbt.ptr, ctypes.c_float(1e-5), y.ptr, M, N, K, F16, None, beamc.LN_FUSED,
+                                 ws.ptr, ws.nbytes, stream)
+        assert rc == 0, L.beam_last_error().decode()
+
+    want = []
+    for i in range(2):
+        launch(i, None)
+        beamc.sync()
+        want.append(sets[i][1].to_numpy().copy())
+    beamc._check(L.beam_set_ln_spin_limit(500000))
+    try:
+        for rep in range(30):
+            for i in range(2):
+                sets[i][1].fill_bytes(0xEE)
+            beamc.sync()
+            for _ in range(4):
+                for i in range(2):
+                    launch(i, streams[i])
+            for i in range(2):
+                flag = ctypes.c_int(1)
+                beamc._check(L.beam_gemmrc_ln_timed_out(sets[i][2].ptr, streams[i], ctypes.byref(flag)))
+                assert flag.value == 0, f"stream {i} gave up waiting (repetition {rep})"
+                assert (sets[i][1].to_numpy() == want[i]).all(), f"stream {i}, repetition {rep}"
+    finally:
+        beamc._check(L.beam_set_ln_spin_limit(4 << 20))
+        for s in streams:
+            beamc._check(L.beam_stream_destroy(s))
+        for d, y, ws in sets:
+            for t in d + [y, ws]:
+                t.free()
+
+
 def test_ln_default_call_never_lacks_workspace(gpu, beamc, oracle):
     """M=1024, N=8192, K=2048 without a tile: the library's tile for that K takes the two-pass path (32 column
     tiles of 256 fit the fused kernel, but the tile chosen is another); the Python wrapper sizes its buffer for
