@@ -204,9 +204,7 @@ def extra_splitk(_C):
             "hbm_frac": round(bytes_alg / (best_split[1] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
 
 
-def extra_ln(_C):
-    """fused GEMM+LayerNorm at 4096^3 against the plain GEMM of the same tile."""
-    M = N = K = 4096
+def ln_against_plain(_C, M, N, K):
     a = _C.DeviceArray.from_numpy(_C.host_normal((M, K), _C.F16, 22, 0, 0.0, K ** -0.5))
     b = _C.DeviceArray.from_numpy(_C.host_normal((N, K), _C.F16, 22, 1, 0.0, K ** -0.5))
     g = _C.DeviceArray.from_numpy(_C.host_normal((N,), _C.F16, 22, 2, 1.0, 0.1))
@@ -221,6 +219,14 @@ def extra_ln(_C):
     return {"shape": [M, N, K], "gemm_us": round(plain * 1e3, 1), "gemm_ln_us": round(fused * 1e3, 1),
             "overhead": round(fused / plain - 1.0, 4),
             "gemm_ln_TFLOPs": round(2.0 * M * N * K / (fused * 1e-3) / 1e12, 1)}
+
+
+def extra_ln(_C):
+    """fused GEMM+LayerNorm at 4096^3 against the plain GEMM, each with the tile the library picks for it; and the
+    same for a few other shapes (one round of small tiles, several rounds of large ones, ragged edges)."""
+    out = ln_against_plain(_C, 4096, 4096, 4096)
+    out["other_shapes"] = [ln_against_plain(_C, *s) for s in ((2048, 2048, 2048), (8192, 8192, 4096), (3000, 5000, 2000))]
+    return out
 
 
 def extra_silu(_C):
