@@ -221,11 +221,49 @@ def ln_against_plain(_C, M, N, K):
             "gemm_ln_TFLOPs": round(2.0 * M * N * K / (fused * 1e-3) / 1e12, 1)}
 
 
+def ln_two_pass(_C, M, N, K):
+    """The two-pass form at the same shape, and its normalisation pass alone (reads fp32 X, writes 16-bit Y)."""
+    a = _C.DeviceArray.from_numpy(_C.host_normal((M, K), _C.F16, 22, 0, 0.0, K ** -0.5))
+    b = _C.DeviceArray.from_numpy(_C.host_normal((N, K), _C.F16, 22, 1, 0.0, K ** -0.5))
+    g = _C.DeviceArray.from_numpy(_C.host_normal((N,), _C.F16, 22, 2, 1.0, 0.1))
+    bt = _C.DeviceArray.from_numpy(_C.host_normal((N,), _C.F16, 22, 3, 0.0, 0.1))
+    c = _C.DeviceArray((M, N))
+    two = settled_ms(lambda w, n: _C.bench(_C.OP_GEMM_LN, a, b, c, gamma=g, beta=bt, ln_mode=_C.LN_TWOPASS, warmup=w, iters=n))
+    apply_ms = settled_ms(lambda w, n: _C.bench(_C.OP_PROBE_LN_APPLY, a, b, c, gamma=g, beta=bt, warmup=w, iters=n))
+    for x in (a, b, g, bt, c):
+        x.free()
+    apply_bytes = 6.0 * M * N + 4.0 * N
+    return {"two_pass_us": round(two * 1e3, 1), "apply_pass_us": round(apply_ms * 1e3, 2),
+            "apply_pass_GBs": round(apply_bytes / (apply_ms * 1e-3) / 1e9, 1),
+            "apply_pass_hbm_frac": round(apply_bytes / (apply_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+
+
 def extra_ln(_C):
     """fused GEMM+LayerNorm at 4096^3 against the plain GEMM, each with the tile the library picks for it; and the
     same for a few other shapes (one round of small tiles, several rounds of large ones, ragged edges)."""
     out = ln_against_plain(_C, 4096, 4096, 4096)
-    out["other_shapes"] = [ln_against_plain(_C, *s) for s in ((2048, 2048, 2048), (8192, 8192, 4096), (3000, 5000, 2000))]
+    out["frac_of_mfma_peak"] = round(out["gemm_ln_TFLOPs"] / PEAK_TFLOPS, 4)
+    out.update(ln_two_pass(_C, 4096, 4096, 4096))
+    out["other_shapes"] = [ln_against_plain(_C, *s) for s in ((2048, 2048, 2048), (8192, 8192, 4096), (3000, 5000, 2000),
+                                                              (6144, 6144, 2048))]
+    return out
+
+
+def mfma_ceiling(_C, headline_tflops):
+    """What the matrix cores of THIS device sustain with operands in registers and no memory instruction at all
+    (beam_probe_mfma: one wavefront per SIMD, launches of about 0.7 ms like the headline kernel's), on operands of
+    the headline workload's distribution and on zeros, and the headline kernel's throughput as a fraction of it."""
+    out = {}
+    for key, dtype, shape, data in (("fp16_16x16x32_normal", _C.F16, _C.MFMA_16X16X32, _C.PROBE_NORMAL),
+                                    ("fp16_16x16x32_zeros", _C.F16, _C.MFMA_16X16X32, _C.PROBE_ZEROS),
+                                    ("fp16_32x32x16_normal", _C.F16, _C.MFMA_32X32X16, _C.PROBE_NORMAL),
+                                    ("bf16_16x16x32_normal", _C.BF16, _C.MFMA_16X16X32, _C.PROBE_NORMAL)):
+        _, tflops = _C.probe_mfma(dtype, shape, data, passes=1600, warmup=150, iters=200)
+        out[key + "_TFLOPs"] = round(tflops, 1)
+    out["ceiling_frac_of_peak"] = round(out["fp16_16x16x32_normal_TFLOPs"] / PEAK_TFLOPS, 4)
+    out["headline_over_ceiling"] = round(headline_tflops / out["fp16_16x16x32_normal_TFLOPs"], 4)
+    out["note"] = ("register-only MFMA loop on every SIMD; 'normal' = operands N(0,1)/sqrt(8192), the headline workload's "
+                   "distribution: the part is power limited on such data, zeros run at the full clock")
     return out
 
 
@@ -413,6 +451,21 @@ def main():
         del ref
     for x in (a, b, c):
         x.free()
+    if not args.no_extra:
+        try:
+            extra["mfma_ceiling"] = mfma_ceiling(_C, steady["TFLOPs"])
+        except Exception as e:  # noqa: BLE001
+            extra["mfma_ceiling"] = {"error": f"{type(e).__name__}: {e}"}
+        # the companion kernels against the roofline that bounds each (recomputable from the figures beside them)
+        sk, ln = extra.get("splitk", {}), extra.get("gemm_ln", {})
+        extra["rooflines"] = {
+            "splitk_256x256x32768": {"bound": "hbm", "us": sk.get("splitk_us"), "achieved_GBs": sk.get("hbm_GBs"),
+                                     "peak_GBs": HBM_PEAK_GBS, "frac": sk.get("hbm_frac"), "bytes": 2.0 * (256 * 32768 * 2 + 256 * 256)},
+            "gemm_ln_fused_4096cube": {"bound": "mfma", "us": ln.get("gemm_ln_us"), "achieved_TFLOPs": ln.get("gemm_ln_TFLOPs"),
+                                       "peak_TFLOPs": PEAK_TFLOPS, "frac": ln.get("frac_of_mfma_peak")},
+            "ln_apply_kernel_4096sq": {"bound": "hbm", "us": ln.get("apply_pass_us"), "achieved_GBs": ln.get("apply_pass_GBs"),
+                                       "peak_GBs": HBM_PEAK_GBS, "frac": ln.get("apply_pass_hbm_frac"), "bytes": 6.0 * 4096 * 4096 + 4.0 * 4096},
+        }
     out["extra"] = {"headline_steady": steady, **extra}
     print(json.dumps(out))
     if "check" in out and not out["check"]["ok"]:

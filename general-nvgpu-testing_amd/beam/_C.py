@@ -81,7 +81,7 @@ def _load() -> ctypes.CDLL:
     L.beam_gemmrc_splitk.argtypes = [vp, vp, vp, i, i, i, i, cfgp, i, vp, sz, vp]
     L.beam_splitk_effective.argtypes = [i, i, i, cfgp, i]
     L.beam_set_splitk_two_launches.argtypes = [i]
-    L.beam_gemmrc_splitk_timed_out.argtypes = [vp, i, i, i, vp, ctypes.POINTER(i)]
+    L.beam_gemmrc_splitk_timed_out.argtypes = [vp, sz, i, i, i, vp, ctypes.POINTER(i)]
     L.beam_splitk_noalloc_max_bytes.argtypes = []
     L.beam_splitk_noalloc_max_bytes.restype = sz
     L.beam_gemmrc_splitk_noalloc.argtypes = [vp, vp, vp, i, i, i, i, cfgp, i, vp]
@@ -93,6 +93,7 @@ def _load() -> ctypes.CDLL:
     L.beam_gemmrc_ln_workspace_bytes_for.argtypes = [i, i, i, cfgp, i]
     L.beam_gemmrc_ln_workspace_bytes_for.restype = sz
     L.beam_gemmrc_ln_ex.argtypes = [vp, vp, vp, vp, ctypes.c_float, vp, i, i, i, i, cfgp, i, vp, sz, vp]
+    L.beam_gemmrc_ln_checked.argtypes = [vp, vp, vp, vp, ctypes.c_float, vp, i, i, i, i, cfgp, vp, sz, vp, ctypes.POINTER(i)]
     L.beam_set_ln_spin_limit.argtypes = [i]
     L.beam_set_verbose.argtypes = [i]
     L.beam_gemmrc_ln_workspace_reset.argtypes = [vp]
@@ -120,6 +121,11 @@ def _load() -> ctypes.CDLL:
     L.beam_sync.argtypes = [vp]
     L.beam_host_fill_uniform.argtypes = [vp, sz, i, ctypes.c_uint64, ctypes.c_uint64]
     L.beam_host_fill_normal.argtypes = [vp, sz, i, ctypes.c_uint64, ctypes.c_uint64, ctypes.c_float, ctypes.c_float]
+    # test and measurement surface (include/beam_hip_debug.h)
+    L.beam_probe_mfma.argtypes = [i, i, i, i, i, i, vp, ctypes.POINTER(ctypes.c_float), ctypes.POINTER(ctypes.c_double)]
+    L.beam_dbg_ln_plan_bytes.argtypes = [i, i, i, cfgp, i, i, i, i]
+    L.beam_dbg_ln_plan_bytes.restype = sz
+    L.beam_dbg_assume_compute_units.argtypes = [i]
     L.beam_dbg_tile_of_workgroup.argtypes = [i, i, i, i, ctypes.POINTER(i), ctypes.POINTER(i)]
     L.beam_dbg_lds_offset.argtypes = [i, i]
     L.beam_dbg_kmajor_lds_offset.argtypes = [i, i, i]
@@ -355,7 +361,7 @@ def _splitk(a, b, c, cfgp, split_k_slices: int, check: bool = False) -> None:
                                   ws.ptr if ws else None, ws.nbytes if ws else 0, st))
     if check and ws is not None:
         flag = ctypes.c_int(0)
-        _check(lib.beam_gemmrc_splitk_timed_out(ws.ptr, M, N, s, st, ctypes.byref(flag)))
+        _check(lib.beam_gemmrc_splitk_timed_out(ws.ptr, ws.nbytes, M, N, s, st, ctypes.byref(flag)))
         if flag.value:
             raise BeamError(4, "split-K: a reducing workgroup gave up waiting for the slices of its tile; "
                                "the outputs concerned are NaN")
@@ -382,14 +388,19 @@ def gemmrc_splitk_spec(a, b, c, shape_threadblock=(128, 128), shape_warp=(64, 64
 
 
 LN_AUTO, LN_TWOPASS, LN_FUSED = 0, 1, 2
+# the library's default bound on the waits of its kernels (beam_set_ln_spin_limit), for code that changes and restores it
+DEFAULT_SPIN_LIMIT = 16384
 
 
 def gemmrc_ln(a, b, c, gamma, beta, eps: float = 1e-5, config: Optional[TileConfig] = None,
-              mode: int = LN_AUTO, check: bool = False) -> None:
+              mode: int = LN_AUTO, check: bool = True) -> bool:
     """c = LayerNorm_N(a @ b.T) * gamma + beta, statistics from the fp32 accumulators.
-    mode: LN_AUTO (fused single kernel when N / block_n <= 64), LN_TWOPASS, LN_FUSED.
-    check: wait for the result and raise BeamError if the fused kernel gave up waiting for a band (its
-    workgroups need the device to themselves; the rows concerned are NaN then)."""
+    mode: LN_AUTO (one kernel when N / block_n <= 64 on a 256-CU device, else two passes), LN_TWOPASS, LN_FUSED.
+    check (the default): wait for the result.  The workgroups of the one-kernel form wait for one another, boundedly,
+    which assumes that they have the device to themselves; when other work keeps the device occupied and that wait
+    runs out, LN_AUTO repeats the call as two passes (the return value is then True, and c is right either way) and
+    an explicit LN_FUSED raises BeamError.  check=False launches and returns at once, like the other operators: the
+    rows concerned are NaN if that ever happens, and gemmrc_ln_timed_out() tells."""
     pa, pb, pc, M, N, K, d, st = _problem(a, b, c)
     pg, sg, dg, _ = _describe(gamma)
     pbt, sbt, dbt, _ = _describe(beta)
@@ -397,15 +408,22 @@ def gemmrc_ln(a, b, c, gamma, beta, eps: float = 1e-5, config: Optional[TileConf
         raise BeamError(1, "gamma and beta must be [N] of the same dtype as a, b, c")
     cfg = config.to_c() if config is not None else None
     cfgp = ctypes.byref(cfg) if cfg else None
-    need = lib.beam_gemmrc_ln_workspace_bytes_for(M, N, K, cfgp, mode)
+    # operands aligned to an element only run on the plain kernels, which need room for an fp32 copy of the product
+    aligned = ((pa | pb | pc) & 15) == 0 and ((pg | pbt) & 7) == 0
+    need = lib.beam_gemmrc_ln_workspace_bytes_for(M, N, K, cfgp, mode) if aligned else lib.beam_gemmrc_ln_workspace_bytes_ex(M, N, cfgp, mode)
     ws = _get_ln_workspace(need)
+    if check and mode == LN_AUTO:
+        fell_back = ctypes.c_int(0)
+        _check(lib.beam_gemmrc_ln_checked(pa, pb, pg, pbt, eps, pc, M, N, K, d, cfgp, ws.ptr, ws.nbytes, st, ctypes.byref(fell_back)))
+        return bool(fell_back.value)
     _check(lib.beam_gemmrc_ln_ex(pa, pb, pg, pbt, eps, pc, M, N, K, d, cfgp, mode, ws.ptr, ws.nbytes, st))
     if check:
         flag = ctypes.c_int(0)
         _check(lib.beam_gemmrc_ln_timed_out(ws.ptr, st, ctypes.byref(flag)))
         if flag.value:
             raise BeamError(4, "fused GEMM+LayerNorm gave up waiting for a band of workgroups (device shared with "
-                               "other work?); use mode=LN_TWOPASS")
+                               "other work?); use mode=LN_AUTO or LN_TWOPASS")
+    return False
 
 
 def gemmrc_ln_timed_out() -> bool:
@@ -502,6 +520,7 @@ cutlass_parallel_gemmrc_lnr = parallel_gemmrc_silu
 OP_GEMM, OP_SPLITK, OP_GEMM_LN, OP_GEMM_SILU, OP_SILU, OP_MATMUL_NN = 0, 1, 2, 3, 4, 5
 # launches that measure what the machine allows: an empty kernel, two of them, a split-K launch with only its loads
 OP_PROBE_EMPTY, OP_PROBE_EMPTY_PAIR, OP_PROBE_SPLITK_LOADS = 6, 7, 8
+OP_PROBE_LN_APPLY = 9  # the normalisation pass of a two-pass GEMM+LayerNorm alone (after such a call on the shared workspace)
 
 
 def bench(op: int, a, b, c, config: Optional[TileConfig] = None, split_k: int = 0, gamma=None, beta=None,
@@ -526,14 +545,28 @@ def bench(op: int, a, b, c, config: Optional[TileConfig] = None, split_k: int = 
         if s < 0:
             raise BeamError(2, lib.beam_last_error().decode())
         ws = _get_workspace(max(lib.beam_splitk_workspace_bytes(M, N, s), 1))
-    elif op == 2:
+    elif op in (OP_GEMM_LN, OP_PROBE_LN_APPLY):
         q.gamma, q.beta = _describe(gamma)[0], _describe(beta)[0]
-        ws = _get_ln_workspace(lib.beam_gemmrc_ln_workspace_bytes_for(M, N, K, cfgp, ln_mode))
+        ws = _get_ln_workspace(lib.beam_gemmrc_ln_workspace_bytes_for(M, N, K, cfgp, LN_TWOPASS if op == OP_PROBE_LN_APPLY else ln_mode))
     if ws is not None:
         q.ws, q.ws_bytes = ws.ptr, ws.nbytes
     ms = ctypes.c_float()
     _check(lib.beam_bench(op, ctypes.byref(q), cfgp, warmup, iters, st, ctypes.byref(ms)))
     return ms.value
+
+
+MFMA_16X16X32, MFMA_32X32X16 = 0, 1
+PROBE_NORMAL, PROBE_ZEROS = 0, 1
+
+
+def probe_mfma(dtype: int = F16, mfma_shape: int = MFMA_16X16X32, data: int = PROBE_NORMAL, passes: int = 1600,
+               warmup: int = 100, iters: int = 200):
+    """(milliseconds per launch, TFLOP/s) of the register-only matrix-core loop: every SIMD of the device issues
+    passes x 1024 cycles of MFMAs on operands that sit in registers, no memory instruction at all.  What the
+    matrix cores sustain on that data at the clock the power cap allows."""
+    ms, flop = ctypes.c_float(), ctypes.c_double()
+    _check(lib.beam_probe_mfma(dtype, mfma_shape, data, passes, warmup, iters, None, ctypes.byref(ms), ctypes.byref(flop)))
+    return ms.value, flop.value / (ms.value * 1e-3) / 1e12
 
 
 def do_bench(fn, warmup: int = 5, rep: int = 20, stream=None) -> float:

@@ -9,7 +9,8 @@
 namespace beam {
 
 // C[mn] (16-bit) = sum over `splits` fp32 slices of ws[splits][mn], added in slice order.
-hipError_t launch_splitk_reduce(const float* ws, void* C, size_t mn, int splits, int dtype,
+// sync_header, if not null: the synchronisation words of a split-K workspace; their "latest launch" word is cleared.
+hipError_t launch_splitk_reduce(const float* ws, void* C, size_t mn, int splits, int dtype, int* sync_header,
                                 hipStream_t stream);
 
 // Y[M][N] (16-bit) = normalise fp32 X[M][N] with per-(row, column tile) (mean, M2) pairs.

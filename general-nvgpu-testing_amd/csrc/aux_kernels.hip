@@ -25,8 +25,10 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 // CUTLASS's reduce kernel, cuda/cutlass_kernels/cutlass_gemmrc_splitk.cu:73-75).
 template <typename T>
 __global__ void __launch_bounds__(64) splitk_reduce_kernel(const float* __restrict__ ws, T* __restrict__ C,
-                                                            size_t mn, int splits) {
+                                                            size_t mn, int splits, int* sync_header) {
   typedef typename Vec4Of<T>::type vec4;
+  // the latest call on this workspace is not a one-launch one: whatever time-out its header records is not this call's
+  if (sync_header != nullptr && blockIdx.x == 0 && threadIdx.x == 0) sync_header[kSkLaunchTag] = 0;
   const size_t quads = mn / 4;
   const size_t stride = (size_t)gridDim.x * blockDim.x;
   for (size_t q = (size_t)blockIdx.x * blockDim.x + threadIdx.x; q < quads; q += stride) {
@@ -320,7 +322,7 @@ hipError_t launch_zero_ints(int* ints, int n, hipStream_t stream) {
   return hipGetLastError();
 }
 
-hipError_t launch_splitk_reduce(const float* ws, void* C, size_t mn, int splits, int dtype,
+hipError_t launch_splitk_reduce(const float* ws, void* C, size_t mn, int splits, int dtype, int* sync_header,
                                 hipStream_t stream) {
   // one wavefront per workgroup: even a 256 x 256 output spreads over 256 CUs
   size_t quads = (mn + 3) / 4;
@@ -329,10 +331,10 @@ hipError_t launch_splitk_reduce(const float* ws, void* C, size_t mn, int splits,
   if (blocks > 16384) blocks = 16384;
   if (dtype == BEAM_BF16)
     hipLaunchKernelGGL(splitk_reduce_kernel<__bf16>, dim3((unsigned)blocks), dim3(64), 0, stream, ws,
-                       (__bf16*)C, mn, splits);
+                       (__bf16*)C, mn, splits, sync_header);
   else
     hipLaunchKernelGGL(splitk_reduce_kernel<_Float16>, dim3((unsigned)blocks), dim3(64), 0, stream, ws,
-                       (_Float16*)C, mn, splits);
+                       (_Float16*)C, mn, splits, sync_header);
   return hipGetLastError();
 }
 

@@ -16,7 +16,7 @@
 
 #include <unistd.h>
 
-#include "../../include/beam_hip.h"
+#include "../../include/beam_hip_debug.h"
 #include "aux_kernels.h"
 #include "kernel_set.h"
 #include "tile_map.h"
@@ -54,8 +54,12 @@ struct Device {
 };
 Device g_dev;
 std::mutex g_dev_mu;
-// polls of statistics slots (about a microsecond each) before a thread of a fused LayerNorm workgroup gives up
-std::atomic<int> g_ln_spin_limit{4 << 20};
+// Polls before a waiting thread gives up: of statistics slots in the fused LayerNorm (3-4 us each once the pauses
+// between tries have grown: about 60 ms), of a tile's flags in the one-launch split-K (about 1 us each).  What a
+// workgroup legitimately waits for is resident with it and at most a tile's K loop behind, so the bound is there
+// for a device that other work keeps occupied: giving up then costs milliseconds, and the caller's retry as two
+// passes (beam_gemmrc_ln_checked) gives the result.
+std::atomic<int> g_ln_spin_limit{16384};
 // Nonces of fused GEMM+LayerNorm and one-launch split-K launches: consecutive numbers from a start that differs from process to process
 // (memory recycled from another process of this library then holds tags of another sequence).
 std::atomic<unsigned> g_ln_nonce{(unsigned)std::chrono::steady_clock::now().time_since_epoch().count() * 2654435761u ^
@@ -751,15 +755,24 @@ int beam_gemmrc_splitk(const void* A, const void* B, void* C, int M, int N, int 
     }
   }
   BEAM_HIP(ks->launch[dtype][kEpiPartial][c.pipeline](p, dim3((unsigned)(p.tiles_m * p.tiles_n * s), 1, 1), st));
-  BEAM_HIP(launch_splitk_reduce((const float*)ws, C, (size_t)M * N, s, dtype, st));
+  // Where the workspace has synchronisation words, the reduce kernel marks them "no one-launch call is the latest":
+  // a time-out recorded by an earlier one-launch call on this workspace must not be read as this call's.
+  const size_t hdr_at = align_up(need, 256);
+  int* hdr = ws_bytes >= hdr_at + 4 * (size_t)kSkFlags ? (int*)((char*)ws + hdr_at) : nullptr;
+  BEAM_HIP(launch_splitk_reduce((const float*)ws, C, (size_t)M * N, s, dtype, hdr, st));
   return BEAM_OK;
 }
 
-int beam_gemmrc_splitk_timed_out(const void* ws, int M, int N, int split_k_effective, void* stream, int* timed_out) {
-  if (!ws || !timed_out || M <= 0 || N <= 0 || split_k_effective < 1) return fail(BEAM_ERR_INVALID, "bad argument");
+int beam_gemmrc_splitk_timed_out(const void* ws, size_t ws_bytes, int M, int N, int split_k_effective, void* stream,
+                                 int* timed_out) {
+  if (!timed_out || M <= 0 || N <= 0 || split_k_effective < 1) return fail(BEAM_ERR_INVALID, "bad argument");
+  *timed_out = 0;
   BEAM_HIP(hipStreamSynchronize((hipStream_t)stream));
   int hdr[4] = {0, 0, 0, 0};
   const size_t sync_at = align_up(splitk_partial_bytes(M, N, split_k_effective), 256);
+  // One slice, or a workspace that ends with the partial sums: the call had no waiting workgroups (plain kernel, or
+  // partial + reduce kernel), and there are no synchronisation words to read.
+  if (!ws || split_k_effective == 1 || ws_bytes < sync_at + sizeof hdr) return BEAM_OK;
   BEAM_HIP(hipMemcpy(hdr, (const char*)ws + sync_at, sizeof hdr, hipMemcpyDeviceToHost));
   *timed_out = hdr[kSkMagic] == kSkMagicValue && hdr[kSkLaunchTag] != 0 && hdr[kSkTimeout] == hdr[kSkLaunchTag];
   return BEAM_OK;
@@ -771,7 +784,9 @@ int beam_gemmrc_splitk_noalloc(const void* A, const void* B, void* C, int M, int
                                const beam_tile_cfg* cfg, int split_k, void* stream) {
   int rc = beam_init();
   if (rc) return rc;
-  if (M > 0 && N > 0 && K > 0) {
+  bool generic = false;
+  if ((rc = check_problem(A, B, C, M, N, K, dtype, &generic))) return rc;
+  if (M > 0 && N > 0 && K > 0 && !generic) {  // (the plain kernel, one pass, needs no workspace)
     const int s = beam_splitk_effective(M, N, K, cfg, split_k);
     if (s < 0) return BEAM_ERR_UNSUPPORTED;  // the message is already set
     const size_t need = s > 1 ? splitk_partial_bytes(M, N, s) : 0;
@@ -880,39 +895,103 @@ static int ln_resolve_cfg(const beam_tile_cfg* cfg, int M, int N, int K, int mod
   return BEAM_OK;
 }
 
+// What a GEMM+LayerNorm call does and the workspace it needs: one function, so that the entry point and the
+// workspace queries cannot disagree.
+//   plain     the problem is outside what the tiled kernels take (K % 8, K beyond a descriptor, operands aligned to
+//             an element only): plain GEMM into fp32 X, then a row-wise LayerNorm
+//   capturing the stream is being captured: AUTO then means two passes (a replayed graph may share the device with
+//             other work, which the fused kernel's residency argument does not cover); an explicit FUSED is honoured
+//   wide_io   Y, gamma and beta are 16-byte aligned (the 4-wavefront kernel's vector accesses)
+struct LnPlan {
+  enum Kind { kPlain, kTwoPass, kFused } kind;
+  beam_tile_cfg c;
+  const KernelSet* ks;
+  bool w4;  // fused, on the kernel of gemm_w4.h
+  size_t need;
+};
+static int ln_plan(int M, int N, int K, const beam_tile_cfg* cfg, int mode, bool plain, bool capturing, bool wide_io, LnPlan* out) {
+  out->ks = nullptr;
+  out->w4 = false;
+  if (plain) {
+    out->kind = LnPlan::kPlain;
+    out->need = ln_generic_need(M, N);
+    return BEAM_OK;
+  }
+  if (capturing && mode == BEAM_LN_AUTO) mode = BEAM_LN_TWOPASS;
+  int rc = ln_resolve_cfg(cfg, M, N, K, mode, &out->c, &out->ks);
+  if (rc) return rc;
+  beam_tile_cfg& c = out->c;
+  if (mode == BEAM_LN_FUSED && !ln_fused_applies(c, *out->ks, N))
+    return fail(BEAM_ERR_UNSUPPORTED, "fused LayerNorm: needs a device of %d CUs and at most 64 column tiles (N=%d, block_n=%d, %d CUs)",
+                kNumXcd * 32, N, c.block_n, g_dev.cus);
+  mode = ln_resolve_mode(mode, c, *out->ks, N);
+  // The 256 x 256 tile runs on the kernel of gemm_w4.h where that one's preconditions hold (asked for by
+  // name, or as the library's own choice); where they do not, the library's own choice falls back to the
+  // 8-wavefront tile of the same shape.
+  const bool w4_fits = mode == BEAM_LN_FUSED && c.pipeline == 0 && c.block_m == 256 && c.block_n == 256 && K % kBK == 0 &&
+                       K >= kW4MinK && N % 8 == 0 && N <= (1 << 21) && wide_io;
+  if (!cfg && !w4_fits && c.block_m == 256 && c.block_n == 256 && c.wave_m == 128 && c.wave_n == 128) {
+    c.wave_n = 64;
+    if ((rc = resolve_cfg(&c, M, N, K, &c, &out->ks))) return rc;
+  }
+  out->w4 = w4_fits && (!cfg || (c.wave_m == 128 && c.wave_n == 128));
+  out->kind = mode == BEAM_LN_FUSED ? LnPlan::kFused : LnPlan::kTwoPass;
+  out->need = ln_workspace_need(M, N, c, mode);
+  return BEAM_OK;
+}
+
+// Enough for beam_gemmrc_ln_ex(M, N, K, cfg, mode) on operands aligned as the tiled kernels need them.  AUTO covers
+// both forms it can resolve to (one kernel eagerly, two passes under stream capture and as the retry of
+// beam_gemmrc_ln_checked), which also covers the plain path.
 size_t beam_gemmrc_ln_workspace_bytes_for(int M, int N, int K, const beam_tile_cfg* cfg, int mode) {
   if (M <= 0 || N <= 0 || K < 0) return 0;
   if (K % 8 != 0 || K > kMaxK) return ln_generic_need(M, N);
   (void)beam_init();  // AUTO depends on the device
-  beam_tile_cfg c;
-  const KernelSet* ks;
-  if (ln_resolve_cfg(cfg, M, N, K, mode, &c, &ks)) return 0;
-  return ln_workspace_need(M, N, c, ln_resolve_mode(mode, c, *ks, N));
+  LnPlan eager, captured;
+  if (ln_plan(M, N, K, cfg, mode, false, false, true, &eager)) return 0;
+  if (mode != BEAM_LN_AUTO) return eager.need;
+  if (ln_plan(M, N, K, cfg, mode, false, true, true, &captured)) return eager.need;
+  return eager.need > captured.need ? eager.need : captured.need;
 }
 
+// Enough for any call with these M, N, cfg and mode: every K, every alignment, captured or not.
 size_t beam_gemmrc_ln_workspace_bytes_ex(int M, int N, const beam_tile_cfg* cfg, int mode) {
   if (M <= 0 || N <= 0) return 0;
-  // a given tile does not depend on K (but a problem the tiled kernels refuse -- odd K, odd addresses -- needs fp32 X)
+  size_t need = ln_generic_need(M, N);  // K % 8 != 0, operands aligned to an element only
+  auto take = [&](size_t n) { need = n > need ? n : need; };
+  // a given tile does not depend on K
   if (cfg) {
-    const size_t tiled = beam_gemmrc_ln_workspace_bytes_for(M, N, 64, cfg, mode), plain = ln_generic_need(M, N);
-    return tiled > plain ? tiled : plain;
+    take(beam_gemmrc_ln_workspace_bytes_for(M, N, 64, cfg, mode));
+    return need;
   }
   // Without a tile the library picks one from (M, N, K), and K is not known here: the largest need over
-  // every tile it can pick.
+  // every tile it can pick, in every form `mode` can resolve to.
   (void)beam_init();
-  size_t need = 0;
   for (int i = 0; i < beam_num_configs(); ++i) {
     beam_tile_cfg c;
     const KernelSet* ks;
     if (beam_get_config(i, &c) || resolve_cfg(&c, M, N, 64, &c, &ks)) continue;
-    const size_t n = ln_workspace_need(M, N, c, ln_resolve_mode(mode, c, *ks, N));
-    need = n > need ? n : need;
+    take(ln_workspace_need(M, N, c, ln_resolve_mode(mode, c, *ks, N)));
+    if (mode == BEAM_LN_AUTO) take(ln_workspace_need(M, N, c, BEAM_LN_TWOPASS));
   }
   return need;
 }
 
 size_t beam_gemmrc_ln_workspace_bytes(int M, int N, const beam_tile_cfg* cfg) {
   return beam_gemmrc_ln_workspace_bytes_ex(M, N, cfg, BEAM_LN_AUTO);
+}
+
+size_t beam_dbg_ln_plan_bytes(int M, int N, int K, const beam_tile_cfg* cfg, int mode, int plain, int capturing, int wide_io) {
+  LnPlan plan;
+  if (M <= 0 || N <= 0 || K < 0 || ln_plan(M, N, K, cfg, mode, plain != 0 || K % 8 != 0 || K > kMaxK, capturing != 0, wide_io != 0, &plan)) return 0;
+  return plan.need;
+}
+
+int beam_dbg_assume_compute_units(int compute_units) {
+  std::lock_guard<std::mutex> lk(g_dev_mu);
+  if (g_dev.status == BEAM_OK) return fail(BEAM_ERR_INVALID, "a device has been probed: its own CU count stands");
+  g_dev.cus = compute_units;
+  return BEAM_OK;
 }
 
 int beam_gemmrc_ln_ex(const void* A, const void* B, const void* gamma, const void* beta, float eps, void* Y,
@@ -928,47 +1007,29 @@ int beam_gemmrc_ln_ex(const void* A, const void* B, const void* gamma, const voi
   if (mode < BEAM_LN_AUTO || mode > BEAM_LN_FUSED) return fail(BEAM_ERR_INVALID, "unknown LayerNorm mode %d", mode);
   if ((rc = beam_init())) return rc;
   hipStream_t st = (hipStream_t)stream;
-  if (ln_is_generic(generic, gamma, beta)) {
+  hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+  if (st != nullptr) (void)hipStreamIsCapturing(st, &capturing);
+  LnPlan plan;
+  if ((rc = ln_plan(M, N, K, cfg, mode, ln_is_generic(generic, gamma, beta), capturing != hipStreamCaptureStatusNone,
+                    (((uintptr_t)Y | (uintptr_t)gamma | (uintptr_t)beta) & 15) == 0, &plan)))
+    return rc;
+  const size_t need = plan.need;
+  if (!ws || ws_bytes < need)
+    return fail(BEAM_ERR_WORKSPACE, "GEMM+LayerNorm needs %zu bytes of workspace, got %zu", need, ws_bytes);
+  if (plan.kind == LnPlan::kPlain) {
     // What the tiled kernels cannot take: the plain GEMM into fp32 X, then a row-wise LayerNorm (whatever mode was named).
-    const size_t need = ln_generic_need(M, N);
-    if (!ws || ws_bytes < need)
-      return fail(BEAM_ERR_WORKSPACE, "GEMM+LayerNorm needs %zu bytes of workspace, got %zu", need, ws_bytes);
     if ((uintptr_t)ws & 15) return fail(BEAM_ERR_UNSUPPORTED, "workspace must be 16-byte aligned");
     if (K == 0) BEAM_HIP(launch_fill_floats((float*)ws, (size_t)M * N, 0.0f, st));
     else BEAM_HIP(launch_generic_gemm(A, B, ws, M, N, K, dtype, false, true, st));
     BEAM_HIP(launch_ln_rows((const float*)ws, gamma, beta, Y, M, N, eps, dtype, st));
     return BEAM_OK;
   }
-  // The fused kernel's workgroups wait for one another; whether a replayed graph meets the residency that
-  // wait relies on (other graph branches may share the device) is the caller's business: under stream
-  // capture AUTO takes the two-pass path, an explicit FUSED is honoured.
-  hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
-  if (st != nullptr) (void)hipStreamIsCapturing(st, &capturing);
-  if (capturing != hipStreamCaptureStatusNone && mode == BEAM_LN_AUTO) mode = BEAM_LN_TWOPASS;
-  beam_tile_cfg c;
-  const KernelSet* ks;
-  if ((rc = ln_resolve_cfg(cfg, M, N, K, mode, &c, &ks))) return rc;
-  if (mode == BEAM_LN_FUSED && !ln_fused_applies(c, *ks, N))
-    return fail(BEAM_ERR_UNSUPPORTED, "fused LayerNorm: needs a device of %d CUs and at most 64 column tiles (N=%d, block_n=%d, %d CUs)",
-                kNumXcd * 32, N, c.block_n, g_dev.cus);
-  mode = ln_resolve_mode(mode, c, *ks, N);
-  // The 256 x 256 tile runs on the kernel of gemm_w4.h where that one's preconditions hold (asked for by
-  // name, or as the library's own choice); where they do not, the library's own choice falls back to the
-  // 8-wavefront tile of the same shape.
-  const bool w4_fits = mode == BEAM_LN_FUSED && c.pipeline == 0 && c.block_m == 256 && c.block_n == 256 && K % kBK == 0 &&
-                       K >= kW4MinK && N % 8 == 0 && N <= (1 << 21) &&
-                       (((uintptr_t)Y | (uintptr_t)gamma | (uintptr_t)beta) & 15) == 0;
-  if (!cfg && !w4_fits && c.block_m == 256 && c.block_n == 256 && c.wave_m == 128 && c.wave_n == 128) {
-    c.wave_n = 64;
-    if ((rc = resolve_cfg(&c, M, N, K, &c, &ks))) return rc;
-  }
-  const size_t need = ln_workspace_need(M, N, c, mode);
-  if (!ws || ws_bytes < need)
-    return fail(BEAM_ERR_WORKSPACE, "GEMM+LayerNorm needs %zu bytes of workspace, got %zu", need, ws_bytes);
   if ((uintptr_t)ws & 255) return fail(BEAM_ERR_UNSUPPORTED, "workspace must be 256-byte aligned");
+  const beam_tile_cfg& c = plan.c;
+  const KernelSet* ks = plan.ks;
   GemmParams p = base_params(A, B, M, N, K, c);
   // K == 0: the kernels run with an empty K range and produce x = 0, i.e. y = beta.
-  if (mode == BEAM_LN_FUSED) {
+  if (plan.kind == LnPlan::kFused) {
     p.C = Y;
     // Launches that share a workspace must be ordered (same stream): overlapping ones would race on the sets.
     const size_t set_bytes = ln_fused_set_bytes(p.tiles_m, p.tiles_n, c.block_m);
@@ -1018,7 +1079,7 @@ int beam_gemmrc_ln_ex(const void* A, const void* B, const void* gamma, const voi
     } else {
       grid = (unsigned)band_block_grid(p.tiles_m, p.group_m, p.group_n);
     }
-    if (w4_fits && (!cfg || (c.wave_m == 128 && c.wave_n == 128))) {
+    if (plan.w4) {
       BEAM_HIP(launch_gemm_w4_ln(p, dtype, dim3(grid, 1, 1), st));
       return BEAM_OK;
     }
@@ -1038,9 +1099,38 @@ int beam_gemmrc_ln(const void* A, const void* B, const void* gamma, const void* 
   return beam_gemmrc_ln_ex(A, B, gamma, beta, eps, Y, M, N, K, dtype, cfg, BEAM_LN_AUTO, ws, ws_bytes, stream);
 }
 
+int beam_gemmrc_ln_checked(const void* A, const void* B, const void* gamma, const void* beta, float eps, void* Y,
+                           int M, int N, int K, int dtype, const beam_tile_cfg* cfg, void* ws, size_t ws_bytes,
+                           void* stream, int* fell_back) {
+  if (fell_back) *fell_back = 0;
+  hipStream_t st = (hipStream_t)stream;
+  hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+  if (st != nullptr) (void)hipStreamIsCapturing(st, &capturing);
+  // (captured: AUTO is two passes, which wait for nothing; a stream being captured cannot be waited for anyway)
+  int rc = beam_gemmrc_ln_ex(A, B, gamma, beta, eps, Y, M, N, K, dtype, cfg, BEAM_LN_AUTO, ws, ws_bytes, stream);
+  if (rc || capturing != hipStreamCaptureStatusNone || M == 0 || N == 0) return rc;
+  bool generic;
+  (void)check_problem(A, B, Y, M, N, K, dtype, &generic);
+  LnPlan plan;
+  if (ln_plan(M, N, K, cfg, BEAM_LN_AUTO, ln_is_generic(generic, gamma, beta), false,
+              (((uintptr_t)Y | (uintptr_t)gamma | (uintptr_t)beta) & 15) == 0, &plan) || plan.kind != LnPlan::kFused)
+    return BEAM_OK;  // nothing in the call waits for anything
+  int timed_out = 0;
+  if ((rc = beam_gemmrc_ln_timed_out(ws, stream, &timed_out))) return rc;
+  if (!timed_out) return BEAM_OK;
+  if (fell_back) *fell_back = 1;
+  if ((rc = beam_gemmrc_ln_ex(A, B, gamma, beta, eps, Y, M, N, K, dtype, cfg, BEAM_LN_TWOPASS, ws, ws_bytes, stream))) return rc;
+  BEAM_HIP(hipStreamSynchronize(st));
+  return BEAM_OK;
+}
+
 int beam_gemmrc_ln_workspace_reset(const void* ws) {
   if (!ws) return fail(BEAM_ERR_INVALID, "null workspace");
-  BEAM_HIP(hipMemset(const_cast<void*>(ws), 0, ln_fused_header_bytes()));  // forgets a recorded time-out; never needed
+  // Forgets a recorded time-out (never needed).  The replay counter behind these words stays: it is part of the tag
+  // of captured launches, and a counter that went back could hand a replay the tag of an earlier one, whose
+  // statistics words would then pass for published.
+  static_assert(kLnHdrTimeout < 3 && kLnHdrMagic < 3 && kLnHdrLaunchTag < 3 && kLnHdrReplay == 3, "header words");
+  BEAM_HIP(hipMemset(const_cast<void*>(ws), 0, 3 * sizeof(int)));
   return BEAM_OK;
 }
 
@@ -1113,6 +1203,18 @@ int beam_bench(int op, const beam_problem* q, const beam_tile_cfg* cfg, int warm
       }
       case BEAM_OP_PROBE_SPLITK_LOADS:
         return probe_splitk_loads(q, cfg, (hipStream_t)stream);
+      case BEAM_OP_PROBE_LN_APPLY: {
+        // the second kernel of a two-pass GEMM+LayerNorm alone, on the fp32 X and statistics a two-pass call left in ws
+        int rc = beam_init();
+        if (rc) return rc;
+        LnPlan plan;
+        if ((rc = ln_plan(q->M, q->N, q->K, cfg, BEAM_LN_TWOPASS, q->K % 8 != 0 || q->K > kMaxK, false, true, &plan))) return rc;
+        if (plan.kind != LnPlan::kTwoPass || !q->ws || q->ws_bytes < plan.need) return fail(BEAM_ERR_WORKSPACE, "needs the workspace of a two-pass call");
+        const float* stats = (const float*)((const char*)q->ws + align_up((size_t)q->M * q->N * sizeof(float), 256));
+        BEAM_HIP(launch_ln_apply((const float*)q->ws, stats, q->gamma, q->beta, q->C, q->M, q->N, (q->N + plan.c.block_n - 1) / plan.c.block_n,
+                                 plan.c.block_n, q->eps, q->dtype, (hipStream_t)stream));
+        return BEAM_OK;
+      }
       default:
         return fail(BEAM_ERR_INVALID, "unknown op %d", op);
     }
@@ -1137,6 +1239,34 @@ int beam_bench(int op, const beam_problem* q, const beam_tile_cfg* cfg, int warm
   if (rc) return rc;
   if (he != hipSuccess) return hip_fail(he, "event timing");
   *avg_ms = ms / (float)iters;
+  return BEAM_OK;
+}
+
+int beam_probe_mfma(int dtype, int mfma_shape, int data, int passes, int warmup, int iters, void* stream, float* avg_ms,
+                    double* flop_per_launch) {
+  if (!avg_ms || iters < 1 || warmup < 0 || passes < 1) return fail(BEAM_ERR_INVALID, "bad probe arguments");
+  if (dtype != BEAM_F16 && dtype != BEAM_BF16) return fail(BEAM_ERR_UNSUPPORTED, "dtype %d: only fp16 (0) and bf16 (1)", dtype);
+  if (mfma_shape != BEAM_MFMA_16X16X32 && mfma_shape != BEAM_MFMA_32X32X16) return fail(BEAM_ERR_INVALID, "unknown MFMA shape %d", mfma_shape);
+  if (data != BEAM_PROBE_DATA_NORMAL && data != BEAM_PROBE_DATA_ZEROS) return fail(BEAM_ERR_INVALID, "unknown data kind %d", data);
+  int rc = beam_init();
+  if (rc) return rc;
+  const int cus = g_dev.cus > 0 && g_dev.cus <= 1024 ? g_dev.cus : 256;
+  hipStream_t st = (hipStream_t)stream;
+  for (int i = 0; i < warmup; ++i) BEAM_HIP(launch_probe_mfma(dtype, mfma_shape, cus, passes, data == BEAM_PROBE_DATA_ZEROS, st));
+  hipEvent_t e0, e1;
+  BEAM_HIP(hipEventCreate(&e0));
+  BEAM_HIP(hipEventCreate(&e1));
+  hipError_t he = hipEventRecord(e0, st);
+  for (int i = 0; i < iters && he == hipSuccess; ++i) he = launch_probe_mfma(dtype, mfma_shape, cus, passes, data == BEAM_PROBE_DATA_ZEROS, st);
+  if (he == hipSuccess) he = hipEventRecord(e1, st);
+  if (he == hipSuccess) he = hipEventSynchronize(e1);
+  float ms = 0.0f;
+  if (he == hipSuccess) he = hipEventElapsedTime(&ms, e0, e1);
+  (void)hipEventDestroy(e0);
+  (void)hipEventDestroy(e1);
+  if (he != hipSuccess) return hip_fail(he, "matrix-core probe");
+  *avg_ms = ms / (float)iters;
+  if (flop_per_launch) *flop_per_launch = (double)cus * 4.0 * (double)passes * 1024.0 * 1024.0;
   return BEAM_OK;
 }
 

@@ -7,13 +7,8 @@ namespace beam {
 template <typename T, bool C_NT, bool LN = false>
 static hipError_t launch_w4_t(const GemmParams& p, dim3 grid, hipStream_t stream) {
   auto kern = gemmrc_w4_kernel<T, C_NT, LN>;
-  static bool configured = false;  // benign race: the attribute call is idempotent
-  if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       GemmW4<T>::LDS_BYTES);
-    if (e != hipSuccess) return e;
-    configured = true;
-  }
+  static std::atomic<unsigned long long> configured{0};
+  if (hipError_t e = allow_lds_once(configured, reinterpret_cast<const void*>(kern), GemmW4<T>::LDS_BYTES); e != hipSuccess) return e;
   hipLaunchKernelGGL(kern, grid, dim3(GemmW4<T>::NT), GemmW4<T>::LDS_BYTES, stream, p);
   return hipGetLastError();
 }

@@ -8,13 +8,8 @@ template <typename T, bool C_NT>
 static hipError_t launch_w4_kmajor_t(const GemmParams& p, dim3 grid, hipStream_t stream) {
   using Tile = GemmW4<T, C_NT, false, 4, 8, 2, true>;
   auto kern = gemmrc_w4_kernel<T, C_NT, false, 4, 8, 2, true>;
-  static bool configured = false;  // benign race: the attribute call is idempotent
-  if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       Tile::LDS_BYTES);
-    if (e != hipSuccess) return e;
-    configured = true;
-  }
+  static std::atomic<unsigned long long> configured{0};
+  if (hipError_t e = allow_lds_once(configured, reinterpret_cast<const void*>(kern), Tile::LDS_BYTES); e != hipSuccess) return e;
   hipLaunchKernelGGL(kern, grid, dim3(Tile::NT), Tile::LDS_BYTES, stream, p);
   return hipGetLastError();
 }

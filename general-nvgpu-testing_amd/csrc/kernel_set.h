@@ -4,6 +4,8 @@
 
 #include <hip/hip_runtime.h>
 
+#include <atomic>
+
 #include "../../include/beam_hip.h"
 #include "gemm_kernel.h"
 
@@ -26,17 +28,27 @@ struct KernelSet {
   GemmLauncher launch_partial_fused[2][3];
 };
 
+// Raises a kernel's dynamic LDS limit on the current device the first time the kernel is launched there: the
+// attribute is a property of (kernel, device), so `done` keeps one bit per device index.  (A race between two
+// first launches is benign: the call is idempotent.)
+inline hipError_t allow_lds_once(std::atomic<unsigned long long>& done, const void* kern, int lds_bytes) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  const unsigned long long bit = 1ull << (dev & 63);
+  if (done.load(std::memory_order_acquire) & bit) return hipSuccess;
+  e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+  if (e != hipSuccess) return e;
+  done.fetch_or(bit, std::memory_order_release);
+  return hipSuccess;
+}
+
 template <typename T, int BM, int BN, int WVM, int WVN, int EPI, int AST, int BST, bool B_KMAJOR = false>
 hipError_t launch_gemm(const GemmParams& p, dim3 grid, hipStream_t stream) {
   using Tile = GemmTile<T, BM, BN, WVM, WVN, EPI, AST, BST, B_KMAJOR>;
   auto kern = gemmrc_kernel<T, BM, BN, WVM, WVN, EPI, AST, BST, B_KMAJOR>;
-  static bool configured = false;  // benign race: the attribute call is idempotent
-  if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, Tile::LDS_BYTES);
-    if (e != hipSuccess) return e;
-    configured = true;
-  }
+  static std::atomic<unsigned long long> configured{0};
+  if (hipError_t e = allow_lds_once(configured, reinterpret_cast<const void*>(kern), Tile::LDS_BYTES); e != hipSuccess) return e;
   hipLaunchKernelGGL(kern, grid, dim3(Tile::NT), Tile::LDS_BYTES, stream, p);
   return hipGetLastError();
 }
@@ -141,5 +153,8 @@ hipError_t launch_gemm_w4_ln(const GemmParams& p, int dtype, dim3 grid, hipStrea
 // pipeline, fp16, with its loads and fragment reads but no MFMAs and no stores (kEpiProbeLoads); hipErrorInvalidValue
 // for any other tile.
 hipError_t launch_probe_splitk_loads(const GemmParams& p, int block_m, int block_n, dim3 grid, hipStream_t stream);
+// Measurement only: `workgroups` (<= 1024) x 4 wavefronts, each issuing passes x 1024 matrix-core cycles of MFMAs on
+// operands in registers (mfma_shape 0: 16x16x32, 1: 32x32x16; zeros: all-zero operands instead of N(0,1)/sqrt(8192)).
+hipError_t launch_probe_mfma(int dtype, int mfma_shape, int workgroups, int passes, int zeros, hipStream_t stream);
 
 }  // namespace beam

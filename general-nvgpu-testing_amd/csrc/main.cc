@@ -20,6 +20,10 @@
 //             [--ln-mode auto|twopass|fused]   (--op ln)
 //             --op probe-empty | probe-empty-pair | probe-splitk-loads: launches that measure what the machine
 //             allows (an empty kernel, two of them, the split-K partial kernel with nothing but its loads)
+//             --op probe-mfma [--dtype fp16|bf16] [--mfma 16x16x32|32x32x16] [--data normal|zeros] [--passes P]
+//             [--seconds S]: a register-only loop of MFMAs on every SIMD (no memory instruction), i.e. what
+//             the matrix cores sustain on this data at the clock the power cap allows; S > 0 keeps it running
+//             for about S seconds, printing a line per second (for sampling power and clock beside it)
 //   beam_host --tune --m M --n N --k K [--dtype fp16|bf16]
 //   beam_host --copy MiB      device-to-device copy of known size (calibrates profiler byte counters)
 #include <cmath>
@@ -32,7 +36,7 @@
 #include <string>
 #include <vector>
 
-#include "../../include/beam_hip.h"
+#include "../../include/beam_hip_debug.h"
 
 namespace {
 
@@ -272,7 +276,7 @@ BEAM_TEST(splitk_consistency) {
     BEAM_REQUIRE(c, beam_gemmrc_splitk(da.p, db.p, dc.p, M, N, K, BEAM_F16, &cfg, s, dw.p, (size_t)eff * M * N * 4, nullptr));
     if (dc.download16() != first) c.fail("split_k = " + std::to_string(s) + ": a workspace without flags gives other bits");
     int timed_out = 1;
-    BEAM_REQUIRE(c, beam_gemmrc_splitk_timed_out(dw.p, M, N, eff, nullptr, &timed_out));
+    BEAM_REQUIRE(c, beam_gemmrc_splitk_timed_out(dw.p, dw.bytes, M, N, eff, nullptr, &timed_out));
     if (timed_out) c.fail("split_k = " + std::to_string(s) + ": time-out reported");
   }
   return c;
@@ -534,18 +538,50 @@ int cli_bench_silu(const Args& a, Problem& p, const beam_tile_cfg& cfg) {
   return 0;
 }
 
+// The register-only matrix-core loop (beam_probe_mfma): launches of about 0.7 ms, like the 8192^3 kernel.
+int cli_probe_mfma(const Args& a) {
+  const int dtype = a.str("dtype", "fp16") == "bf16" ? BEAM_BF16 : BEAM_F16;
+  const std::string shape = a.str("mfma", "16x16x32"), data = a.str("data", "normal");
+  if ((shape != "16x16x32" && shape != "32x32x16") || (data != "normal" && data != "zeros")) {
+    std::fprintf(stderr, "--mfma 16x16x32|32x32x16, --data normal|zeros\n");
+    return 2;
+  }
+  const int mfma = shape == "32x32x16" ? BEAM_MFMA_32X32X16 : BEAM_MFMA_16X16X32;
+  const int kind = data == "zeros" ? BEAM_PROBE_DATA_ZEROS : BEAM_PROBE_DATA_NORMAL;
+  const int passes = a.num("passes", 1600), iters = a.num("iters", 200);
+  const double seconds = std::atof(a.str("seconds", "0").c_str());
+  int warmup = a.num("warmup", 100);
+  double spent = 0.0;
+  do {
+    float ms = 0;
+    double flop = 0;
+    if (beam_probe_mfma(dtype, mfma, kind, passes, warmup, iters, nullptr, &ms, &flop) != BEAM_OK) {
+      std::fprintf(stderr, "probe failed: %s\n", beam_last_error());
+      return 1;
+    }
+    std::printf("probe-mfma %s v_mfma_f32_%s %s operands, %d passes of 1024 matrix-core cycles per wavefront: %.4f ms per launch  "
+                "%.1f TFLOP/s = %.3f of 2500\n", dtype ? "bf16" : "fp16", shape.c_str(), data.c_str(), passes, ms, flop / ms / 1e9,
+                flop / ms / 1e9 / 2500.0);
+    std::fflush(stdout);
+    spent += (double)ms * 1e-3 * (warmup + iters);
+    warmup = 0;
+  } while (spent < seconds);
+  return 0;
+}
+
 int cli_bench(const Args& a) {
   const int M = a.num("m", 8192), N = a.num("n", 8192), K = a.num("k", 8192);
   const int dtype = a.str("dtype", "fp16") == "bf16" ? BEAM_BF16 : BEAM_F16;
   const std::string opname = a.str("op", "gemm");
-  const int op = opname == "splitk" ? BEAM_OP_SPLITK
-                 : opname == "ln"   ? BEAM_OP_GEMM_LN
-                 : opname == "nn"   ? BEAM_OP_MATMUL_NN  // B read as [K][N]
+  if (opname == "probe-mfma") return cli_probe_mfma(a);
+  const int op = opname == "splitk" ? (int)BEAM_OP_SPLITK
+                 : opname == "ln"   ? (int)BEAM_OP_GEMM_LN
+                 : opname == "nn"   ? (int)BEAM_OP_MATMUL_NN  // B read as [K][N]
                  // what the machine allows: empty launches, and a split-K launch with nothing but its loads
-                 : opname == "probe-empty"        ? BEAM_OP_PROBE_EMPTY
-                 : opname == "probe-empty-pair"   ? BEAM_OP_PROBE_EMPTY_PAIR
-                 : opname == "probe-splitk-loads" ? BEAM_OP_PROBE_SPLITK_LOADS
-                                                  : BEAM_OP_GEMM;
+                 : opname == "probe-empty"        ? (int)BEAM_OP_PROBE_EMPTY
+                 : opname == "probe-empty-pair"   ? (int)BEAM_OP_PROBE_EMPTY_PAIR
+                 : opname == "probe-splitk-loads" ? (int)BEAM_OP_PROBE_SPLITK_LOADS
+                                                  : (int)BEAM_OP_GEMM;
   const bool splitk_like = op == BEAM_OP_SPLITK || op == BEAM_OP_PROBE_SPLITK_LOADS;
   beam_tile_cfg cfg;
   int split = 1;

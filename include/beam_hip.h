@@ -113,10 +113,13 @@ size_t beam_splitk_workspace_bytes(int M, int N, int split_k);
 int beam_gemmrc_splitk(const void* A, const void* B, void* C, int M, int N, int K, int dtype,
                        const beam_tile_cfg* cfg, int split_k, void* ws, size_t ws_bytes,
                        void* stream);
-/* Waits for `stream`; *timed_out = 1 if a reducing workgroup of the latest one-launch split-K call on this
- * workspace gave up waiting (its outputs are NaN).  split_k_effective: beam_splitk_effective of that call.
- * Does not happen on a working device; the bound exists so that no kernel of the library can wait for ever. */
-int beam_gemmrc_splitk_timed_out(const void* ws, int M, int N, int split_k_effective, void* stream, int* timed_out);
+/* Waits for `stream`; *timed_out = 1 if the latest split-K call on this workspace ran as one launch and one of its
+ * reducing workgroups gave up waiting (its outputs are NaN).  ws_bytes, M, N: as given to that call;
+ * split_k_effective: beam_splitk_effective of that call.  0 for a call that had no waiting workgroups (one slice,
+ * two launches, a workspace that ends with the partial sums).  Does not happen on a working device; the bound
+ * exists so that no kernel of the library can wait for ever. */
+int beam_gemmrc_splitk_timed_out(const void* ws, size_t ws_bytes, int M, int N, int split_k_effective, void* stream,
+                                 int* timed_out);
 /* on != 0: beam_gemmrc_splitk always runs as two launches.  Off by default (environment:
  * BEAM_SPLITK_TWO_LAUNCHES=1).  Results are the same bits either way. */
 int beam_set_splitk_two_launches(int on);
@@ -158,34 +161,48 @@ int beam_gemmrc_ln(const void* A, const void* B, const void* gamma, const void* 
  *                   workgroup publishes its own and polls, boundedly, for the others'), then every
  *                   workgroup normalises and stores its own tile.  Needs all column tiles of a band
  *                   resident at once: N / block_n <= 64, a device of 256 CUs in 8 XCDs, and the device
- *                   not shared with other work while it runs.
+ *                   not shared with other work while it runs (otherwise the wait runs into its bound, the
+ *                   rows concerned come out as NaN and beam_gemmrc_ln_timed_out says so;
+ *                   beam_gemmrc_ln_checked then repeats the call as two passes by itself).
  *   BEAM_LN_TWOPASS the GEMM kernel stores fp32 X and per-tile statistics, a second kernel normalises.
  *   BEAM_LN_AUTO    fused when it applies, else two-pass (what beam_gemmrc_ln does); two-pass under
  *                   stream capture. */
 typedef enum beam_ln_mode { BEAM_LN_AUTO = 0, BEAM_LN_TWOPASS = 1, BEAM_LN_FUSED = 2 } beam_ln_mode;
-/* Workspace bytes.  _for is exact for the call beam_gemmrc_ln_ex(M, N, K, cfg, mode) will make; the
- * forms without K return, for cfg == NULL, the largest need over every tile the library could pick
- * for some K (with a tile given they are exact as well). */
+/* Workspace bytes.  _for is enough for the call beam_gemmrc_ln_ex(M, N, K, cfg, mode) on operands aligned as the
+ * tiled kernels need them (A, B, Y 16 bytes, gamma and beta 8): exact for BEAM_LN_TWOPASS and BEAM_LN_FUSED; for
+ * BEAM_LN_AUTO the larger of the two forms it can resolve to (one kernel eagerly; two passes under stream capture
+ * and as the retry of beam_gemmrc_ln_checked).  The forms without K are enough for any call with these M, N, cfg and
+ * mode: every K (cfg == NULL: every tile the library could pick), operands aligned to an element only, captured or
+ * not. */
 size_t beam_gemmrc_ln_workspace_bytes_for(int M, int N, int K, const beam_tile_cfg* cfg, int mode);
 size_t beam_gemmrc_ln_workspace_bytes_ex(int M, int N, const beam_tile_cfg* cfg, int mode);
 int beam_gemmrc_ln_ex(const void* A, const void* B, const void* gamma, const void* beta, float eps,
                       void* Y, int M, int N, int K, int dtype, const beam_tile_cfg* cfg, int mode,
                       void* ws, size_t ws_bytes, void* stream);
+/* beam_gemmrc_ln (BEAM_LN_AUTO) for callers that want the result whatever else runs on the device.  Synchronous:
+ * after the call it waits for `stream`; if the one-kernel form gave up waiting for a band of workgroups (a device that
+ * other work keeps occupied: beam_gemmrc_ln_timed_out), it runs the call again as two passes, which wait for
+ * nothing, and waits for that.  *fell_back (may be NULL) = 1 then.  ws_bytes as for BEAM_LN_AUTO.  Under stream
+ * capture it is beam_gemmrc_ln (two passes, nothing to check).  What the Python layer's gemmrc_ln calls by default. */
+int beam_gemmrc_ln_checked(const void* A, const void* B, const void* gamma, const void* beta, float eps, void* Y,
+                           int M, int N, int K, int dtype, const beam_tile_cfg* cfg, void* ws, size_t ws_bytes,
+                           void* stream, int* fell_back);
 /* The fused path's workspace needs no preparation and carries no state from call to call: every
  * fused launch has a tag that no earlier launch had, and a statistics word counts only if it carries
  * that tag (a stray word passes with probability 2^-32, and both words of a row have to).  So a fresh
  * buffer, one the allocator hands out again, one used for another shape or written over by somebody
  * else all work as they are, and the library keeps no host-side record of workspaces.  Launches that
- * share one workspace must be ordered on one stream.  This call only zeroes the 256-byte header
- * (synchronously), which forgets a recorded time-out; nothing requires it. */
+ * share one workspace must be ordered on one stream.  This call only zeroes the header's record of the latest
+ * launch and its time-out (synchronously; the replay counter of captured launches stays); nothing requires it. */
 int beam_gemmrc_ln_workspace_reset(const void* ws);
 /* Waits for `stream`, then *timed_out = 1 if the latest fused call on this workspace gave up
  * waiting for a band: the rows concerned are then NaN in Y.  Only possible if the device could not
  * hold a whole band of workgroups at once, e.g. because another process occupied most of it.  The
  * record names the launch it is about, so every fused call starts with a clean slate. */
 int beam_gemmrc_ln_timed_out(const void* ws, void* stream, int* timed_out);
-/* Bound of that wait: polls of statistics slots per thread (roughly a microsecond each; default
- * 4 Mi).  0 makes every thread that finds a slot unpublished give up at once; -1 makes every wait give
+/* Bound of that wait: polls of statistics slots per thread (3-4 microseconds each once the pauses between
+ * tries have grown; default 16384, about 60 ms: what a workgroup legitimately waits for is at most one tile's K loop
+ * behind it).  0 makes every thread that finds a slot unpublished give up at once; -1 makes every wait give
  * up whatever it finds: the kernel still ends normally and the flag is set, which is how the failure
  * path is exercised without hanging anything.  The same number bounds the wait of the reducing workgroups
  * of the one-launch split-K (polls of a tile's flags). */
@@ -194,9 +211,11 @@ int beam_set_ln_spin_limit(int polls);
 /* ---- GEMM with an independent elementwise job hidden in its K loop ------------------------ */
 
 /* C = A . B^T as beam_gemmrc and, in the same launch, Y[i] = silu(X[i]) = X[i] / (1 + exp(-X[i]))
- * for i in [0, count): 16-bit in, fp32 arithmetic, round-to-nearest 16-bit out.  The array is dealt
- * out over the GEMM's workgroups and streamed one 16-byte vector per thread per K tile, so the
- * elementwise traffic rides in the memory-side slack of the matrix-core-bound loop.  Replaces
+ * for i in [0, count): 16-bit in, fp32 arithmetic, round-to-nearest 16-bit out.  The array is cut into
+ * units of 4, 8 or 16 bytes (the narrowest with which the job still ends inside the K loop), dealt out in
+ * contiguous runs over the GEMM's workgroups and carried, a few units per K tile, by the wavefronts that
+ * issue the operand loads, so the elementwise traffic rides in the memory-side slack of the
+ * matrix-core-bound loop.  Replaces
  * entry_cute_parallel_gemmrc_lnr (cuda/cute_kernels/cute_gemm_ln.cu:230-245, kernel :24-228, bound
  * as cutlass_parallel_gemmrc_lnr in cuda/cute_kernels/main.cc), whose lnA/lnB are X/Y here and whose
  * lnM*lnN is `count`.  Unlike the reference, which gives the job to a quarter of the workgroups and
@@ -234,13 +253,7 @@ typedef enum beam_op {
   BEAM_OP_GEMM_LN = 2,
   BEAM_OP_GEMM_SILU = 3, /* beam_parallel_gemmrc_silu */
   BEAM_OP_SILU = 4,      /* beam_silu alone            */
-  BEAM_OP_MATMUL_NN = 5, /* beam_matmul_nn             */
-  /* Not operators: launches that measure what the machine allows (no counterpart in the reference). */
-  BEAM_OP_PROBE_EMPTY = 6,        /* one empty kernel of 256 workgroups x 256 threads                */
-  BEAM_OP_PROBE_EMPTY_PAIR = 7,   /* two empty kernels in a row (256 x 256, then 1024 x 64 threads)   */
-  BEAM_OP_PROBE_SPLITK_LOADS = 8  /* the partial kernel of BEAM_OP_SPLITK for the same arguments with its
-                                     loads and LDS reads but no MFMAs and no stores, and no reduction;
-                                     fp16, tiles 64x128 (wave 32x64) and 64x64 (wave 32x32), pipeline 2 */
+  BEAM_OP_MATMUL_NN = 5  /* beam_matmul_nn             */
 } beam_op;
 
 typedef struct beam_problem {
@@ -275,7 +288,7 @@ int beam_event_destroy(void* event);
 
 /* ---- streams and graphs (so that hosts need no other GPU runtime) -------------------------- */
 
-/* Every operator above is one or two kernel launches on the caller's stream and neither allocates nor
+/* Every operator above is one to three kernel launches on the caller's stream and neither allocates nor
  * synchronises, so a sequence of them can be captured once and replayed as a HIP graph: the usual cure
  * for launch-bound loops of small GEMMs (a split-K call is one launch of 13 us).  The reference
  * has no counterpart (it launches on the legacy default stream, cuda/cute_kernels/cute_gemm_128x128.cu:
@@ -310,36 +323,6 @@ int beam_sync(void* stream);
 int beam_host_fill_uniform(void* dst_host, size_t n, int dtype, uint64_t seed, uint64_t tensor_id);
 int beam_host_fill_normal(void* dst_host, size_t n, int dtype, uint64_t seed, uint64_t tensor_id,
                           float mean, float scale);
-
-/* ---- index maps, exported for host-side verification ---------------------------------------- */
-
-/* Workgroup id -> (tile_m, tile_n) as the kernels compute it (divisions done as multiplications by constants the
- * host prepares), and the same map written with plain divisions, which defines it. */
-int beam_dbg_tile_of_workgroup(int wg, int tiles_m, int tiles_n, int group_m, int* tm, int* tn);
-int beam_dbg_tile_of_workgroup_by_division(int wg, int tiles_m, int tiles_n, int group_m, int* tm, int* tn);
-/* n / d (n < 2^31, d >= 1) through the multiplier the host would prepare for d. */
-unsigned beam_dbg_fast_div(unsigned n, unsigned d);
-/* Byte offset of (row, 16-byte chunk) inside an LDS stage. */
-int beam_dbg_lds_offset(int row, int chunk);
-/* Byte offset of element (k, n), n a multiple of 4, inside a K-major LDS stage of block_n columns
- * (B stored [K][N], beam_matmul_nn). */
-int beam_dbg_kmajor_lds_offset(int k, int n, int block_n);
-/* The tile a beam_gemmrc_ln call without a tile takes for its one-kernel form on a device of `compute_units` CUs
- * (the library's LayerNorm cost model; BEAM_ERR_UNSUPPORTED where that form applies with no tile). */
-int beam_dbg_ln_default_config(int M, int N, int K, int compute_units, beam_tile_cfg* cfg);
-/* The 4-wavefront kernel with B stored [K][N] (256 columns, 512 bytes per row of k in an LDS slot): the XOR code of
- * the 16-byte chunks of row k, and the byte offset of the 8 bytes that lane 16 g + 4 e + q supplies to the first
- * transposing read of 16-column block b (0..7) of the wavefront's column half wn (0, 1). */
-int beam_dbg_w4_kmajor_swizzle(int k);
-int beam_dbg_w4_kmajor_read_offset(int wn, int b, int g, int e, int q);
-/* Workgroup id -> tile of the padded band-block grid used by the fused GEMM+LayerNorm (tm = -1:
- * the id is padding), and the size of that grid. */
-int beam_dbg_band_block_tile(int wg, int tiles_m, int tiles_n, int gb, int gc, int* tm, int* tn);
-int beam_dbg_band_block_grid(int tiles_m, int gb, int gc);
-/* The same for the order that keeps whole bands (bx at a time) on one XCD, used when a band is
- * short enough for it. */
-int beam_dbg_band_xcd_tile(int wg, int tiles_m, int tiles_n, int bx, int* tm, int* tn);
-int beam_dbg_band_xcd_grid(int tiles_m, int tiles_n, int bx);
 
 #ifdef __cplusplus
 }

@@ -1,4 +1,4 @@
-"""libbeam_hip.so loads without a GPU and exports every function include/beam_hip.h declares."""
+"""libbeam_hip.so loads without a GPU and exports every function include/beam_hip.h and beam_hip_debug.h declare."""
 import ctypes
 import os
 import re
@@ -6,8 +6,8 @@ import re
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
-def declared_functions():
-    text = open(os.path.join(ROOT, "include", "beam_hip.h")).read()
+def declared_functions(header="beam_hip.h"):
+    text = open(os.path.join(ROOT, "include", header)).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     names = re.findall(r"\b(beam_[a-z0-9_]+)\s*\(", text)
     return sorted(set(names))
@@ -19,13 +19,19 @@ def test_every_declared_symbol_is_exported(beamc):
     lib = ctypes.CDLL(beamc.library_path())
     missing = [n for n in names if not hasattr(lib, n)]
     assert not missing, missing
+    # the operators' header carries no test or measurement surface; that lives in the second header
+    assert not [n for n in names if n.startswith(("beam_dbg_", "beam_probe_"))]
+    debug = declared_functions("beam_hip_debug.h")
+    assert len(debug) >= 10 and all(n.startswith(("beam_dbg_", "beam_probe_")) for n in debug), debug
+    assert not [n for n in debug if not hasattr(lib, n)]
 
 
 def test_header_compiles_as_c(tmp_path):
     """The header is plain C (no C++ types in the boundary)."""
     import subprocess
     src = tmp_path / "t.c"
-    src.write_text('#include "beam_hip.h"\nint main(void) { beam_tile_cfg c = {0}; (void)c; return BEAM_OK; }\n')
+    src.write_text('#include "beam_hip.h"\n#include "beam_hip_debug.h"\n'
+                   'int main(void) { beam_tile_cfg c = {0}; (void)c; return BEAM_OK + 0 * BEAM_OP_PROBE_EMPTY; }\n')
     subprocess.run(["gcc", "-std=c99", "-Wall", "-Werror", "-I", os.path.join(ROOT, "include"), "-c", str(src),
                     "-o", str(tmp_path / "t.o")], check=True)
 

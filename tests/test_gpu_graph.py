@@ -99,6 +99,20 @@ def test_graph_replay_matches_eager(gpu, beamc):
             want = snapshot()
             for k in want:
                 assert (got[k] == want[k]).all(), f"replay {replay}, second in a row: {k} differs from the eager result"
+        # A reset of the fused LayerNorm's workspace between two replays (what a caller does after a time-out) forgets
+        # the recorded launch but not the replay counter: the replay behind it still gets a tag of its own, and the
+        # statistics the replay before it left in the workspace do not pass for its own.
+        chk(L.beam_gemmrc_ln_workspace_reset(ws_lnf.ptr))
+        upload()
+        poison()
+        chk(L.beam_graph_launch(graph, stream))
+        chk(L.beam_sync(stream))
+        got = snapshot()
+        poison()
+        sequence(None)
+        want = snapshot()
+        for k in want:
+            assert (got[k] == want[k]).all(), f"replay after a workspace reset: {k} differs from the eager result"
     finally:
         chk(L.beam_graph_destroy(graph))
         chk(L.beam_stream_destroy(stream))

@@ -143,17 +143,61 @@ def test_ln_fused_timeout_is_reported_not_hung(gpu, beamc):
     y = beamc.DeviceArray((M, N))
     try:
         assert beamc.lib.beam_set_ln_spin_limit(-1) == 0
-        beamc.gemmrc_ln(da, db, y, dg, dbt, mode=beamc.LN_FUSED)
+        beamc.gemmrc_ln(da, db, y, dg, dbt, mode=beamc.LN_FUSED, check=False)
         beamc.sync()
         assert beamc.gemmrc_ln_timed_out()
         assert np.isnan(y.to_numpy().view(np.float16)).all()
         with pytest.raises(beamc.BeamError):
             beamc.gemmrc_ln(da, db, y, dg, dbt, mode=beamc.LN_FUSED, check=True)
     finally:
-        beamc.lib.beam_set_ln_spin_limit(4 << 20)
+        beamc.lib.beam_set_ln_spin_limit(beamc.DEFAULT_SPIN_LIMIT)
     beamc.gemmrc_ln(da, db, y, dg, dbt, mode=beamc.LN_FUSED, check=True)  # the flag was cleared by this call
     assert (y.to_numpy() == good).all()
     for x in (da, db, dg, dbt, y):
+        x.free()
+
+
+def test_default_call_recovers_from_a_forced_timeout(gpu, beamc, oracle):
+    """The default Python call (LN_AUTO, checking) gives the right result even when the one-kernel form cannot
+    finish its exchange: with the spin limit at -1 every wait gives up at once (every kernel still ends normally),
+    the call notices, runs again as two passes and says so.  The C entry behind it (beam_gemmrc_ln_checked) reports
+    the same through its flag; without the forced time-out neither falls back."""
+    import ctypes
+    M, N, K = 512, 4096, 256
+    a, b, g_, bt = make_ln_inputs(beamc, M, N, K, F16, 27)
+    ref = oracle.gemmrc_ln(a, b, g_, bt, 1e-5, F16)
+    two_pass = run_ln(beamc, a, b, g_, bt, F16, mode=beamc.LN_TWOPASS)
+    da, db = beamc.DeviceArray.from_numpy(a), beamc.DeviceArray.from_numpy(b)
+    dg, dbt = beamc.DeviceArray.from_numpy(g_), beamc.DeviceArray.from_numpy(bt)
+    y = beamc.DeviceArray((M, N))
+    L = beamc.lib
+    assert L.beam_gemmrc_ln_workspace_bytes_for(M, N, K, None, beamc.LN_AUTO) >= \
+        max(L.beam_gemmrc_ln_workspace_bytes_for(M, N, K, None, m) for m in (beamc.LN_FUSED, beamc.LN_TWOPASS))
+    ws = beamc.DeviceArray((L.beam_gemmrc_ln_workspace_bytes_for(M, N, K, None, beamc.LN_AUTO),), itemsize=1)
+    try:
+        y.fill_bytes(0xEE)
+        assert beamc.gemmrc_ln(da, db, y, dg, dbt) is False       # a quiet device: one kernel, no retry
+        check_ln(oracle, y.to_numpy(), ref, F16, "default call")
+        assert L.beam_set_ln_spin_limit(-1) == 0
+        y.fill_bytes(0xEE)
+        assert beamc.gemmrc_ln(da, db, y, dg, dbt) is True        # gave up, ran again as two passes
+        got = y.to_numpy()
+        check_ln(oracle, got, ref, F16, "default call with every wait forced to give up")
+        assert (got == two_pass).all()
+        y.fill_bytes(0xEE)
+        fell_back = ctypes.c_int(0)
+        rc = L.beam_gemmrc_ln_checked(da.ptr, db.ptr, dg.ptr, dbt.ptr, ctypes.c_float(1e-5), y.ptr, M, N, K, F16, None,
+                                      ws.ptr, ws.nbytes, None, ctypes.byref(fell_back))
+        assert rc == 0 and fell_back.value == 1, L.beam_last_error().decode()
+        assert (y.to_numpy() == two_pass).all()
+    finally:
+        L.beam_set_ln_spin_limit(beamc.DEFAULT_SPIN_LIMIT)
+    fell_back = ctypes.c_int(1)
+    rc = L.beam_gemmrc_ln_checked(da.ptr, db.ptr, dg.ptr, dbt.ptr, ctypes.c_float(1e-5), y.ptr, M, N, K, F16, None,
+                                  ws.ptr, ws.nbytes, None, ctypes.byref(fell_back))
+    assert rc == 0 and fell_back.value == 0
+    check_ln(oracle, y.to_numpy(), ref, F16, "checked call, normal budget")
+    for x in (da, db, dg, dbt, y, ws):
         x.free()
 
 
@@ -269,7 +313,7 @@ def test_two_fused_launches_share_the_device(gpu, beamc):
                 assert flag.value == 0, f"stream {i} gave up waiting (repetition {rep})"
                 assert (sets[i][1].to_numpy() == want[i]).all(), f"stream {i}, repetition {rep}"
     finally:
-        beamc._check(L.beam_set_ln_spin_limit(4 << 20))
+        beamc._check(L.beam_set_ln_spin_limit(beamc.DEFAULT_SPIN_LIMIT))
         for s in streams:
             beamc._check(L.beam_stream_destroy(s))
         for d, y, ws in sets:

@@ -53,7 +53,7 @@ def test_one_launch_equals_two_launches(gpu, beamc):
                     assert (one == two).all(), (M, N, K, dtype, split, bm, bn, tm, tn, pipe)
                 assert not (one == 0xEEEE).any()
                 flag = ctypes.c_int(1)
-                assert L.beam_gemmrc_splitk_timed_out(ws.ptr, M, N, s, None, ctypes.byref(flag)) == 0 and flag.value == 0
+                assert L.beam_gemmrc_splitk_timed_out(ws.ptr, ws.nbytes, M, N, s, None, ctypes.byref(flag)) == 0 and flag.value == 0
         for t in (a, b, c):
             t.free()
     ws.free()
@@ -147,7 +147,7 @@ def test_bounded_wait_gives_up_visibly(gpu, beamc):
     try:
         bad = _call(beamc, a, b, c, M, N, K, F16, cfg, 16, ws, False)
         flag = ctypes.c_int(0)
-        assert L.beam_gemmrc_splitk_timed_out(ws.ptr, M, N, s, None, ctypes.byref(flag)) == 0 and flag.value == 1
+        assert L.beam_gemmrc_splitk_timed_out(ws.ptr, ws.nbytes, M, N, s, None, ctypes.byref(flag)) == 0 and flag.value == 1
         assert np.isnan(bad.view(np.float16)).all()
         with pytest.raises(beamc.BeamError):
             beamc.gemmrc_splitk_spec(a, b, c, shape_threadblock=(64, 64), shape_warp=(32, 32), split_k_slices=16,
@@ -157,7 +157,7 @@ def test_bounded_wait_gives_up_visibly(gpu, beamc):
     again = _call(beamc, a, b, c, M, N, K, F16, cfg, 16, ws, False)
     assert (again == good).all()
     flag = ctypes.c_int(1)
-    assert L.beam_gemmrc_splitk_timed_out(ws.ptr, M, N, s, None, ctypes.byref(flag)) == 0 and flag.value == 0
+    assert L.beam_gemmrc_splitk_timed_out(ws.ptr, ws.nbytes, M, N, s, None, ctypes.byref(flag)) == 0 and flag.value == 0
     beamc.gemmrc_splitk_spec(a, b, c, shape_threadblock=(64, 64), shape_warp=(32, 32), split_k_slices=16, pipeline=2, check=True)
     for t in (a, b, c, ws):
         t.free()

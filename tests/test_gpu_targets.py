@@ -14,7 +14,8 @@ def _best(fn, rounds=3):
 
 
 def test_headline_throughput(gpu, beamc):
-    """fp16 8192^3 on N(0,1)/sqrt(K) data: 1390-1515 TFLOP/s measured across machines."""
+    """fp16 8192^3 on N(0,1)/sqrt(K) data: 1468-1570 TFLOP/s measured across machines (the 8-wavefront kernel this
+    one replaced: 1445 on its best machine)."""
     M = N = K = 8192
     a = beamc.DeviceArray.from_numpy(beamc.host_normal((M, K), F16, 7, 0, 0.0, K ** -0.5))
     b = beamc.DeviceArray.from_numpy(beamc.host_normal((N, K), F16, 7, 1, 0.0, K ** -0.5))
@@ -24,7 +25,7 @@ def test_headline_throughput(gpu, beamc):
     finally:
         for t in (a, b, c):
             t.free()
-    assert 2.0 * M * N * K / (ms * 1e-3) / 1e12 >= 1250.0, ms
+    assert 2.0 * M * N * K / (ms * 1e-3) / 1e12 >= 1400.0, ms
 
 
 def test_splitk_three_times_faster_than_no_split(gpu, beamc):
@@ -42,7 +43,7 @@ def test_splitk_three_times_faster_than_no_split(gpu, beamc):
         for t in (a, b, c):
             t.free()
     assert plain >= 3.0 * split, (plain, split)
-    assert split <= 0.020, split  # ms; 13.5-16 us measured
+    assert split <= 0.016, split  # ms; 12.5-14 us measured
 
 
 def test_fused_layernorm_within_ten_percent_of_plain_gemm(gpu, beamc):

@@ -377,22 +377,45 @@ def test_roofline_calculator():
 
 
 def test_ln_workspace_query_covers_every_default_call(beamc):
-    """The size queries without K must cover whatever tile the library picks once it knows K (a call without a
-    tile): for every shape, query(M, N) >= exact need(M, N, K), and with a tile given the two agree."""
+    """The workspace queries against what the entry point insists on (beam_dbg_ln_plan_bytes is the function
+    beam_gemmrc_ln_ex computes its requirement with), on a host without a GPU and with a 256-CU device assumed (where
+    AUTO is the one-kernel form):
+    query(M, N) covers every path a call can take -- any K (also K % 8 != 0), operands aligned to an element only,
+    a stream being captured (AUTO is two passes then), Y / gamma / beta 16-byte aligned or not;
+    query_for(M, N, K) covers every path of a call on aligned operands, captured or not; with a tile given and two
+    passes the two queries agree."""
+    import ctypes
+    import itertools
     L = beamc.lib
-    for M in (64, 300, 1024, 4096, 16384):
-        for N in (40, 1000, 4096, 8192, 20000):
-            loose = L.beam_gemmrc_ln_workspace_bytes_ex(M, N, None, beamc.LN_AUTO)
-            assert loose == L.beam_gemmrc_ln_workspace_bytes(M, N, None)
-            for K in (8, 64, 200, 2048, 32768):
-                exact = L.beam_gemmrc_ln_workspace_bytes_for(M, N, K, None, beamc.LN_AUTO)
-                assert 0 < exact <= loose, (M, N, K, exact, loose)
-            for cfg in (beamc.TileConfig(128, 128, 64, 64), beamc.TileConfig(256, 256, 128, 64)):
-                import ctypes
-                c = cfg.to_c()
-                for mode in (beamc.LN_AUTO, beamc.LN_TWOPASS):
-                    assert L.beam_gemmrc_ln_workspace_bytes_ex(M, N, ctypes.byref(c), mode) == \
-                        L.beam_gemmrc_ln_workspace_bytes_for(M, N, 4096, ctypes.byref(c), mode)
+    modes = (beamc.LN_AUTO, beamc.LN_TWOPASS, beamc.LN_FUSED)
+    tiles = (None, beamc.TileConfig(128, 128, 64, 64), beamc.TileConfig(256, 256, 128, 64), beamc.TileConfig(256, 256, 128, 128))
+    try:
+        for cus in (0, 256):
+            assert L.beam_dbg_assume_compute_units(cus) == 0, "this test needs a host without a GPU"
+            fused_seen = 0
+            for M, N in itertools.product((64, 300, 1024, 4096, 16384), (40, 1000, 4096, 8192, 20000)):
+                assert L.beam_gemmrc_ln_workspace_bytes_ex(M, N, None, beamc.LN_AUTO) == L.beam_gemmrc_ln_workspace_bytes(M, N, None)
+                for cfg, mode in itertools.product(tiles, modes):
+                    c = cfg.to_c() if cfg else None
+                    cp = ctypes.byref(c) if cfg else None
+                    loose = L.beam_gemmrc_ln_workspace_bytes_ex(M, N, cp, mode)
+                    assert loose >= M * N * 4  # the plain path's fp32 copy of the product
+                    for K in (8, 64, 200, 203, 2048, 32768):
+                        exact = L.beam_gemmrc_ln_workspace_bytes_for(M, N, K, cp, mode)
+                        for plain, capturing, wide in itertools.product((0, 1), repeat=3):
+                            plan = L.beam_dbg_ln_plan_bytes(M, N, K, cp, mode, plain, capturing, wide)
+                            if plan == 0:  # a form that does not apply (fused on this device / for this N): the call fails too
+                                assert mode == beamc.LN_FUSED and not plain and K % 8 == 0, (cus, M, N, K, mode, plain)
+                                continue
+                            assert plan <= loose, (cus, M, N, K, cfg, mode, plain, capturing, wide, plan, loose)
+                            if not plain:
+                                assert 0 < plan <= exact, (cus, M, N, K, cfg, mode, capturing, wide, plan, exact)
+                            fused_seen += plan < M * N * 4
+                    if cfg and mode != beamc.LN_FUSED:
+                        assert loose == L.beam_gemmrc_ln_workspace_bytes_for(M, N, 4096, cp, mode)
+            assert (fused_seen > 0) == (cus == 256)  # the 256-CU branch really took the one-kernel form
+    finally:
+        L.beam_dbg_assume_compute_units(0)
 
 
 def test_default_tile_model_matches_its_table_and_the_library(beamc):
