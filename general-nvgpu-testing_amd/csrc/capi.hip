@@ -633,6 +633,9 @@ size_t beam_splitk_workspace_bytes(int M, int N, int split_k) {
   return align_up(splitk_partial_bytes(M, N, split_k), 256) + (size_t)sk_sync_bytes(M, N, split_k);
 }
 
+// 1: the fused GEMM+LayerNorm of the 4-wavefront kernel always runs one workgroup per tile (testing: beam_dbg_set_ln_walk)
+static std::atomic<int> g_ln_no_walk{0};
+
 // 0: one launch where it applies, 1: always the partial kernel followed by the reduce kernel
 static std::atomic<int> g_splitk_two_launches{[] {
   const char* e = getenv("BEAM_SPLITK_TWO_LAUNCHES");
@@ -987,6 +990,11 @@ size_t beam_dbg_ln_plan_bytes(int M, int N, int K, const beam_tile_cfg* cfg, int
   return plan.need;
 }
 
+int beam_dbg_set_ln_walk(int on) {
+  g_ln_no_walk.store(on ? 0 : 1);
+  return BEAM_OK;
+}
+
 int beam_dbg_assume_compute_units(int compute_units) {
   std::lock_guard<std::mutex> lk(g_dev_mu);
   if (g_dev.status == BEAM_OK) return fail(BEAM_ERR_INVALID, "a device has been probed: its own CU count stands");
@@ -1079,8 +1087,18 @@ int beam_gemmrc_ln_ex(const void* A, const void* B, const void* gamma, const voi
     } else {
       grid = (unsigned)band_block_grid(p.tiles_m, p.group_m, p.group_n);
     }
+    // the band orders' divisors as multipliers (tile_map.h: band_order_divs)
+    p.divs = band_order_divs(p.tiles_n, p.group_m, p.group_n);
     if (plan.w4) {
-      BEAM_HIP(launch_gemm_w4_ln(p, dtype, dim3(grid, 1, 1), st));
+      // More ids than CUs: one workgroup per CU walks the ids w, w + CUs, ... of the same order, with the next
+      // tile's first operand tiles arriving while the band's statistics are exchanged (gemm_w4.h says why no
+      // chain of waits closes: a band's ids lie within fewer than 256 of each other in all three orders).  The
+      // walking form keeps the epilogue's scratch inside the two LDS slots the operand ring leaves free, which
+      // holds a band of up to 32 column tiles; wider bands keep one workgroup per tile.
+      p.ln_ids = (int)grid;
+      const unsigned cus = (unsigned)g_dev.cus;
+      const bool walk = grid > cus && p.tiles_n <= kW4LnCompactTiles && !g_ln_no_walk.load(std::memory_order_relaxed);
+      BEAM_HIP(launch_gemm_w4_ln(p, dtype, dim3(walk ? cus : grid, 1, 1), st));
       return BEAM_OK;
     }
     BEAM_HIP(ks->launch[dtype][kEpiLnFused][c.pipeline](p, dim3(grid, 1, 1), st));
@@ -1456,5 +1474,13 @@ int beam_dbg_band_block_tile(int wg, int tiles_m, int tiles_n, int gb, int gc, i
 }
 
 int beam_dbg_band_block_grid(int tiles_m, int gb, int gc) { return band_block_grid(tiles_m, gb, gc); }
+
+int beam_dbg_band_order_tile(int id, int tiles_m, int tiles_n, int group_m, int group_n, int* tm, int* tn) {
+  if (tiles_m < 1 || tiles_n < 1 || group_m < 1 || id < 0 || !tm || !tn) return fail(BEAM_ERR_INVALID, "bad band-order query");
+  const TileCoord t = band_order_tile(id, tiles_m, tiles_n, group_m, group_n, band_order_divs(tiles_n, group_m, group_n));
+  *tm = t.tm;
+  *tn = t.tn;
+  return BEAM_OK;
+}
 
 }  // extern "C"

@@ -18,6 +18,8 @@ hipError_t launch_gemm_w4(const GemmParams& p, int dtype, dim3 grid, hipStream_t
   return dtype == BEAM_BF16 ? launch_w4_t<__bf16, false>(p, grid, stream) : launch_w4_t<_Float16, false>(p, grid, stream);
 }
 
+static_assert(kW4LnCompactTiles == GemmW4<_Float16, false, true>::kLnCompactTiles, "the host's bound is the kernel's");
+
 hipError_t launch_gemm_w4_ln(const GemmParams& p, int dtype, dim3 grid, hipStream_t stream) {
   return dtype == BEAM_BF16 ? launch_w4_t<__bf16, false, true>(p, grid, stream) : launch_w4_t<_Float16, false, true>(p, grid, stream);
 }

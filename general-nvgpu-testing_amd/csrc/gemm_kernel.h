@@ -120,6 +120,8 @@ struct GemmParams {
   int group_m;   // rasterisation group height in tiles (fused LayerNorm: bands per band group)
   int group_n;   // fused LayerNorm: columns of a band group owned by one XCD; 0: whole bands, group_m of them, per XCD;
                  // -1: band after band, workgroup id = band * tiles_n + column (no padding)
+  int ln_ids;    // fused LayerNorm on the kernel of gemm_w4.h: ids of that order, padding included; the grid may be smaller
+                 // (a workgroup then walks the ids blockIdx, blockIdx + gridDim, ...)
   TileDivs divs; // the tile maps' divisors as multipliers (tile_map.h), made by the host from tiles_m, tiles_n, group_m
   // Side job (kEpiStoreSide): y[i] = silu(x[i]) over a flat 16-bit array.  The whole 8-element
   // groups of the array are cut into units of side_width bytes (16, 8 or 4), dealt out in

@@ -134,9 +134,13 @@ __host__ __device__ inline int w4_b_row(int b, int r) { return 32 * (b >> 1) + 4
 // four issue: loads issued faster than that stall the wavefront, and with it its MFMAs, at issue.
 // C_NT: C is stored non-temporal (an output larger than the last-level cache: its lines then do not push
 // operand panels out of the caches).
-// LN: the fused GEMM+LayerNorm of gemm_kernel.h (kEpiLnFused) with this K loop: one output tile per
-// workgroup in the band order of tile_map.h, and after the K loop the same exchange of per-row (mean, M2)
-// pairs between the column tiles of a row band, normalisation in registers, Y stored once.
+// LN: the fused GEMM+LayerNorm of gemm_kernel.h (kEpiLnFused) with this K loop: output tiles in the band
+// order of tile_map.h, and after each tile's K loop the same exchange of per-row (mean, M2) pairs between the
+// column tiles of a row band, normalisation in registers, Y stored once.  A workgroup walks the ids
+// blockIdx, blockIdx + gridDim, ... of that order: with a grid as large as the order it has one tile, with a
+// grid of one workgroup per CU it walks several, and the operand ring then runs through the tile boundary as
+// in the plain kernel -- the next tile's first operand tiles arrive while the band's statistics are
+// exchanged (walking_layer_norm below says why nobody waits for ever).
 // B_KMAJOR: B is stored [K][N].
 template <typename T, bool C_NT = false, bool LN = false, int SB = 4, int SA = 8, int G0 = 2, bool B_KMAJOR = false>
 struct GemmW4 {
@@ -175,6 +179,7 @@ struct GemmW4 {
     return m;
   }
   static constexpr int LAST_READ = last_read(0) > last_read(1) ? last_read(0) : last_read(1);
+  static constexpr int kLnStores = FM * FN / 2;  // 16-byte stores per wavefront of a LayerNorm epilogue (32)
   static_assert(LAST_B + 3 < 64 && LAST_A + 3 < 64 && LAST_READ + 2 < LAST_A, "room for the scalar bookkeeping");
   static_assert(load_at(0, LAST_B) == LPT - 1 && load_at(1, LAST_A) == LPT - 1 && LAST_B < 62 && LAST_A < 62, "loads fit a step");
 
@@ -188,13 +193,22 @@ struct GemmW4 {
     const int n_k = K / kBK;
     const int total_tiles = p.tiles_m * p.tiles_n;
     const int first_tile = blockIdx.x, tile_step = gridDim.x;
+    // LN: id of the band order -> tile (tm < 0: the band grids are padded), and the first id from `id` on, in
+    // steps of the grid, that is a tile (>= p.ln_ids: none)
+    auto ln_next_id = [&](int id, TileCoord* tc) {
+      for (; id < p.ln_ids; id += tile_step) {
+        *tc = band_order_tile(id, p.tiles_m, p.tiles_n, p.group_m, p.group_n, p.divs);
+        if (tc->tm >= 0) break;
+      }
+      return id;
+    };
+    int ln_id = 0;
     TileCoord ln_tile{0, 0};
     if constexpr (LN) {
-      ln_tile = p.group_n > 0    ? band_block_tile(blockIdx.x, p.tiles_m, p.tiles_n, p.group_m, p.group_n)
-                : p.group_n == 0 ? band_xcd_tile(blockIdx.x, p.tiles_m, p.tiles_n, p.group_m)
-                                 : TileCoord{(int)blockIdx.x / p.tiles_n, (int)blockIdx.x % p.tiles_n};
-      if (ln_tile.tm < 0) return;  // the band grids are padded
+      ln_id = ln_next_id(first_tile, &ln_tile);
+      if (ln_id >= p.ln_ids) return;
     }
+    // (LN: the number of tiles is found on the way; the streams' descriptors are made from `has_tile` flags)
     const int my_tiles = LN ? 1 : (total_tiles - first_tile + tile_step - 1) / tile_step;
     const int g_total = my_tiles * n_k;  // K tiles this workgroup multiplies
 
@@ -221,10 +235,7 @@ struct GemmW4 {
 
     // Operand rows of the workgroup's j-th output tile as (address, bytes) of a buffer descriptor; empty
     // past its last tile: such loads are issued and counted like any other and touch no memory.
-    auto tile_coord = [&](int j) {
-      if constexpr (LN) return ln_tile;
-      else return tile_of_workgroup(first_tile + j * tile_step, p.tiles_m, p.tiles_n, p.group_m, p.divs);
-    };
+    auto tile_coord = [&](int j) { return tile_of_workgroup(first_tile + j * tile_step, p.tiles_m, p.tiles_n, p.group_m, p.divs); };
     auto rows_of_a = [&](int j, TileCoord tc) {
       if (j >= my_tiles) return make_rsrc(p.A, 0u);
       const int row0 = tc.tm * BM;
@@ -260,7 +271,9 @@ struct GemmW4 {
     // instruction.  The loads are therefore invisible to the compiler's wait-count bookkeeping; every wait
     // for them in this kernel is an explicit s_waitcnt vmcnt.
     auto set_load_target = [&](const Stream& st, auto i_tag) __attribute__((always_inline)) {
-      asm volatile("s_add_u32 m0, %0, %1" ::"s"(st.lds), "n"(decltype(i_tag)::value * 4096) : "memory");
+      // (the add writes the scalar condition bit: without that in the clobber list the compiler keeps a compare's
+      // result alive across this statement and selects on the add's carry instead)
+      asm volatile("s_add_u32 m0, %0, %1" ::"s"(st.lds), "n"(decltype(i_tag)::value * 4096) : "memory", "scc");
     };
     auto load_tile_part = [&](const Stream& st, unsigned voff) __attribute__((always_inline)) {
       asm volatile("buffer_load_dwordx4 %0, %1, %2 offen lds" ::"v"(voff), "s"(st.rows), "s"(st.koff) : "memory");
@@ -390,6 +403,11 @@ struct GemmW4 {
     Stream ld_a, ld_b;         // where the next A / B loads go
     __amdgpu_buffer_rsrc_t next_a, next_b;  // operand rows of the output tile after the one the streams are at
     int rd_a = 0, rd_b = B_REGION;  // slots (byte offsets) of the K tile being multiplied
+    // LN, FIRST: the accumulators hold nothing that step A could complete (the previous tile was finished and
+    // stored by its epilogue; set 1 is stale), so step A issues no MFMA -- a one-cycle no-op stands in for each,
+    // which also keeps the wait state between a write of M0 and the load that uses it.  after_epilogue: the
+    // youngest memory operations of this wavefront are then the 32 stores of that epilogue, not loads.
+    bool after_epilogue = false;
     auto k_tile = [&](auto first_tag) __attribute__((always_inline)) {
       constexpr bool FIRST = decltype(first_tag)::value;
       const char* sa = smem + rd_a;
@@ -401,13 +419,20 @@ struct GemmW4 {
         // share one operand (fewer input toggles; this part is power limited)
         constexpr int i = m >> 3, b = (i & 1) ? 7 - (m & 7) : (m & 7);
         constexpr int blk = 8 * i + b;
-        if constexpr (half == 0) Mfma::template fma<blk>(fb1[b], fa1[i]);
+        if constexpr (half == 0 && LN && FIRST) asm volatile("s_nop 0");
+        else if constexpr (half == 0) Mfma::template fma<blk>(fb1[b], fa1[i]);
         else if constexpr (FIRST) Mfma::template first<blk>(fb0[b], fa0[i]);
         else Mfma::template fma<blk>(fb0[b], fa0[i]);
         // the gap
         if constexpr (gap == G0 - 1) {
           // Two MFMAs of the previous K tile are in the matrix core's queue while the wavefronts meet.
-          wait_vm_and_lds<LPT>();  // my fills of this K tile have landed (the youngest 8 are A of the next one)
+          // my fills of this K tile have landed (the youngest 8 are A of the next one) ...
+          if constexpr (LN && FIRST) {
+            if (after_epilogue) wait_vm_and_lds<kLnStores>();
+            else wait_vm_and_lds<LPT>();
+          } else {
+            wait_vm_and_lds<LPT>();
+          }
           bare_barrier();          // ... everyone's have, and everyone is done reading the slots refilled below
         }
         constexpr int ld = load_at(half, m), rd = read_at(half, m);
@@ -451,28 +476,71 @@ struct GemmW4 {
       });
     };
 
-    if (g_total > 0) {
-      // Prologue: A and B of K tile 0, A of K tile 1 (oldest first: the first wait is about tile 0).
-      TileCoord tc_cur = tile_coord(0);
-      const __amdgpu_buffer_rsrc_t rows_a0 = rows_of_a(0, tc_cur), rows_b0 = rows_of_b(0, tc_cur);
-      next_a = rows_a0;  // (never used: K >= 3 tiles, so no stream wraps before the loop below sets them)
+    auto load_whole_tile = [&](const Stream& st, const unsigned(&voff)[LPT]) __attribute__((always_inline)) {
+      w4_static_for<0, LPT>([&](auto i_tag) __attribute__((always_inline)) {
+        set_load_target(st, i_tag);
+        asm volatile("s_nop 0");  // the wait state between the write of M0 and its use
+        load_tile_part(st, voff[decltype(i_tag)::value]);
+      });
+    };
+    // Prologue: A and B of K tile 0, A of K tile 1 (oldest first: the first wait is about tile 0).
+    auto prologue = [&](__amdgpu_buffer_rsrc_t rows_a0, __amdgpu_buffer_rsrc_t rows_b0) __attribute__((always_inline)) {
+      next_a = rows_a0;  // (never used: K >= 3 tiles, so no stream wraps before the loops below set them)
       next_b = rows_b0;
       ld_a = Stream{rows_a0, 0, wave * 1024};
       ld_b = Stream{rows_b0, 0, B_REGION + wave * 1024};
-      auto load_whole_tile = [&](const Stream& st, const unsigned(&voff)[LPT]) __attribute__((always_inline)) {
-        w4_static_for<0, LPT>([&](auto i_tag) __attribute__((always_inline)) {
-          set_load_target(st, i_tag);
-          asm volatile("s_nop 0");  // the wait state between the write of M0 and its use
-          load_tile_part(st, voff[decltype(i_tag)::value]);
-        });
-      };
       load_whole_tile(ld_a, voff_a);
       load_whole_tile(ld_b, voff_b);
       advance(ld_a, wrap_a, next_a, 0, B_REGION, a_step, a_end, -1);
       advance(ld_b, wrap_b, next_b, B_REGION, LDS_BYTES, b_step, b_end, -1);
       load_whole_tile(ld_a, voff_a);
       advance(ld_a, wrap_a, next_a, 0, B_REGION, a_step, a_end, -1);
+    };
+    // The second half of a tile's last K tile is in set 1.
+    auto drain = [&]() __attribute__((always_inline)) {
+      w4_static_for<0, 64>([&](auto m_tag) __attribute__((always_inline)) {
+        constexpr int m = decltype(m_tag)::value;
+        Mfma::template fma<m>(fb1[m & 7], fa1[m >> 3]);
+      });
+      asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+    };
 
+    if constexpr (LN) {
+      TileCoord tc = ln_tile;
+      prologue(rows_of_a(0, tc), rows_of_b(0, tc));
+      // Scratch of the epilogue: compact (inside the two operand slots the ring leaves free at a tile boundary)
+      // when a band has at most kLnCompactTiles column tiles, else all of LDS -- the host then gives every
+      // workgroup one tile, and nothing is in flight when the K loop ends.
+      const bool compact = p.tiles_n <= kLnCompactTiles;
+      for (;;) {
+        // The streams move on to the workgroup's next tile while this one is multiplied, as in the plain kernel.
+        TileCoord tc_next = tc;
+        const int next_id = ln_next_id(ln_id + tile_step, &tc_next);
+        const bool has_next = next_id < p.ln_ids;  // (uniform)
+        next_a = rows_of_a(has_next ? 0 : 1, tc_next);
+        next_b = rows_of_b(has_next ? 0 : 1, tc_next);
+        k_tile(std::true_type{});
+        for (int h = 1; h < n_k; ++h) k_tile(std::false_type{});
+        // Behind a workgroup's last tile the streams' fills are empty (they touch no memory and return at once): they
+        // are waited for here, so that nothing is on its way into LDS when the epilogue reuses it or the kernel ends.
+        // In front of a further tile the fills are that tile's first operand tiles, and nobody waits for them yet.
+        if (!has_next) wait_vm_and_lds<0>();
+        drain();
+        out = out_tile_of(0, tc);
+        // After K tile h: rd_a / rd_b are the slots of K tile h + 1 (the next tile's first, already there or on
+        // its way, like A of the one after it); the slots K tile h was in are free until the next K loop's first
+        // loads, which come behind a barrier that every wavefront reaches only after its epilogue.
+        const int free_a = rd_a == 0 ? B_REGION - SLOT : rd_a - SLOT;
+        const int free_b = rd_b == B_REGION ? B_REGION + SLOT : B_REGION;
+        layer_norm_epilogue(p, smem, tc, out, compact, free_a, free_b);
+        if (!has_next) break;
+        ln_id = next_id;
+        tc = tc_next;
+        after_epilogue = true;
+      }
+    } else if (g_total > 0) {
+      TileCoord tc_cur = tile_coord(0);
+      prologue(rows_of_a(0, tc_cur), rows_of_b(0, tc_cur));
       for (int j = 0; j < my_tiles; ++j) {
         // The streams move on to tile j + 1 while tile j is multiplied: A in its last but one K tile,
         // B in its last.  With K = 3 tiles that is this very K tile, so the rows come first.
@@ -484,21 +552,13 @@ struct GemmW4 {
         out = out_tile_of(j, tc_j);  // from here on the accumulators belong to tile j
         for (int h = 1; h < n_k; ++h) k_tile(std::false_type{});
       }
-      // Drain: the second half of the last K tile is in set 1; then the last tile's output.
+      // Drain, then the last tile's output.
       wait_vm_and_lds<0>();
-      w4_static_for<0, 64>([&](auto m_tag) __attribute__((always_inline)) {
-        constexpr int m = decltype(m_tag)::value;
-        Mfma::template fma<m>(fb1[m & 7], fa1[m >> 3]);
+      drain();
+      w4_static_for<0, FM * FN / 2>([&](auto o_tag) __attribute__((always_inline)) {
+        constexpr int o = decltype(o_tag)::value;
+        store_pair(std::integral_constant<int, o / 4>{}, std::integral_constant<int, o % 4>{}, std::true_type{});
       });
-      asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
-      if constexpr (!LN) {
-        w4_static_for<0, FM * FN / 2>([&](auto o_tag) __attribute__((always_inline)) {
-          constexpr int o = decltype(o_tag)::value;
-          store_pair(std::integral_constant<int, o / 4>{}, std::integral_constant<int, o % 4>{}, std::true_type{});
-        });
-      } else {
-        layer_norm_epilogue(p, smem, ln_tile, out);
-      }
     }
   }
 
@@ -506,8 +566,30 @@ struct GemmW4 {
   // The same five steps as the kEpiLnFused epilogue of gemm_kernel.h, for this kernel's accumulator layout:
   // row block i of a lane is 32 values (blocks 8 i .. 8 i + 7) of row 128 wm + 16 i + r, in the four groups of
   // 8 columns 128 wn + 32 q + 8 g; a row of the tile is spread over 4 lane groups x 2 wavefronts = 8 slots.
+  // Thread t owns row t of the tile in steps 2 to 4 (256 threads, 256 rows).
+  //
+  // Scratch.  compact: the operand ring keeps running through the tile boundary, so three of the five LDS slots
+  // hold the next tile's first operand tiles (landed or in flight) and only the two slots of the K tile just
+  // multiplied are free: the lane partials (18 KiB) go into the free A slot, behind the 2 KiB that will hold the
+  // rows' final (mean, rstd); the pairs of the band's column tiles (2 KiB per tile: 8 bytes per row) are gathered
+  // into the free B slot (tiles 0 .. 15) and, the lane partials being dead by then, into the free A slot from its
+  // start (tiles 16 .. 31).  A thread only ever touches its own row's 8 bytes of each of those 2 KiB, and it writes
+  // its row's (mean, rstd) when it has merged its pairs, so the last 2 KiB may lie where tile 16's pairs were.
+  // Hence kLnCompactTiles = 32.  Otherwise (up to 64 column tiles) all of LDS is used: the caller has made sure
+  // that nothing is in flight and that no tile follows.
+  //
+  // Why nobody waits for ever when workgroups walk several tiles (one workgroup per CU, all resident): ids of the
+  // band order that are 256 apart belong to one workgroup, which takes them in rising order and publishes a
+  // tile's statistics before it waits for anything.  The tiles of one band lie within fewer than 256 consecutive
+  // ids in each of the three orders (a band group of the padded orders is at most 8 x 32 ids; a band of the plain
+  // order at most 64).  If tile T1 waits for T2 of its band, and T2 has not started because its workgroup is
+  // still waiting at an earlier tile T3, then id(T3) <= id(T2) - 256 < id(T1): every such step leads to a strictly
+  // smaller id, so no chain of waits returns to where it began, and the smallest id in any chain waits only for
+  // tiles whose K loops are running or done.
+  static constexpr int kLnCompactTiles = 32;
   template <typename OutTileT>
-  static __device__ __forceinline__ void layer_norm_epilogue(const GemmParams& p, char* smem, TileCoord tc, const OutTileT& out) {
+  static __device__ __forceinline__ void layer_norm_epilogue(const GemmParams& p, char* smem, TileCoord tc, const OutTileT& out,
+                                                             bool compact, int free_a, int free_b) {
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave & 1, wn = wave >> 1;
@@ -515,6 +597,14 @@ struct GemmW4 {
     const int N = p.N;
     const int col0 = tc.tn * BN;
     constexpr int SLOTS = 8, PITCH = SLOTS + 1;  // (a row of `part` is padded by one pair: see gemm_kernel.h)
+    // Every barrier here is a bare one behind a wait for this wavefront's LDS accesses only: __syncthreads() would
+    // also wait for the next tile's operand loads in flight.  The wait is assembly with a memory clobber: given the
+    // s_waitcnt builtin, the compiler is free to sink the LDS stores in front of it to behind it (it sees no
+    // dependence), and the other wavefronts then read what has not been written yet.
+    auto lds_barrier = [&]() __attribute__((always_inline)) {
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      bare_barrier();
+    };
     // gamma / beta of this lane's four column groups: issued now, used in step 5
     bool q_valid[4];
     vec8 gv[4], bv[4];
@@ -527,9 +617,16 @@ struct GemmW4 {
     }
     const int my_cols = 8 * ((int)q_valid[0] + (int)q_valid[1] + (int)q_valid[2] + (int)q_valid[3]);
     const bool full = col0 + BN <= N;
-    __syncthreads();  // every wavefront is done with the operand slots: LDS is free
-    float* red = (float*)smem;   // [BM][2] tile statistics, later (mean, rstd) of the whole row
-    float* part = red + BM * 2;  // [BM][PITCH][2], later the gathered pairs of the band [tiles_n][BM][2]
+    bare_barrier();  // every wavefront is done with the slots of the last K tile (its fragments are in registers)
+    float* red = (float*)(smem + (compact ? free_a : 0));  // [BM][2]: (mean, rstd) of the whole row, written in step 4
+    float* part = red + BM * 2;                             // [BM][PITCH][2] lane partials
+    // The pairs of this thread's row, one per column tile of the band, 2 KiB apart: tiles 0 .. n0 - 1 from g0 on,
+    // the others from g1 on.
+    const int n0 = compact ? (p.tiles_n < 16 ? p.tiles_n : 16) : p.tiles_n;
+    const int n1 = p.tiles_n - n0;
+    float* g0 = (compact ? (float*)(smem + free_b) : part) + tid * 2;
+    float* g1 = red + tid * 2;
+    constexpr int GP = BM * 2;  // floats from one tile's pairs to the next
     // 1. per-lane (mean, M2) over the lane's columns of each of its rows, dropped into LDS
     w4_static_for<0, FM>([&](auto i_tag) __attribute__((always_inline)) {
       constexpr int i = decltype(i_tag)::value;
@@ -551,89 +648,176 @@ struct GemmW4 {
       part[(rl * PITCH + wn * 4 + g) * 2 + 0] = mean;
       part[(rl * PITCH + wn * 4 + g) * 2 + 1] = m2;
     });
-    __syncthreads();
+    lds_barrier();
     // 2. one thread per row merges the 8 slots in a fixed order (Chan's update) ...
-    {
-      const int rl = tid;  // 256 threads, 256 rows
-      float mean = 0.0f, m2 = 0.0f, n_acc = 0.0f;
-      if (full) {
-        // every slot covers 32 columns: the mean of the slot means, then M2 about it -- the merge below for
-        // equal counts, in the same fixed order, without its divisions
-        float mw[SLOTS], qw[SLOTS];
+    const int rl = tid;
+    float mean = 0.0f, m2 = 0.0f, n_acc = 0.0f;
+    if (full) {
+      // every slot covers 32 columns: the mean of the slot means, then M2 about it -- the merge below for
+      // equal counts, in the same fixed order, without its divisions
+      float mw[SLOTS], qw[SLOTS];
 #pragma unroll
-        for (int slot = 0; slot < SLOTS; ++slot) {
-          mw[slot] = part[(rl * PITCH + slot) * 2 + 0];
-          qw[slot] = part[(rl * PITCH + slot) * 2 + 1];
-          mean += mw[slot];
-        }
-        mean *= 1.0f / (float)SLOTS;
+      for (int slot = 0; slot < SLOTS; ++slot) {
+        mw[slot] = part[(rl * PITCH + slot) * 2 + 0];
+        qw[slot] = part[(rl * PITCH + slot) * 2 + 1];
+        mean += mw[slot];
+      }
+      mean *= 1.0f / (float)SLOTS;
 #pragma unroll
-        for (int slot = 0; slot < SLOTS; ++slot) {
-          const float d = mw[slot] - mean;
-          m2 += qw[slot] + 32.0f * d * d;
-        }
+      for (int slot = 0; slot < SLOTS; ++slot) {
+        const float d = mw[slot] - mean;
+        m2 += qw[slot] + 32.0f * d * d;
       }
-#pragma unroll
-      for (int slot = 0; slot < (full ? 0 : SLOTS); ++slot) {
-        int cnt = 0;
-#pragma unroll
-        for (int q = 0; q < 4; ++q) cnt += (col0 + (slot >> 2) * 128 + 32 * q + 8 * (slot & 3) < N) ? 8 : 0;
-        if (cnt == 0) continue;
-        const float mw = part[(rl * PITCH + slot) * 2 + 0];
-        const float qw = part[(rl * PITCH + slot) * 2 + 1];
-        const float nb = (float)cnt;
-        const float tot = n_acc + nb;
-        const float delta = mw - mean;
-        mean += delta * (nb / tot);
-        m2 += qw + delta * delta * (n_acc * nb / tot);
-        n_acc = tot;
-      }
-      // ... and publishes the tile's pair (gemm_kernel.h: ln_publish, two tagged 8-byte words per row)
-      const unsigned tag = ln_launch_tag(p);
-      ln_sign_header(p, tag);
-      ln_publish(p, ((size_t)tc.tm * p.tiles_n + tc.tn) * BM + rl, mean, m2, tag);
-      __syncthreads();  // `part` is free again
-      // 3. gather the band's pairs into LDS, polling (boundedly) what is not published yet
-      float* gathered = part;
-      // (8 slots in flight; 16 measure the same and cost scalar registers parked in vector lanes.  The codegen
-      // test watches this kernel: a compiler short of ordinary registers parks values in accumulation registers,
-      // i.e. in the accumulators.)
-      ln_gather<NT, 8>(p, tag, (size_t)tc.tm * p.tiles_n * BM, p.tiles_n * BM, tid, (unsigned long long*)gathered);
-      __syncthreads();
-      // 4. merge in tile order -> (mean, rstd) of the whole row
-      mean = 0.0f;
-      m2 = 0.0f;
-      n_acc = 0.0f;
-      const bool even_tiles = (N % BN) == 0;  // every column tile is full: equal weights
-      if (even_tiles) {
-        for (int t = 0; t < p.tiles_n; ++t) mean += gathered[((size_t)t * BM + rl) * 2 + 0];
-        mean *= 1.0f / (float)p.tiles_n;
-        for (int t = 0; t < p.tiles_n; ++t) {
-          const float d = gathered[((size_t)t * BM + rl) * 2 + 0] - mean;
-          m2 += gathered[((size_t)t * BM + rl) * 2 + 1] + (float)BN * d * d;
-        }
-      }
-      for (int t = 0; t < (even_tiles ? 0 : p.tiles_n); ++t) {
-        int cw = N - t * BN;
-        cw = cw > BN ? BN : cw;
-        const float mw = gathered[((size_t)t * BM + rl) * 2 + 0];
-        const float qw = gathered[((size_t)t * BM + rl) * 2 + 1];
-        const float nb = (float)cw;
-        const float tot = n_acc + nb;
-        const float delta = mw - mean;
-        mean += delta * (nb / tot);
-        m2 += qw + delta * delta * (n_acc * nb / tot);
-        n_acc = tot;
-      }
-      red[rl * 2 + 0] = mean;
-      red[rl * 2 + 1] = even_tiles ? __builtin_amdgcn_rsqf(m2 * (1.0f / (float)N) + p.eps) : 1.0f / sqrtf(m2 / (float)N + p.eps);
     }
-    __syncthreads();
-    // 5. normalise the accumulators and store Y: a pair of blocks is one 16-byte store per lane
+#pragma unroll
+    for (int slot = 0; slot < (full ? 0 : SLOTS); ++slot) {
+      int cnt = 0;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) cnt += (col0 + (slot >> 2) * 128 + 32 * q + 8 * (slot & 3) < N) ? 8 : 0;
+      if (cnt == 0) continue;
+      const float mw = part[(rl * PITCH + slot) * 2 + 0];
+      const float qw = part[(rl * PITCH + slot) * 2 + 1];
+      const float nb = (float)cnt;
+      const float tot = n_acc + nb;
+      const float delta = mw - mean;
+      mean += delta * (nb / tot);
+      m2 += qw + delta * delta * (n_acc * nb / tot);
+      n_acc = tot;
+    }
+    // ... and publishes the tile's pair (gemm_kernel.h: ln_publish, two tagged 8-byte words per row)
+    const unsigned tag = ln_launch_tag(p);
+    ln_sign_header(p, tag);
+    ln_publish(p, ((size_t)tc.tm * p.tiles_n + tc.tn) * BM + rl, mean, m2, tag);
+    lds_barrier();  // `part` is free again
+    // 3. gather the pairs of this thread's row from the band's other column tiles into LDS, 16 tiles' worth in
+    //    flight at once, fetching again -- boundedly -- what does not carry the launch's tag yet (the protocol of
+    //    gemm_kernel.h's ln_gather).  A batch costs a round trip to memory (1.3 us measured), whatever its size: a band
+    //    of 32 column tiles took 5.1-5.7 us in batches of 8.  (32 in flight need 128 registers, and the compiler then
+    //    parks values in accumulation registers, i.e. in the accumulators: the codegen test watches for that.)  The
+    {
+      const unsigned long long* w0s = (const unsigned long long*)p.stats + (size_t)tc.tm * p.tiles_n * BM + rl;
+      const unsigned long long* w1s = (const unsigned long long*)p.next_stats + (size_t)tc.tm * p.tiles_n * BM + rl;
+      const unsigned not_tag = ~tag;
+      constexpr int INFLIGHT = 16;
+      int polls = 0;
+      for (int t0 = 0; t0 < p.tiles_n; t0 += INFLIGHT) {
+        unsigned long long a[INFLIGHT], b[INFLIGHT];
+        unsigned missing = 0;  // bit u: column tile t0 + u is still to be fetched
+#pragma unroll
+        for (int u = 0; u < INFLIGHT; ++u) {
+          a[u] = 0;
+          b[u] = 0;
+          missing |= (t0 + u < p.tiles_n) ? (1u << u) : 0u;  // (the tile's own pair comes back like the others')
+        }
+        while (missing != 0) {
+#pragma unroll
+          for (int u = 0; u < INFLIGHT; ++u) {
+            if (missing & (1u << u)) {
+              a[u] = __hip_atomic_load(w0s + (size_t)(t0 + u) * BM, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+              b[u] = __hip_atomic_load(w1s + (size_t)(t0 + u) * BM, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+          }
+          // (a negative limit: treat everything as unpublished -- how the host forces the time-out in a test)
+#pragma unroll
+          for (int u = 0; u < INFLIGHT; ++u)
+            if ((missing & (1u << u)) && (unsigned)(a[u] >> 32) == tag && (unsigned)(b[u] >> 32) == not_tag && p.spin_limit >= 0)
+              missing &= ~(1u << u);
+          if (missing == 0) break;
+          if (++polls > p.spin_limit) {
+            p.timeout_flag[kLnHdrTimeout] = (int)tag;
+#pragma unroll
+            for (int u = 0; u < INFLIGHT; ++u)
+              if (missing & (1u << u)) {
+                a[u] = 0x7fc00000ull;
+                b[u] = 0x7fc00000ull;
+              }
+            break;
+          }
+          for (int z = 0; z < (polls < 8 ? polls : 8); ++z) __builtin_amdgcn_s_sleep(8);
+        }
+#pragma unroll
+        for (int u = 0; u < INFLIGHT; ++u) {
+          const int t = t0 + u;
+          if (t < p.tiles_n) {
+            float* at = t < n0 ? g0 + t * GP : g1 + (t - n0) * GP;
+            at[0] = __uint_as_float((unsigned)a[u]);
+            at[1] = __uint_as_float((unsigned)b[u]);
+          }
+        }
+      }
+    }
+    // (the pairs a thread merges are the ones it stored itself: no barrier in between)
+    // 4. merge in tile order -> (mean, rstd) of the whole row.  The pairs come back from LDS 32 at a time, all reads of
+    //    a chunk in flight together (a loop that waits for one read per step is bound by the latency of each).
+    mean = 0.0f;
+    m2 = 0.0f;
+    n_acc = 0.0f;
+    const bool even_tiles = (N % BN) == 0;  // every column tile is full: equal weights
+    constexpr int CH = 16;
+    static_assert(CH == 16, "a chunk is what the free B slot holds in the compact layout");
+    float mw[CH], qw[CH];
+    auto load_chunk = [&](int c) __attribute__((always_inline)) {
+      // tiles 16 c .. 16 c + 15: from g0 on; in the compact layout the second chunk starts at g1.  (Every pointer
+      // formed here lies inside LDS: an address below its start, even as an intermediate value to which an
+      // instruction's offset field is added, reads as zeros.)
+      const float* base = c == 0 ? g0 : (compact ? g1 : g0 + CH * GP) + (c - 1) * CH * GP;
+#pragma unroll
+      for (int u = 0; u < CH; ++u) {
+        const bool there = c * CH + u < p.tiles_n;  // (uniform)
+        mw[u] = there ? base[u * GP] : 0.0f;
+        qw[u] = there ? base[u * GP + 1] : 0.0f;
+      }
+    };
+    const int chunks = (p.tiles_n + CH - 1) / CH;
+    if (even_tiles) {
+      for (int c = 0; c < chunks; ++c) {
+        load_chunk(c);
+#pragma unroll
+        for (int u = 0; u < CH; ++u) mean += mw[u];  // (adding the zeros of absent tiles changes nothing)
+      }
+      mean *= 1.0f / (float)p.tiles_n;
+      for (int c = 0; c < chunks; ++c) {
+        if (chunks > 1) load_chunk(c);
+#pragma unroll
+        for (int u = 0; u < CH; ++u) {
+          const float d = mw[u] - mean;
+          m2 += (c * CH + u < p.tiles_n) ? qw[u] + (float)BN * d * d : 0.0f;
+        }
+      }
+    } else {
+      for (int c = 0; c < chunks; ++c) {
+        load_chunk(c);
+#pragma unroll
+        for (int u = 0; u < CH; ++u) {
+          const int t = c * CH + u;
+          if (t < p.tiles_n) {  // (uniform)
+            int cw = N - t * BN;
+            cw = cw > BN ? BN : cw;
+            const float nb = (float)cw;
+            const float tot = n_acc + nb;
+            const float delta = mw[u] - mean;
+            mean += delta * (nb / tot);
+            m2 += qw[u] + delta * delta * (n_acc * nb / tot);
+            n_acc = tot;
+          }
+        }
+      }
+    }
+    red[rl * 2 + 0] = mean;
+    red[rl * 2 + 1] = even_tiles ? __builtin_amdgcn_rsqf(m2 * (1.0f / (float)N) + p.eps) : 1.0f / sqrtf(m2 / (float)N + p.eps);
+    lds_barrier();
+    // 5. normalise the accumulators and store Y: a pair of blocks is one 16-byte store per lane.  The stores go
+    //    through the L2 to memory at once: nothing hides those of a workgroup's last tile, and a kernel ends only
+    //    when its dirty lines have left the L2 (4096^3, one tile per workgroup: 105.7 -> 103.7 us); under a next
+    //    tile's K loop the kind of store measures the same.  One copy of this code for every tile, whatever
+    //    follows it: two instantiations of the same source need not round alike (the compiler fuses the last
+    //    multiply-add with the conversion to 16 bits in one place and not in another, which differs on ties), and
+    //    a workgroup that walks its tiles must give the bits of one that has a single tile.
+    constexpr int AUX = kAuxDeviceScope;
     w4_static_for<0, FM>([&](auto i_tag) __attribute__((always_inline)) {
       constexpr int i = decltype(i_tag)::value;
-      const int rl = wm * 128 + 16 * i + r;
-      const float mean = red[rl * 2 + 0], rstd = red[rl * 2 + 1];
+      const int row = wm * 128 + 16 * i + r;
+      const float row_mean = red[row * 2 + 0], rstd = red[row * 2 + 1];
       const int skip = i * 16 * N * 2;
       const int left = out.bytes - skip;
       const __amdgpu_buffer_rsrc_t rsrc = make_rsrc(out.base + skip, left > 0 ? (unsigned)left : 0u);
@@ -642,11 +826,14 @@ struct GemmW4 {
         vec8 v;
         w4_static_for<0, 8>([&](auto e_tag) __attribute__((always_inline)) {
           constexpr int e = decltype(e_tag)::value;
-          v[e] = (T)((w4_acc_read<4 * (8 * i + 2 * q) + e>() - mean) * rstd * (float)gv[q][e] + (float)bv[q][e]);
+          v[e] = (T)((w4_acc_read<4 * (8 * i + 2 * q) + e>() - row_mean) * rstd * (float)gv[q][e] + (float)bv[q][e]);
         });
-        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(i32x4, v), rsrc, (int)out.voff[q], 0, kAuxDeviceScope);
+        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(i32x4, v), rsrc, (int)out.voff[q], 0, AUX);
       });
     });
+    // (the reads of `red` above are behind the next K loop's first barrier only in program order: a wavefront must
+    // have them before the loads behind that barrier overwrite the slot)
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
   }
 };
 

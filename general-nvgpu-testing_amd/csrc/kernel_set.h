@@ -146,8 +146,10 @@ constexpr int kW4MinK = 192;
 hipError_t launch_gemm_w4(const GemmParams& p, int dtype, dim3 grid, hipStream_t stream);
 // The same with B stored [K][N]; additionally K * N * 2 < 2^31.
 hipError_t launch_gemm_w4_kmajor(const GemmParams& p, int dtype, dim3 grid, hipStream_t stream);
-// Its fused GEMM+LayerNorm form: one workgroup per tile, grid and parameters as for the kEpiLnFused kernels;
-// gamma and beta 16-byte aligned as well.
+// Its fused GEMM+LayerNorm form: parameters as for the kEpiLnFused kernels plus ln_ids, the number of ids of the band
+// order (padding included); a grid of ln_ids workgroups gives every workgroup one tile, a smaller grid (one
+// workgroup per CU) makes them walk, which needs tiles_n <= kW4LnCompactTiles.  gamma and beta 16-byte aligned as well.
+constexpr int kW4LnCompactTiles = 32;
 hipError_t launch_gemm_w4_ln(const GemmParams& p, int dtype, dim3 grid, hipStream_t stream);
 // Measurement only: the split-K partial kernel of the 64 x 128 (wave 32 x 64) or 64 x 64 (wave 32 x 32) tile, deep
 // pipeline, fp16, with its loads and fragment reads but no MFMAs and no stores (kEpiProbeLoads); hipErrorInvalidValue

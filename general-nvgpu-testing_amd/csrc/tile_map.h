@@ -236,6 +236,44 @@ BEAM_HD TileCoord tile_of_workgroup(int wg, int tiles_m, int tiles_n, int group_
   return grouped_tile(xcd_remap(wg, tiles_m * tiles_n), tiles_m, tiles_n, group_m, dv);
 }
 
+// The three workgroup orders of the fused GEMM+LayerNorm as one map with its divisions done by multiplication (what
+// the kernels call; a host test walks it against the defining functions above over every id of many grids).
+//   group_n > 0: band_block_tile with gb = group_m, gc = group_n;  group_n == 0: band_xcd_tile with bx = group_m;
+//   group_n < 0: band after band, id = band * tiles_n + column, no padding.
+BEAM_HD TileDivs band_order_divs(int tiles_n, int group_m, int group_n) {
+  TileDivs d;
+  const int g = group_m < 1 ? 1 : group_m;
+  d.group = make_fast_div((unsigned)(g * (group_n > 0 ? group_n : tiles_n)));  // ids of one XCD per band group
+  d.rows = make_fast_div((unsigned)g);
+  d.rows_last = d.rows;
+  d.tiles = make_fast_div((unsigned)(tiles_n < 1 ? 1 : tiles_n));
+  return d;
+}
+BEAM_HD TileCoord band_order_tile(int id, int tiles_m, int tiles_n, int group_m, int group_n, const TileDivs& dv) {
+  TileCoord t;
+  if (group_n < 0) {
+    t.tm = (int)fast_div((unsigned)id, dv.tiles);
+    t.tn = id - t.tm * tiles_n;
+    return t;
+  }
+  const int xcd = id % kNumXcd;
+  const int local = id / kNumXcd;
+  const int per_group = group_m * (group_n > 0 ? group_n : tiles_n);
+  const int bg = (int)fast_div((unsigned)local, dv.group);
+  const int within = local - bg * per_group;
+  const int col = (int)fast_div((unsigned)within, dv.rows);  // within / group_m
+  const int band = within - col * group_m;
+  if (group_n > 0) {
+    t.tm = bg * group_m + band;
+    t.tn = xcd * group_n + col;
+  } else {
+    t.tm = (bg * kNumXcd + xcd) * group_m + band;
+    t.tn = col;
+  }
+  if (t.tm >= tiles_m || t.tn >= tiles_n) t.tm = -1;
+  return t;
+}
+
 // K range [begin, end) of split slice `z` out of `splits`: every slice gets the same whole
 // number of kBK-wide K tiles (the last ones may be short or empty). Matches the CUTLASS
 // partitioning the reference relies on (cuda/cutlass_kernels/cutlass_gemmrc_splitk.cu:95-99).

@@ -64,6 +64,10 @@ int beam_dbg_kmajor_lds_offset(int k, int n, int block_n);
  * and beta 16-byte aligned).  The entry point computes its requirement with the same function; the workspace queries
  * are tested against it.  0 on error. */
 size_t beam_dbg_ln_plan_bytes(int M, int N, int K, const beam_tile_cfg* cfg, int mode, int plain, int capturing, int wide_io);
+/* on = 0: the fused GEMM+LayerNorm of the 256 x 256 tile of four wavefronts runs one workgroup per tile whatever the
+ * size of the problem; on != 0 (the default): from more tiles than CUs on, one workgroup per CU walks its tiles.
+ * Same bits either way: for tests that compare the two. */
+int beam_dbg_set_ln_walk(int on);
 /* For tests on a host without a GPU: the CU count the library's choices assume when no device could be probed
  * (refused once a device has been). */
 int beam_dbg_assume_compute_units(int compute_units);
@@ -79,6 +83,10 @@ int beam_dbg_w4_kmajor_read_offset(int wn, int b, int g, int e, int q);
  * the id is padding), and the size of that grid. */
 int beam_dbg_band_block_tile(int wg, int tiles_m, int tiles_n, int gb, int gc, int* tm, int* tn);
 int beam_dbg_band_block_grid(int tiles_m, int gb, int gc);
+/* The three orders as the kernels compute them, divisions done by multiplication: group_n > 0 is the band-block
+ * order with gb = group_m and gc = group_n, group_n == 0 the whole-bands order with bx = group_m, group_n < 0 plain
+ * band after band (id = band * tiles_n + column). */
+int beam_dbg_band_order_tile(int id, int tiles_m, int tiles_n, int group_m, int group_n, int* tm, int* tn);
 /* The same for the order that keeps whole bands (bx at a time) on one XCD, used when a band is
  * short enough for it. */
 int beam_dbg_band_xcd_tile(int wg, int tiles_m, int tiles_n, int bx, int* tm, int* tn);

@@ -321,6 +321,33 @@ def test_two_fused_launches_share_the_device(gpu, beamc):
                 t.free()
 
 
+@pytest.mark.parametrize("shape,dtype", [((8192, 8192, 256), F16), ((6144, 6144, 192), F16), ((5000, 7000, 320), F16),
+                                         ((16500, 2048, 256), BF16), ((4100, 8192, 448), BF16), ((9000, 4352, 192), F16)])
+def test_ln_walking_tiles_matches_one_tile_per_workgroup(gpu, beamc, oracle, shape, dtype):
+    """More 256 x 256 tiles than CUs: one workgroup per CU walks its tiles (the next tile's operands arrive while the
+    band's statistics are exchanged) and gives, bit for bit, what one workgroup per tile gives; the oracle agrees.
+    The shapes cover the three workgroup orders (band blocks over all XCDs, whole bands per XCD, band after band),
+    bands of 32 column tiles (the most the walking form takes), ragged edges in M and N, K of 3 to 7 tiles (the
+    operand streams change tile inside a tile's first K tiles), and workgroups with 2, 3 and 5 tiles."""
+    M, N, K = shape
+    a, b, g_, bt = make_ln_inputs(beamc, M, N, K, dtype, 51)
+    ref = oracle.gemmrc_ln(a, b, g_, bt, 1e-5, dtype)
+    cfg = beamc.TileConfig(256, 256, 128, 128)
+    L = beamc.lib
+    try:
+        assert L.beam_dbg_set_ln_walk(0) == 0
+        one_each = run_ln(beamc, a, b, g_, bt, dtype, config=cfg, mode=beamc.LN_FUSED)
+        assert L.beam_dbg_set_ln_walk(1) == 0
+        for rep in range(3):
+            walked = run_ln(beamc, a, b, g_, bt, dtype, config=cfg, mode=beamc.LN_FUSED)
+            assert (walked == one_each).all(), f"{shape}: walking differs from one workgroup per tile (repetition {rep})"
+    finally:
+        L.beam_dbg_set_ln_walk(1)
+    check_ln(oracle, walked, ref, dtype, f"{shape} dtype {dtype} walking")
+    # and the call that names nothing (whatever tile and form the library takes for it)
+    check_ln(oracle, run_ln(beamc, a, b, g_, bt, dtype), ref, dtype, f"{shape} dtype {dtype} default call")
+
+
 def test_ln_default_call_never_lacks_workspace(gpu, beamc, oracle):
     """M=1024, N=8192, K=2048 without a tile: the library's tile for that K takes the two-pass path (32 column
     tiles of 256 fit the fused kernel, but the tile chosen is another); the Python wrapper sizes its buffer for

@@ -472,6 +472,43 @@ def test_splitk_workspace_query_covers_every_small_tile(beamc):
                     assert have >= 4 * (64 + tiles * parts * S), (M, N, S, bm, bn)
 
 
+def test_band_orders_by_multiplication_match_their_definitions(beamc):
+    """The fused GEMM+LayerNorm kernels turn a workgroup id into a tile with divisions done as multiplications; over
+    every id of many grids that is the band-block order, the whole-bands-per-XCD order and the plain band-after-band
+    order as tile_map.h defines them (padding ids included), and in each order the ids of one band lie within fewer
+    than 256 of each other -- what the walking form's freedom from circular waits rests on."""
+    import ctypes
+    L = beamc.lib
+    a, b, c, d = (ctypes.c_int() for _ in range(4))
+    for tiles_m, tiles_n in [(1, 1), (3, 5), (16, 16), (32, 32), (33, 31), (24, 24), (65, 8), (20, 28), (7, 64), (40, 3), (36, 17)]:
+        gc = -(-tiles_n // 8)
+        gb = min(32 // gc, tiles_m)
+        spans = {}
+        grid = L.beam_dbg_band_block_grid(tiles_m, gb, gc)
+        for wg in range(grid):
+            assert L.beam_dbg_band_block_tile(wg, tiles_m, tiles_n, gb, gc, ctypes.byref(a), ctypes.byref(b)) == 0
+            assert L.beam_dbg_band_order_tile(wg, tiles_m, tiles_n, gb, gc, ctypes.byref(c), ctypes.byref(d)) == 0
+            assert (a.value < 0 and c.value < 0) or (a.value, b.value) == (c.value, d.value), (tiles_m, tiles_n, wg)
+            if a.value >= 0:
+                lo, hi = spans.get(a.value, (wg, wg))
+                spans[a.value] = (min(lo, wg), max(hi, wg))
+        assert len(spans) == tiles_m and all(hi - lo < 256 for lo, hi in spans.values())
+        if tiles_n <= 32:
+            bx, spans = 32 // tiles_n, {}
+            grid = L.beam_dbg_band_xcd_grid(tiles_m, tiles_n, bx)
+            for wg in range(grid):
+                assert L.beam_dbg_band_xcd_tile(wg, tiles_m, tiles_n, bx, ctypes.byref(a), ctypes.byref(b)) == 0
+                assert L.beam_dbg_band_order_tile(wg, tiles_m, tiles_n, bx, 0, ctypes.byref(c), ctypes.byref(d)) == 0
+                assert (a.value < 0 and c.value < 0) or (a.value, b.value) == (c.value, d.value), (tiles_m, tiles_n, wg)
+                if a.value >= 0:
+                    lo, hi = spans.get(a.value, (wg, wg))
+                    spans[a.value] = (min(lo, wg), max(hi, wg))
+            assert len(spans) == tiles_m and all(hi - lo < 256 for lo, hi in spans.values())
+        for wg in range(tiles_m * tiles_n):
+            assert L.beam_dbg_band_order_tile(wg, tiles_m, tiles_n, 1, -1, ctypes.byref(c), ctypes.byref(d)) == 0
+            assert (c.value, d.value) == (wg // tiles_n, wg % tiles_n)
+
+
 def test_division_by_multiplication(beamc):
     """The kernels divide by launch constants with a multiply-high and a shift (tile_map.h: FastDiv): exact for
     every numerator below 2^31, checked on small numbers exhaustively, around every multiple of the divisor that a
