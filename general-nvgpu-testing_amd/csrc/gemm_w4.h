@@ -747,58 +747,70 @@ struct GemmW4 {
       }
     }
     // (the pairs a thread merges are the ones it stored itself: no barrier in between)
-    // 4. merge in tile order -> (mean, rstd) of the whole row.  The pairs come back from LDS 32 at a time, all reads of
-    //    a chunk in flight together (a loop that waits for one read per step is bound by the latency of each).
+    // 4. merge in tile order -> (mean, rstd) of the whole row.  The pairs come back from LDS eight at a time, every
+    //    read of a batch issued before the first is used (a loop that waits for one read per step is bound by the
+    //    latency of each), and none of them conditional (the compiler turns a conditional read into a branch): a
+    //    batch that reaches past the last tile reads the last tile again, with weight zero.
     mean = 0.0f;
     m2 = 0.0f;
     n_acc = 0.0f;
     const bool even_tiles = (N % BN) == 0;  // every column tile is full: equal weights
-    constexpr int CH = 16;
-    static_assert(CH == 16, "a chunk is what the free B slot holds in the compact layout");
+    constexpr int CH = 8;
     float mw[CH], qw[CH];
-    auto load_chunk = [&](int c) __attribute__((always_inline)) {
-      // tiles 16 c .. 16 c + 15: from g0 on; in the compact layout the second chunk starts at g1.  (Every pointer
-      // formed here lies inside LDS: an address below its start, even as an intermediate value to which an
-      // instruction's offset field is added, reads as zeros.)
-      const float* base = c == 0 ? g0 : (compact ? g1 : g0 + CH * GP) + (c - 1) * CH * GP;
+    // tiles t0 .. t0 + CH - 1 of the region that starts at `base` and holds n tiles
+    auto load_batch = [&](const float* base, int n, int t0, bool with_m2) __attribute__((always_inline)) {
 #pragma unroll
       for (int u = 0; u < CH; ++u) {
-        const bool there = c * CH + u < p.tiles_n;  // (uniform)
-        mw[u] = there ? base[u * GP] : 0.0f;
-        qw[u] = there ? base[u * GP + 1] : 0.0f;
+        const int t = t0 + u < n ? t0 + u : n - 1;  // (uniform)
+        mw[u] = base[t * GP];
+        if (with_m2) qw[u] = base[t * GP + 1];
       }
     };
-    const int chunks = (p.tiles_n + CH - 1) / CH;
+    // the two regions in tile order: (g0, n0 tiles, first tile 0), (g1, n1 tiles, first tile n0)
     if (even_tiles) {
-      for (int c = 0; c < chunks; ++c) {
-        load_chunk(c);
 #pragma unroll
-        for (int u = 0; u < CH; ++u) mean += mw[u];  // (adding the zeros of absent tiles changes nothing)
+      for (int reg = 0; reg < 2; ++reg) {
+        const float* base = reg == 0 ? g0 : g1;
+        const int n = reg == 0 ? n0 : n1;
+        for (int t0 = 0; t0 < n; t0 += CH) {
+          load_batch(base, n, t0, false);
+#pragma unroll
+          for (int u = 0; u < CH; ++u) mean += t0 + u < n ? mw[u] : 0.0f;
+        }
       }
       mean *= 1.0f / (float)p.tiles_n;
-      for (int c = 0; c < chunks; ++c) {
-        if (chunks > 1) load_chunk(c);
 #pragma unroll
-        for (int u = 0; u < CH; ++u) {
-          const float d = mw[u] - mean;
-          m2 += (c * CH + u < p.tiles_n) ? qw[u] + (float)BN * d * d : 0.0f;
+      for (int reg = 0; reg < 2; ++reg) {
+        const float* base = reg == 0 ? g0 : g1;
+        const int n = reg == 0 ? n0 : n1;
+        for (int t0 = 0; t0 < n; t0 += CH) {
+          load_batch(base, n, t0, true);
+#pragma unroll
+          for (int u = 0; u < CH; ++u) {
+            const float d = mw[u] - mean;
+            m2 += t0 + u < n ? qw[u] + (float)BN * d * d : 0.0f;
+          }
         }
       }
     } else {
-      for (int c = 0; c < chunks; ++c) {
-        load_chunk(c);
 #pragma unroll
-        for (int u = 0; u < CH; ++u) {
-          const int t = c * CH + u;
-          if (t < p.tiles_n) {  // (uniform)
-            int cw = N - t * BN;
-            cw = cw > BN ? BN : cw;
-            const float nb = (float)cw;
-            const float tot = n_acc + nb;
-            const float delta = mw[u] - mean;
-            mean += delta * (nb / tot);
-            m2 += qw[u] + delta * delta * (n_acc * nb / tot);
-            n_acc = tot;
+      for (int reg = 0; reg < 2; ++reg) {
+        const float* base = reg == 0 ? g0 : g1;
+        const int n = reg == 0 ? n0 : n1;
+        for (int t0 = 0; t0 < n; t0 += CH) {
+          load_batch(base, n, t0, true);
+#pragma unroll
+          for (int u = 0; u < CH; ++u) {
+            if (t0 + u < n) {  // (uniform)
+              int cw = N - ((reg == 0 ? 0 : n0) + t0 + u) * BN;
+              cw = cw > BN ? BN : cw;
+              const float nb = (float)cw;
+              const float tot = n_acc + nb;
+              const float delta = mw[u] - mean;
+              mean += delta * (nb / tot);
+              m2 += qw[u] + delta * delta * (n_acc * nb / tot);
+              n_acc = tot;
+            }
           }
         }
       }
