@@ -633,8 +633,11 @@ size_t beam_splitk_workspace_bytes(int M, int N, int split_k) {
   return align_up(splitk_partial_bytes(M, N, split_k), 256) + (size_t)sk_sync_bytes(M, N, split_k);
 }
 
-// 1: the fused GEMM+LayerNorm of the 4-wavefront kernel always runs one workgroup per tile (testing: beam_dbg_set_ln_walk)
-static std::atomic<int> g_ln_no_walk{0};
+// 1: the fused GEMM+LayerNorm of the 4-wavefront kernel always runs one workgroup per tile (beam_set_ln_walk)
+static std::atomic<int> g_ln_no_walk{[] {
+  const char* e = getenv("BEAM_LN_WALK");
+  return e && *e == '0' ? 1 : 0;
+}()};
 
 // 0: one launch where it applies, 1: always the partial kernel followed by the reduce kernel
 static std::atomic<int> g_splitk_two_launches{[] {
@@ -990,7 +993,7 @@ size_t beam_dbg_ln_plan_bytes(int M, int N, int K, const beam_tile_cfg* cfg, int
   return plan.need;
 }
 
-int beam_dbg_set_ln_walk(int on) {
+int beam_set_ln_walk(int on) {
   g_ln_no_walk.store(on ? 0 : 1);
   return BEAM_OK;
 }

@@ -207,6 +207,14 @@ int beam_gemmrc_ln_timed_out(const void* ws, void* stream, int* timed_out);
  * path is exercised without hanging anything.  The same number bounds the wait of the reducing workgroups
  * of the one-launch split-K (polls of a tile's flags). */
 int beam_set_ln_spin_limit(int polls);
+/* How the fused kernel of the 256 x 256 tile of four wavefronts covers a problem of more tiles than CUs.
+ * on != 0 (the default; environment: BEAM_LN_WALK=0 turns it off): one workgroup per CU walks its tiles, the next
+ * tile's first operands arriving while the band's statistics are exchanged.  Every workgroup of the launch must then
+ * be resident at once: on a device that other work occupies in part, bands whose workgroups were not placed time
+ * out (NaN rows, beam_gemmrc_ln_timed_out; beam_gemmrc_ln_checked repeats the call as two passes).  on = 0: one
+ * workgroup per tile in band order, which finishes band by band on whatever part of the device it gets.  The two
+ * forms give the same bits and measure within 2% of each other. */
+int beam_set_ln_walk(int on);
 
 /* ---- GEMM with an independent elementwise job hidden in its K loop ------------------------ */
 

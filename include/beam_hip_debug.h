@@ -64,10 +64,6 @@ int beam_dbg_kmajor_lds_offset(int k, int n, int block_n);
  * and beta 16-byte aligned).  The entry point computes its requirement with the same function; the workspace queries
  * are tested against it.  0 on error. */
 size_t beam_dbg_ln_plan_bytes(int M, int N, int K, const beam_tile_cfg* cfg, int mode, int plain, int capturing, int wide_io);
-/* on = 0: the fused GEMM+LayerNorm of the 256 x 256 tile of four wavefronts runs one workgroup per tile whatever the
- * size of the problem; on != 0 (the default): from more tiles than CUs on, one workgroup per CU walks its tiles.
- * Same bits either way: for tests that compare the two. */
-int beam_dbg_set_ln_walk(int on);
 /* For tests on a host without a GPU: the CU count the library's choices assume when no device could be probed
  * (refused once a device has been). */
 int beam_dbg_assume_compute_units(int compute_units);

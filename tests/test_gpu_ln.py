@@ -335,14 +335,14 @@ def test_ln_walking_tiles_matches_one_tile_per_workgroup(gpu, beamc, oracle, sha
     cfg = beamc.TileConfig(256, 256, 128, 128)
     L = beamc.lib
     try:
-        assert L.beam_dbg_set_ln_walk(0) == 0
+        assert L.beam_set_ln_walk(0) == 0
         one_each = run_ln(beamc, a, b, g_, bt, dtype, config=cfg, mode=beamc.LN_FUSED)
-        assert L.beam_dbg_set_ln_walk(1) == 0
+        assert L.beam_set_ln_walk(1) == 0
         for rep in range(3):
             walked = run_ln(beamc, a, b, g_, bt, dtype, config=cfg, mode=beamc.LN_FUSED)
             assert (walked == one_each).all(), f"{shape}: walking differs from one workgroup per tile (repetition {rep})"
     finally:
-        L.beam_dbg_set_ln_walk(1)
+        L.beam_set_ln_walk(1)
     check_ln(oracle, walked, ref, dtype, f"{shape} dtype {dtype} walking")
     # and the call that names nothing (whatever tile and form the library takes for it)
     check_ln(oracle, run_ln(beamc, a, b, g_, bt, dtype), ref, dtype, f"{shape} dtype {dtype} default call")
