@@ -548,8 +548,9 @@ int cli_probe_mfma(const Args& a) {
   }
   const int mfma = shape == "32x32x16" ? BEAM_MFMA_32X32X16 : BEAM_MFMA_16X16X32;
   const int kind = data == "zeros" ? BEAM_PROBE_DATA_ZEROS : BEAM_PROBE_DATA_NORMAL;
-  const int passes = a.num("passes", 1600), iters = a.num("iters", 200);
   const double seconds = std::atof(a.str("seconds", "0").c_str());
+  // (a launch of 1600 passes takes about a millisecond: with --seconds, one line per second or so)
+  const int passes = a.num("passes", 1600), iters = a.num("iters", seconds > 0 ? 1000 : 200);
   int warmup = a.num("warmup", 100);
   double spent = 0.0;
   do {
