@@ -170,6 +170,11 @@ BEAM_HD TileCoord grouped_tile(int pid, int tiles_m, int tiles_n, int group_m) {
 // 8*gc >= tiles_n, so one band group is exactly what the 8 XCDs hold at once (gb*gc <= CUs per XCD).
 // Every XCD walks the band groups in the same order, and the hardware dispatches the workgroups of an
 // XCD in id order: the earliest unfinished band group is always fully resident, hence no deadlock.
+// Inside its block an XCD takes band after band (columns fastest): a launch that shares the device with
+// another then holds whole bands plus at most one partial band per XCD, and the CUs that the whole bands
+// free are enough to complete the partial ones.  (Bands fastest, the first form of this order, left two
+// launches on two streams with a part of *every* band of a group each: they waited for each other until
+// the driver's time slicing, seconds later, or the poll budget ended it.)
 // The grid is padded (8 * band_groups * gb * gc workgroups); ids that fall outside the tile grid
 // return tm = -1 and the workgroup exits at once.
 BEAM_HD TileCoord band_block_tile(int wg, int tiles_m, int tiles_n, int gb, int gc) {
@@ -179,8 +184,8 @@ BEAM_HD TileCoord band_block_tile(int wg, int tiles_m, int tiles_n, int gb, int 
   const int bg = local / per_group;
   const int within = local - bg * per_group;
   TileCoord t;
-  t.tm = bg * gb + within % gb;
-  t.tn = xcd * gc + within / gb;
+  t.tm = bg * gb + within / gc;
+  t.tn = xcd * gc + within % gc;
   if (t.tm >= tiles_m || t.tn >= tiles_n) t.tm = -1;
   return t;
 }
@@ -191,7 +196,8 @@ BEAM_HD int band_block_grid(int tiles_m, int gb, int gc) {
 }
 
 // The same contract with whole bands on one XCD, for bands short enough (tiles_n * bx <= CUs per
-// XCD): XCD x holds bands (g * 8 + x) * bx .. + bx - 1 in round g, M fastest.  The XCDs of one part
+// XCD): XCD x holds bands (g * 8 + x) * bx .. + bx - 1 in round g, band after band (columns
+// fastest, for the reason given above).  The XCDs of one part
 // run at clocks that differ by several percent under a matrix-core load (measured: the same tiles
 // take 5% longer on some XCDs than on others), so a band spread over all XCDs waits for the slowest
 // of them; a band inside one XCD finishes together.  L2 traffic is the same as for band_block_tile
@@ -203,8 +209,8 @@ BEAM_HD TileCoord band_xcd_tile(int wg, int tiles_m, int tiles_n, int bx) {
   const int g = local / per_group;
   const int within = local - g * per_group;
   TileCoord t;
-  t.tm = (g * kNumXcd + xcd) * bx + within % bx;
-  t.tn = within / bx;
+  t.tm = (g * kNumXcd + xcd) * bx + within / tiles_n;
+  t.tn = within % tiles_n;
   if (t.tm >= tiles_m) t.tm = -1;
   return t;
 }
@@ -244,7 +250,7 @@ BEAM_HD TileDivs band_order_divs(int tiles_n, int group_m, int group_n) {
   TileDivs d;
   const int g = group_m < 1 ? 1 : group_m;
   d.group = make_fast_div((unsigned)(g * (group_n > 0 ? group_n : tiles_n)));  // ids of one XCD per band group
-  d.rows = make_fast_div((unsigned)g);
+  d.rows = make_fast_div((unsigned)(group_n > 0 ? group_n : (tiles_n < 1 ? 1 : tiles_n)));  // columns of an XCD's block
   d.rows_last = d.rows;
   d.tiles = make_fast_div((unsigned)(tiles_n < 1 ? 1 : tiles_n));
   return d;
@@ -261,8 +267,9 @@ BEAM_HD TileCoord band_order_tile(int id, int tiles_m, int tiles_n, int group_m,
   const int per_group = group_m * (group_n > 0 ? group_n : tiles_n);
   const int bg = (int)fast_div((unsigned)local, dv.group);
   const int within = local - bg * per_group;
-  const int col = (int)fast_div((unsigned)within, dv.rows);  // within / group_m
-  const int band = within - col * group_m;
+  const int cols = group_n > 0 ? group_n : tiles_n;
+  const int band = (int)fast_div((unsigned)within, dv.rows);  // within / cols
+  const int col = within - band * cols;
   if (group_n > 0) {
     t.tm = bg * group_m + band;
     t.tn = xcd * group_n + col;

@@ -57,6 +57,10 @@ def test_band_xcd_order(beamc, tiles_m, tiles_n, bx):
         ids = [seen[(band, tn)] for tn in range(tiles_n)]
         assert len({w % 8 for w in ids}) == 1
         assert len({(w // 8) // (bx * tiles_n) for w in ids}) == 1
+        # band after band inside the XCD: the band's workgroups are consecutive in that XCD's sequence, so a launch
+        # that shares the device with another holds at most one partial band per XCD
+        local = sorted(w // 8 for w in ids)
+        assert local == list(range(local[0], local[0] + tiles_n))
 
 
 @pytest.mark.parametrize("tiles_m,tiles_n", [(16, 16), (32, 32), (2, 43), (5, 7), (1, 1), (3, 64), (40, 9)])
@@ -81,6 +85,10 @@ def test_band_block_order(beamc, tiles_m, tiles_n):
     for band in range(tiles_m):
         groups = {(seen[(band, tn)] // 8) // (gb * gc) for tn in range(tiles_n)}
         assert len(groups) == 1
+        # on every XCD the band's workgroups are consecutive in that XCD's sequence (band after band)
+        for xcd in range(8):
+            local = sorted(seen[(band, tn)] // 8 for tn in range(tiles_n) if seen[(band, tn)] % 8 == xcd)
+            assert not local or local == list(range(local[0], local[0] + len(local)))
 
 
 def test_lds_swizzle(beamc):
