@@ -211,14 +211,22 @@ def refit(params, timings, steps=4000, seed=1):
 
 
 LN_TIMINGS = os.path.join(os.path.dirname(os.path.abspath(__file__)), "ln_tile_timings.json")
-# name -> (TFLOP/s per CU, fixed microseconds per round of workgroups); order = the library's candidate order
+# name -> (TFLOP/s per CU, fixed microseconds per round of workgroups); order = the library's candidate order.
+# Two candidates share the 256 x 256 tile: the 4-wavefront kernel (one wavefront per SIMD: the faster K loop, and an
+# epilogue in which nothing overlaps the vector work of its one wavefront) and the 8-wavefront one (two wavefronts per
+# SIMD cover each other's waits in the epilogue): the first wins where K is long, the second where rounds are short.
 LN_PARAMS = {
-    "256x256_w128x128": (7.90, 12.62), "224x256_w112x64": (7.77, 11.56), "192x256_w96x64": (7.49, 10.76),
-    "256x128_w64x64": (6.53, 9.29), "128x256_w64x64": (6.09, 8.77), "128x128_w64x32": (4.85, 6.60),
-    "64x128_w32x64": (3.23, 3.84), "64x64_w32x32": (3.07, 3.19),
+    "256x256_w128x128": (7.44, 19.82), "256x256_w128x64": (6.71, 14.46), "224x256_w112x64": (6.41, 12.49),
+    "192x256_w96x64": (6.15, 11.12), "256x128_w64x64": (5.02, 7.64), "128x256_w64x64": (5.08, 8.11),
+    "128x128_w64x32": (4.89, 7.03), "64x128_w32x64": (3.18, 3.70), "64x64_w32x32": (2.77, 2.79),
 }
-# (fitted on the table's column of the 8-wavefront 256x256 tile; the library runs the 4-wavefront kernel where it fits)
-LN_FIT_COLUMN = {"256x256_w128x128": "256x256_w128x64"}
+LN_FIT_COLUMN = {}
+W4_MIN_K = 192
+
+
+def ln_w4_applies(name, N, K):
+    """The 4-wavefront kernel's own conditions (gemm_w4.h); any other candidate: True."""
+    return name != "256x256_w128x128" or (K % 64 == 0 and K >= W4_MIN_K and N % 8 == 0)
 
 
 def _ln_block(name):
@@ -235,14 +243,22 @@ def ln_fused_applies(name, N, cus=CUS):
     return cus == 256 and tiles_n <= 64 and (tiles_n + 1) * bm * 8 <= lds
 
 
+def ln_rounds(M, N, bm, bn, cus=CUS):
+    """Rounds of workgroups of the one-kernel form: a band's column tiles wait for each other, so a band that
+    straddles two rounds costs both; a round is worth the whole bands it holds."""
+    tiles_m, tiles_n = -(-M // bm), -(-N // bn)
+    per_round = max(1, cus // tiles_n)
+    return -(-tiles_m // per_round)
+
+
 def predict_ln(params, M, N, K, cus=CUS):
     """(name, modelled us) of the tile the library takes for the one-kernel GEMM+LayerNorm, None where none applies."""
     best = None
     for name, (rate, fixed) in params.items():
-        if not ln_fused_applies(name, N, cus):
+        if not ln_fused_applies(name, N, cus) or not ln_w4_applies(name, N, K):
             continue
         bm, bn = _ln_block(name)
-        rounds = -(-(-(-M // bm) * -(-N // bn)) // cus)
+        rounds = ln_rounds(M, N, bm, bn, cus)
         us = rounds * (fixed + 2.0e-6 * bm * bn * K / rate)
         if best is None or us < best[1]:
             best = (name, us)
@@ -276,8 +292,13 @@ def fit_ln(table):
             if col not in row:
                 continue
             M, N, K = map(int, key.split("x"))
+            if not ln_w4_applies(name, N, K):
+                continue
             bm, bn = _ln_block(name)
-            rounds = -(-(-(-M // bm) * -(-N // bn)) // CUS)
+            tiles = -(-M // bm) * -(-N // bn)
+            if tiles < CUS // 2:  # (a tile is not in question where it leaves most of the device idle)
+                continue
+            rounds = ln_rounds(M, N, bm, bn, CUS)
             X.append([rounds, rounds * 2.0e-6 * bm * bn * K])
             y.append(row[col])
         X, y = np.array(X), np.array(y)

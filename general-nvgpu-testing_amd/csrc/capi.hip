@@ -848,24 +848,29 @@ static size_t ln_workspace_need(int M, int N, const beam_tile_cfg& c, int mode) 
 
 // The tile a GEMM+LayerNorm call runs with: the caller's, or the library's; never the deep pipeline.
 // For the one-kernel form (mode AUTO or FUSED on a device it runs on) the library does not take the plain GEMM's
-// tile: every workgroup ends with the epilogue's chain of latencies, one tile per workgroup, so a round of
-// workgroups costs a fixed time that grows with the tile, and rounds count in whole numbers.  The model is that
-// sentence: rounds x (fixed + flops of a tile / rate), rates (TFLOP/s per CU) and fixed costs (us) fitted by
-// least squares to the timings of every tile on 34 shapes (beam/ln_tile_timings.json: the pick is within 1.5%
-// of the best tile in the geometric mean, 16% at worst; the plain GEMM's tile is 7% behind in the mean).
+// tile: every workgroup ends with the epilogue's chain of latencies, so a round of workgroups costs a fixed time
+// that grows with the tile, and rounds count in whole numbers -- of bands, since a band's tiles wait for each other.
+// The model is that sentence: rounds x (fixed + flops of a tile / rate), rates (TFLOP/s per CU) and fixed costs (us)
+// fitted by least squares to the timings of every tile on 34 shapes (beam/ln_tile_timings.json: the pick is within
+// 1.4% of the best tile in the geometric mean, 13% at worst).
 struct LnCandidate {
   beam_tile_cfg cfg;
   double rate, fixed;
 };
+// Two candidates share the 256 x 256 tile: the 4-wavefront kernel of gemm_w4.h (the faster K loop; an epilogue in
+// which nothing overlaps the vector work of its one wavefront per SIMD) and the 8-wavefront one (two wavefronts per
+// SIMD cover each other's waits in the epilogue).  Measured, the first wins by about 1% where K is 4096 and more, the
+// second by 2-14% where a tile's K loop is short (8192 x 8192 x 1024: 152 against 160 us).
 static const LnCandidate kLnCandidates[] = {
-    {{256, 256, 128, 128, 0, 0}, 7.90, 12.62},  // (runs as the 8-wavefront 128 x 64 form where gemm_w4.h's conditions fail)
-    {{224, 256, 112, 64, 0, 0}, 7.77, 11.56},
-    {{192, 256, 96, 64, 0, 0}, 7.49, 10.76},
-    {{256, 128, 64, 64, 0, 0}, 6.53, 9.29},
-    {{128, 256, 64, 64, 0, 0}, 6.09, 8.77},
-    {{128, 128, 64, 32, 0, 0}, 4.85, 6.60},
-    {{64, 128, 32, 64, 0, 0}, 3.23, 3.84},
-    {{64, 64, 32, 32, 0, 0}, 3.07, 3.19},
+    {{256, 256, 128, 128, 0, 0}, 7.44, 19.82},  // (only where gemm_w4.h's conditions hold)
+    {{256, 256, 128, 64, 0, 0}, 6.71, 14.46},
+    {{224, 256, 112, 64, 0, 0}, 6.41, 12.49},
+    {{192, 256, 96, 64, 0, 0}, 6.15, 11.12},
+    {{256, 128, 64, 64, 0, 0}, 5.02, 7.64},
+    {{128, 256, 64, 64, 0, 0}, 5.08, 8.11},
+    {{128, 128, 64, 32, 0, 0}, 4.89, 7.03},
+    {{64, 128, 32, 64, 0, 0}, 3.18, 3.70},
+    {{64, 64, 32, 32, 0, 0}, 2.77, 2.79},
 };
 // The model's pick for a device of `cus` compute units; false if the one-kernel form applies with none of the tiles.
 static bool ln_choose_tile(int M, int N, int K, int cus, beam_tile_cfg* out, const KernelSet** out_ks) {
@@ -874,9 +879,14 @@ static bool ln_choose_tile(int M, int N, int K, int cus, beam_tile_cfg* out, con
   for (const LnCandidate& k : kLnCandidates) {
     beam_tile_cfg c = k.cfg;
     const KernelSet* ks = nullptr;
-    if (resolve_cfg(&c, M, N, K, &c, &ks) != BEAM_OK || !ln_fused_applies_on(c, *ks, N, cus)) continue;
-    const long tiles = (long)((M + c.block_m - 1) / c.block_m) * ((N + c.block_n - 1) / c.block_n);
-    const double rounds = (double)((tiles + cus - 1) / cus);
+    const bool w4 = c.wave_m == 128 && c.wave_n == 128;
+    if (w4 && !(K % kBK == 0 && K >= kW4MinK && N % 8 == 0)) continue;
+    if (resolve_cfg(&c, M, N, K, &c, &ks, -1, w4) != BEAM_OK || !ln_fused_applies_on(c, *ks, N, cus)) continue;
+    // (a band's column tiles wait for each other, so a band that straddles two rounds costs both: a round is
+    // worth the whole bands it holds)
+    const int tiles_m = (M + c.block_m - 1) / c.block_m, tiles_n = (N + c.block_n - 1) / c.block_n;
+    const int bands_per_round = cus / tiles_n > 1 ? cus / tiles_n : 1;
+    const double rounds = (double)((tiles_m + bands_per_round - 1) / bands_per_round);
     const double us = rounds * (k.fixed + 2.0e-6 * c.block_m * c.block_n * (double)K / k.rate);
     if (us < best_us) {
       best_us = us;
@@ -940,7 +950,7 @@ static int ln_plan(int M, int N, int K, const beam_tile_cfg* cfg, int mode, bool
     c.wave_n = 64;
     if ((rc = resolve_cfg(&c, M, N, K, &c, &out->ks))) return rc;
   }
-  out->w4 = w4_fits && (!cfg || (c.wave_m == 128 && c.wave_n == 128));
+  out->w4 = w4_fits && c.wave_m == 128 && c.wave_n == 128;
   out->kind = mode == BEAM_LN_FUSED ? LnPlan::kFused : LnPlan::kTwoPass;
   out->need = ln_workspace_need(M, N, c, mode);
   return BEAM_OK;

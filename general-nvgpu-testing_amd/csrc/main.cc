@@ -601,7 +601,14 @@ int cli_bench(const Args& a) {
   float ms = 0;
   const std::string lnm = a.str("ln-mode", "auto");  // --op ln: auto | twopass | fused
   const int ln_mode = lnm == "twopass" ? BEAM_LN_TWOPASS : lnm == "fused" ? BEAM_LN_FUSED : BEAM_LN_AUTO;
-  int rc = time_op(op, p, &cfg, split, a.num("warmup", 5), a.num("iters", 20), &ms, ln_mode);
+  // GEMM+LayerNorm without a tile on the command line: the library's own choice for that operator (a cost model
+  // of its own, not the plain GEMM's tile); the line below then names what it picked for a device of 256 CUs.
+  const bool ln_auto_tile = op == BEAM_OP_GEMM_LN && !a.has("tile") && !a.has("wave") && !a.has("pipeline") && !a.has("group");
+  if (ln_auto_tile && ln_mode != BEAM_LN_TWOPASS) {
+    beam_tile_cfg picked;
+    if (beam_dbg_ln_default_config(M, N, K, 256, &picked) == BEAM_OK) cfg = picked;
+  }
+  int rc = time_op(op, p, ln_auto_tile ? nullptr : &cfg, split, a.num("warmup", 5), a.num("iters", 20), &ms, ln_mode);
   if (rc != BEAM_OK) {
     std::fprintf(stderr, "bench failed (%d): %s\n", rc, beam_last_error());
     return 1;

@@ -155,8 +155,6 @@ def test_layernorm_tile_model_against_its_timing_table(beamc):
         name = beamc.TileConfig(c.block_m, c.block_n, c.wave_m, c.wave_n, 0, 0).name
         tiles = {k: v for k, v in row.items() if k not in ("default", "plain")}
         picked = tiles[name]
-        if name == "256x256_w128x128" and "256x256_w128x64" in tiles:
-            picked = min(picked, tiles["256x256_w128x64"])
         r = picked / min(tiles.values())
         logs.append(math.log(r))
         worst = max(worst, r)
