@@ -689,11 +689,13 @@ struct GemmW4 {
     ln_sign_header(p, tag);
     ln_publish(p, ((size_t)tc.tm * p.tiles_n + tc.tn) * BM + rl, mean, m2, tag);
     lds_barrier();  // `part` is free again
-    // 3. gather the pairs of this thread's row from the band's other column tiles into LDS, 16 tiles' worth in
-    //    flight at once, fetching again -- boundedly -- what does not carry the launch's tag yet (the protocol of
-    //    gemm_kernel.h's ln_gather).  A batch costs a round trip to memory (1.3 us measured), whatever its size: a band
-    //    of 32 column tiles took 5.1-5.7 us in batches of 8.  (32 in flight need 128 registers, and the compiler then
-    //    parks values in accumulation registers, i.e. in the accumulators: the codegen test watches for that.)  The
+    // 3. gather the pairs of this thread's row from the band's column tiles into LDS, 16 tiles' worth in flight at
+    //    once, fetching again -- boundedly -- what does not carry the launch's tag yet (the protocol of
+    //    gemm_kernel.h's ln_gather).  The tile's own pair comes back through memory like the others'.  What the
+    //    gather costs is a round trip to memory (1.3 us) plus the spread of the band's tiles, whose CUs run at clocks
+    //    several percent apart: 2.6 us for a band of 16 tiles, 5 us for one of 32, with 8 or 16 in flight alike.  (32
+    //    in flight need 128 registers, and the compiler then parks values in accumulation registers, i.e. in the
+    //    accumulators: the codegen test watches for that.)
     {
       const unsigned long long* w0s = (const unsigned long long*)p.stats + (size_t)tc.tm * p.tiles_n * BM + rl;
       const unsigned long long* w1s = (const unsigned long long*)p.next_stats + (size_t)tc.tm * p.tiles_n * BM + rl;
