@@ -216,9 +216,9 @@ LN_TIMINGS = os.path.join(os.path.dirname(os.path.abspath(__file__)), "ln_tile_t
 # epilogue in which nothing overlaps the vector work of its one wavefront) and the 8-wavefront one (two wavefronts per
 # SIMD cover each other's waits in the epilogue): the first wins where K is long, the second where rounds are short.
 LN_PARAMS = {
-    "256x256_w128x128": (7.44, 19.82), "256x256_w128x64": (6.71, 14.46), "224x256_w112x64": (6.41, 12.49),
-    "192x256_w96x64": (6.15, 11.12), "256x128_w64x64": (5.02, 7.64), "128x256_w64x64": (5.08, 8.11),
-    "128x128_w64x32": (4.89, 7.03), "64x128_w32x64": (3.18, 3.70), "64x64_w32x32": (2.77, 2.79),
+    "256x256_w128x128": (7.91, 18.17), "256x256_w128x64": (7.08, 14.13), "224x256_w112x64": (6.94, 12.35),
+    "192x256_w96x64": (6.66, 11.01), "256x128_w64x64": (5.38, 8.00), "128x256_w64x64": (5.41, 8.17),
+    "128x128_w64x32": (5.05, 6.65), "64x128_w32x64": (3.33, 3.54), "64x64_w32x32": (2.98, 2.76),
 }
 LN_FIT_COLUMN = {}
 W4_MIN_K = 192

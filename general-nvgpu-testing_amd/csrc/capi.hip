@@ -852,25 +852,26 @@ static size_t ln_workspace_need(int M, int N, const beam_tile_cfg& c, int mode) 
 // that grows with the tile, and rounds count in whole numbers -- of bands, since a band's tiles wait for each other.
 // The model is that sentence: rounds x (fixed + flops of a tile / rate), rates (TFLOP/s per CU) and fixed costs (us)
 // fitted by least squares to the timings of every tile on 34 shapes (beam/ln_tile_timings.json: the pick is within
-// 1.4% of the best tile in the geometric mean, 13% at worst).
+// 1.5% of the best tile in the geometric mean, 16% at worst).
 struct LnCandidate {
   beam_tile_cfg cfg;
   double rate, fixed;
 };
 // Two candidates share the 256 x 256 tile: the 4-wavefront kernel of gemm_w4.h (the faster K loop; an epilogue in
 // which nothing overlaps the vector work of its one wavefront per SIMD) and the 8-wavefront one (two wavefronts per
-// SIMD cover each other's waits in the epilogue).  Measured, the first wins by about 1% where K is 4096 and more, the
-// second by 2-14% where a tile's K loop is short (8192 x 8192 x 1024: 152 against 160 us).
+// SIMD cover each other's waits in the epilogue).  Measured, the first wins by 3-5% where K is 2048 and more and the
+// rounds are few (4096^3: 100.3 against 105.6 us), the second by 3-14% where a tile's K loop is short (8192 x 8192 x
+// 1024: 146.1 against 150.7 us; 4096 x 16384 x 1024, whose bands are too wide to walk: 166.8 against 190.8).
 static const LnCandidate kLnCandidates[] = {
-    {{256, 256, 128, 128, 0, 0}, 7.44, 19.82},  // (only where gemm_w4.h's conditions hold)
-    {{256, 256, 128, 64, 0, 0}, 6.71, 14.46},
-    {{224, 256, 112, 64, 0, 0}, 6.41, 12.49},
-    {{192, 256, 96, 64, 0, 0}, 6.15, 11.12},
-    {{256, 128, 64, 64, 0, 0}, 5.02, 7.64},
-    {{128, 256, 64, 64, 0, 0}, 5.08, 8.11},
-    {{128, 128, 64, 32, 0, 0}, 4.89, 7.03},
-    {{64, 128, 32, 64, 0, 0}, 3.18, 3.70},
-    {{64, 64, 32, 32, 0, 0}, 2.77, 2.79},
+    {{256, 256, 128, 128, 0, 0}, 7.91, 18.17},  // (only where gemm_w4.h's conditions hold)
+    {{256, 256, 128, 64, 0, 0}, 7.08, 14.13},
+    {{224, 256, 112, 64, 0, 0}, 6.94, 12.35},
+    {{192, 256, 96, 64, 0, 0}, 6.66, 11.01},
+    {{256, 128, 64, 64, 0, 0}, 5.38, 8.00},
+    {{128, 256, 64, 64, 0, 0}, 5.41, 8.17},
+    {{128, 128, 64, 32, 0, 0}, 5.05, 6.65},
+    {{64, 128, 32, 64, 0, 0}, 3.33, 3.54},
+    {{64, 64, 32, 32, 0, 0}, 2.98, 2.76},
 };
 // The model's pick for a device of `cus` compute units; false if the one-kernel form applies with none of the tiles.
 static bool ln_choose_tile(int M, int N, int K, int cus, beam_tile_cfg* out, const KernelSet** out_ks) {
