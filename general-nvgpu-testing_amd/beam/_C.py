@@ -127,6 +127,7 @@ def _load() -> ctypes.CDLL:
     L.beam_dbg_ln_plan_bytes.restype = sz
     L.beam_dbg_assume_compute_units.argtypes = [i]
     L.beam_set_ln_walk.argtypes = [i]
+    L.beam_dbg_set_splitk_self_reduce.argtypes = [i]
     L.beam_dbg_tile_of_workgroup.argtypes = [i, i, i, i, ctypes.POINTER(i), ctypes.POINTER(i)]
     L.beam_dbg_lds_offset.argtypes = [i, i]
     L.beam_dbg_kmajor_lds_offset.argtypes = [i, i, i]

@@ -639,6 +639,10 @@ static std::atomic<int> g_ln_no_walk{[] {
   return e && *e == '0' ? 1 : 0;
 }()};
 
+// 1: the one-launch split-K runs without reducing workgroups where its multiplying workgroups fit one round of the
+// CUs; each of them reduces its share of its tile (beam_dbg_set_splitk_self_reduce: a measurement, off by default)
+static std::atomic<int> g_splitk_self_reduce{0};
+
 // 0: one launch where it applies, 1: always the partial kernel followed by the reduce kernel
 static std::atomic<int> g_splitk_two_launches{[] {
   const char* e = getenv("BEAM_SPLITK_TWO_LAUNCHES");
@@ -756,7 +760,8 @@ int beam_gemmrc_splitk(const void* A, const void* B, void* C, int M, int N, int 
       p.sk_sync = (int*)((char*)ws + sync_at);
       p.ln_nonce = g_ln_nonce.fetch_add(1, std::memory_order_relaxed) + 1;
       p.spin_limit = g_ln_spin_limit.load();
-      BEAM_HIP(one_launch(p, dim3((unsigned)(tiles * s + tiles * parts), 1, 1), st));
+      p.sk_self = g_splitk_self_reduce.load(std::memory_order_relaxed) && tiles * s <= cus ? 1 : 0;
+      BEAM_HIP(one_launch(p, dim3((unsigned)(tiles * s + (p.sk_self ? 0 : tiles * parts)), 1, 1), st));
       return BEAM_OK;
     }
   }
@@ -1002,6 +1007,11 @@ size_t beam_dbg_ln_plan_bytes(int M, int N, int K, const beam_tile_cfg* cfg, int
   LnPlan plan;
   if (M <= 0 || N <= 0 || K < 0 || ln_plan(M, N, K, cfg, mode, plain != 0 || K % 8 != 0 || K > kMaxK, capturing != 0, wide_io != 0, &plan)) return 0;
   return plan.need;
+}
+
+int beam_dbg_set_splitk_self_reduce(int on) {
+  g_splitk_self_reduce.store(on != 0);
+  return BEAM_OK;
 }
 
 int beam_set_ln_walk(int on) {

@@ -138,6 +138,9 @@ struct GemmParams {
   // behind the partial sums in the caller's workspace.  Never has to be initialised (see sk_launch_tag).
   int* sk_sync;
   int sk_out;  // kEpiPartialFused: outputs per thread of a reducing workgroup (4, 2 or 1)
+  // kEpiPartialFused, measurement only: 1 = no reducing workgroups; the multiplying workgroup of (tile, slice s)
+  // reduces parts s, s + splits, ... of its tile itself.  Every multiplying workgroup must then be resident at once.
+  int sk_self;
 };
 
 // ---- statistics exchange of the fused GEMM+LayerNorm (both K loops: this file's and gemm_w4.h's) ----------
@@ -1323,6 +1326,14 @@ struct GemmTile {
         if (tid < P) {
           const size_t f = ((size_t)(tc.tm * p.tiles_n + tc.tn) * P + tid) * p.splits + slice;
           __hip_atomic_store(p.sk_sync + kSkFlags + f, (int)sk_launch_tag(p.ln_nonce), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        if (p.sk_self) {  // (uniform)
+          const int t = tc.tm * p.tiles_n + tc.tn;
+          for (int q = slice; q < P; q += p.splits) {
+            if (p.sk_out == 4) splitk_reduce_part_of<4>(p, t * P + q);
+            else if (p.sk_out == 2) splitk_reduce_part_of<2>(p, t * P + q);
+            else splitk_reduce_part_of<1>(p, t * P + q);
+          }
         }
         return;
       }

@@ -64,6 +64,11 @@ int beam_dbg_kmajor_lds_offset(int k, int n, int block_n);
  * and beta 16-byte aligned).  The entry point computes its requirement with the same function; the workspace queries
  * are tested against it.  0 on error. */
 size_t beam_dbg_ln_plan_bytes(int M, int N, int K, const beam_tile_cfg* cfg, int mode, int plain, int capturing, int wide_io);
+/* A measurement, off by default: on != 0 makes the one-launch split-K run without reducing workgroups wherever its
+ * multiplying workgroups fit one round of the CUs; the workgroup of (tile, slice s) then adds parts s, s + slices, ...
+ * of its tile itself.  Same bits.  Unlike the shipped form this needs every workgroup of the launch resident at once
+ * (the wait is bounded all the same). */
+int beam_dbg_set_splitk_self_reduce(int on);
 /* For tests on a host without a GPU: the CU count the library's choices assume when no device could be probed
  * (refused once a device has been). */
 int beam_dbg_assume_compute_units(int compute_units);

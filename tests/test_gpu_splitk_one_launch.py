@@ -59,6 +59,38 @@ def test_one_launch_equals_two_launches(gpu, beamc):
     ws.free()
 
 
+def test_self_reducing_workgroups_give_the_same_bits(gpu, beamc):
+    """The measurement form without reducing workgroups (every multiplying workgroup adds its share of its tile):
+    the same bits as two launches, where the slices outnumber the parts of a tile, equal them and are fewer; twice in
+    a row on one never-cleared workspace; no time-out."""
+    L = beamc.lib
+    ws = beamc.DeviceArray((64 << 20,), itemsize=1)
+    ws.fill_bytes(0x5C)
+    cases = [(256, 256, 32768, F16, 32, (64, 128, 32, 64), 2), (256, 256, 32768, F16, 16, (64, 64, 32, 32), 2),
+             (64, 128, 65536, F16, 64, (64, 64, 32, 32), 0), (128, 128, 8192, BF16, 4, (64, 64, 32, 32), 0),
+             (200, 136, 4104, BF16, 7, (64, 128, 32, 64), 2), (256, 256, 8192, F16, 3, (128, 128, 64, 64), 0)]
+    assert L.beam_dbg_set_splitk_self_reduce(1) == 0
+    try:
+        for seed, (M, N, K, dtype, split, tile, pipe) in enumerate(cases):
+            a = beamc.DeviceArray.from_numpy(beamc.host_uniform((M, K), dtype, 90 + seed, 0), dtype)
+            b = beamc.DeviceArray.from_numpy(beamc.host_uniform((N, K), dtype, 90 + seed, 1), dtype)
+            c = beamc.DeviceArray((M, N), dtype)
+            cfg = beamc.TileConfig(*tile, pipe, 0).to_c()
+            s = L.beam_splitk_effective(M, N, K, ctypes.byref(cfg), split)
+            assert s > 1
+            two = _call(beamc, a, b, c, M, N, K, dtype, cfg, split, ws, True)
+            for _ in range(2):
+                one = _call(beamc, a, b, c, M, N, K, dtype, cfg, split, ws, False)
+                assert (one == two).all(), (M, N, K, dtype, split, tile, pipe)
+            flag = ctypes.c_int(1)
+            assert L.beam_gemmrc_splitk_timed_out(ws.ptr, ws.nbytes, M, N, s, None, ctypes.byref(flag)) == 0 and flag.value == 0
+            for t in (a, b, c):
+                t.free()
+    finally:
+        L.beam_dbg_set_splitk_self_reduce(0)
+        ws.free()
+
+
 def test_random_shapes_tiles_and_slice_counts(gpu, beamc):
     """80 seeded random problems (ragged M, N a multiple of 4, K a multiple of 8 with tails inside slices), random
     small tile, LDS depth and slice count, both dtypes, one never-cleared workspace: the two forms agree bit for bit."""
