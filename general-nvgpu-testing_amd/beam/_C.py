@@ -375,6 +375,13 @@ def set_splitk_two_launches(on: bool) -> None:
     _check(lib.beam_set_splitk_two_launches(1 if on else 0))
 
 
+def set_ln_walk(on: bool) -> None:
+    """True (default): from more 256 x 256 tiles than CUs on, the fused GEMM+LayerNorm of the 4-wavefront kernel runs
+    one workgroup per CU walking its tiles (every workgroup of the launch must then be resident at once); False: one
+    workgroup per tile in band order, which finishes band by band on whatever share of the device it gets.  Same bits."""
+    _check(lib.beam_set_ln_walk(1 if on else 0))
+
+
 def gemmrc_splitk(a, b, c, split_k_slices: int = 0, check: bool = False) -> None:
     """Split-K with the library's default tile for the problem; split_k_slices <= 0: the library
     picks the slice count as well (one full round of workgroups)
