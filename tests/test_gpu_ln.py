@@ -357,3 +357,28 @@ def test_ln_default_call_never_lacks_workspace(gpu, beamc, oracle):
     ref = oracle.gemmrc_ln(a, b, g_, bt, 1e-5, F16)
     got = run_ln(beamc, a, b, g_, bt, F16)
     check_ln(oracle, got, ref, F16, "default call 1024 x 8192 x 2048")
+
+
+def test_walking_kernel_ends_when_every_wait_gives_up(gpu, beamc):
+    """The walking form of the 4-wavefront kernel (1024 tiles on 256 workgroups) with the spin limit at -1: every
+    wait of every tile gives up at once, the workgroups still walk all their tiles and end normally, every row is
+    NaN and the record says so; the next call with the normal budget is right again, with no reset in between."""
+    M, N, K = 8192, 8192, 256
+    w4 = beamc.TileConfig(256, 256, 128, 128)
+    a, b, g_, bt = make_ln_inputs(beamc, M, N, K, F16, 33)
+    good = run_ln(beamc, a, b, g_, bt, F16, config=w4, mode=beamc.LN_FUSED)
+    da, db = beamc.DeviceArray.from_numpy(a), beamc.DeviceArray.from_numpy(b)
+    dg, dbt = beamc.DeviceArray.from_numpy(g_), beamc.DeviceArray.from_numpy(bt)
+    y = beamc.DeviceArray((M, N))
+    try:
+        assert beamc.lib.beam_set_ln_spin_limit(-1) == 0
+        beamc.gemmrc_ln(da, db, y, dg, dbt, config=w4, mode=beamc.LN_FUSED, check=False)
+        beamc.sync()
+        assert beamc.gemmrc_ln_timed_out()
+        assert np.isnan(y.to_numpy().view(np.float16)).all()
+    finally:
+        beamc.lib.beam_set_ln_spin_limit(beamc.DEFAULT_SPIN_LIMIT)
+    beamc.gemmrc_ln(da, db, y, dg, dbt, config=w4, mode=beamc.LN_FUSED, check=True)
+    assert (y.to_numpy() == good).all()
+    for x in (da, db, dg, dbt, y):
+        x.free()
